@@ -1,0 +1,36 @@
+// C interface of the kernel library (libtokenmill_hip.so). Every function returns 0 on success,
+// TM_ERR_ARG (1) for sizes or types the kernel does not run, TM_ERR_LAUNCH (2) if the launch failed.
+// Pointers are device pointers; `stream` is a hipStream_t. dtype codes: 0 = float32, 1 = bfloat16.
+#pragma once
+#include <hip/hip_runtime.h>
+
+extern "C" {
+
+int tm_embed_gather(const void* table, int dtype, const int* ids, float* out, int T, int hidden, int vocab,
+                    hipStream_t stream);
+
+int tm_add_rmsnorm(float* resid, const void* delta, const int* rows, const void* weight, int w_dtype, void* out,
+                   int dtype, int R, int hidden, float eps, hipStream_t stream);
+
+int tm_rope_kv_write(void* qkv, int dtype, int T, int H, int KVH, int D, int rot, const float* cos_t,
+                     const float* sin_t, const int* positions, const int* slots, void* k_pool, void* v_pool,
+                     int write_kv, hipStream_t stream);
+
+int tm_silu_mul(const void* gu, void* out, int dtype, int T, int I, hipStream_t stream);
+
+int tm_convert(const void* in, int in_dtype, void* out, int out_dtype, long long n, hipStream_t stream);
+
+int tm_gemm_nt_tiled(const void* A, int lda, const void* W, const void* bias, int bias_dtype, void* C, int ldc,
+                     int M, int N, int K, int in_dtype, int out_dtype, hipStream_t stream);
+
+int tm_attn_paged_generic(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
+                          const void* v_pool, const int* block_tables, int table_width, const int* seq_of_token,
+                          const int* positions, int T, int H, int KVH, int D, int page, float scale, int window,
+                          int dtype, hipStream_t stream);
+
+int tm_argmax_rows(const float* logits, int R, int V, int* out, hipStream_t stream);
+
+int tm_sample_rows(const float* logits, int R, int V, const float* temperature, const int* top_k,
+                   const float* top_p, const float* u, int* out, hipStream_t stream);
+
+}  // extern "C"

@@ -1,0 +1,209 @@
+// Row-wise kernels: embedding rows, residual add + RMSNorm, rotary position encoding fused with
+// the cache write, SiLU(gate)*up, type conversion.
+//
+// Exactness: the residual stream is 32-bit; sums of squares, the reciprocal root and the rotation
+// are 32-bit; a bfloat16 result is rounded once, where the tensor is stored.
+#include "common.h"
+#include "api.h"
+
+// ------------------------------------------------------------------------------------------
+// embedding rows -> 32-bit residual stream           (reference src/infer/model/qwen2.py:46)
+// ------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void embed_gather_kernel(const T* __restrict__ table, const int* __restrict__ ids,
+                                    float* __restrict__ out, int hidden, int vocab) {
+    const int t = blockIdx.x;
+    int id = ids[t];
+    id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);       // the host rejects such ids; never read outside
+    const T* row = table + (size_t)id * hidden;
+    float* o = out + (size_t)t * hidden;
+    for (int c = threadIdx.x; c < hidden; c += blockDim.x) o[c] = Elem<T>::load(row + c);
+}
+
+extern "C" int tm_embed_gather(const void* table, int dtype, const int* ids, float* out, int T,
+                               int hidden, int vocab, hipStream_t stream) {
+    if (T <= 0) return TM_OK;
+    if (hidden <= 0 || vocab <= 0) return TM_ERR_ARG;
+    if (dtype == TM_F32)
+        embed_gather_kernel<float><<<T, 256, 0, stream>>>((const float*)table, ids, out, hidden, vocab);
+    else if (dtype == TM_BF16)
+        embed_gather_kernel<bf16_t><<<T, 256, 0, stream>>>((const bf16_t*)table, ids, out, hidden, vocab);
+    else
+        return TM_ERR_ARG;
+    TM_CHECK_LAUNCH();
+    return TM_OK;
+}
+
+// ------------------------------------------------------------------------------------------
+// residual += delta ; out = weight * round(residual * rsqrt(mean(residual^2) + eps))
+//                                                    (reference src/infer/model/layers.py:41-44,
+//                                                     src/infer/model/qwen2.py:22-23)
+// rows == nullptr: row r of the residual is updated in place.
+// rows != nullptr: row rows[r] is read (residual + delta), nothing is written back, out row r.
+// ------------------------------------------------------------------------------------------
+template <typename T, typename WT>
+__global__ void add_rmsnorm_kernel(float* __restrict__ resid, const T* __restrict__ delta,
+                                   const int* __restrict__ rows, const WT* __restrict__ weight,
+                                   T* __restrict__ out, int hidden, float eps) {
+    __shared__ float red[4];
+    const int r = blockIdx.x;
+    const size_t src = rows ? (size_t)rows[r] : (size_t)r;
+    float* x = resid + src * hidden;
+    const T* d = delta ? delta + src * hidden : nullptr;
+    T* o = out + (size_t)r * hidden;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < hidden; c += 256) {
+        float v = x[c];
+        if (d) v += Elem<T>::load(d + c);
+        if (d && !rows) x[c] = v;
+        ss += v * v;
+    }
+    ss = block_sum<256>(ss, red);
+    const float rs = rsqrtf(ss / (float)hidden + eps);
+    for (int c = threadIdx.x; c < hidden; c += 256) {
+        float v = x[c];
+        if (d && rows) v += Elem<T>::load(d + c);          // in-place rows already hold the sum
+        const float n = Elem<T>::round(v * rs);            // rounded BEFORE the weight multiplies
+        Elem<T>::store(o + c, Elem<WT>::load(weight + c) * n);
+    }
+}
+
+extern "C" int tm_add_rmsnorm(float* resid, const void* delta, const int* rows, const void* weight,
+                              int w_dtype, void* out, int dtype, int R, int hidden, float eps,
+                              hipStream_t stream) {
+    if (R <= 0) return TM_OK;
+    if (hidden <= 0 || !(eps > 0.f)) return TM_ERR_ARG;
+    if (dtype == TM_F32 && w_dtype == TM_F32)
+        add_rmsnorm_kernel<float, float><<<R, 256, 0, stream>>>(resid, (const float*)delta, rows,
+                                                               (const float*)weight, (float*)out, hidden, eps);
+    else if (dtype == TM_BF16 && w_dtype == TM_BF16)
+        add_rmsnorm_kernel<bf16_t, bf16_t><<<R, 256, 0, stream>>>(resid, (const bf16_t*)delta, rows,
+                                                                 (const bf16_t*)weight, (bf16_t*)out, hidden, eps);
+    else if (dtype == TM_BF16 && w_dtype == TM_F32)
+        add_rmsnorm_kernel<bf16_t, float><<<R, 256, 0, stream>>>(resid, (const bf16_t*)delta, rows,
+                                                                (const float*)weight, (bf16_t*)out, hidden, eps);
+    else
+        return TM_ERR_ARG;
+    TM_CHECK_LAUNCH();
+    return TM_OK;
+}
+
+// ------------------------------------------------------------------------------------------
+// Rotary position encoding of q and k in place, then k and v of every token to its cache slot.
+//   qkv row = [H heads of q | KVH heads of k | KVH heads of v], each D wide.
+//   pairs (j, j + rot/2) for j < rot/2; elements >= rot pass through
+//                                                    (reference src/infer/model/layers.py:55-64;
+//                                                     cache write: src/infer/kv/paged_cache.py:40-43)
+//   cos/sin: [max_pos, rot/2] 32-bit; cos == nullptr means no rotation (cache write only).
+//   slot < 0: the token's k and v are not stored (padding rows).
+// ------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void rope_kv_write_kernel(T* __restrict__ qkv, int H, int KVH, int D, int rot,
+                                     const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+                                     const int* __restrict__ positions, const int* __restrict__ slots,
+                                     T* __restrict__ k_pool, T* __restrict__ v_pool, int write_kv) {
+    const int t = blockIdx.x, hh = blockIdx.y;
+    const int width = (H + 2 * KVH) * D;
+    T* x = qkv + (size_t)t * width + (size_t)hh * D;
+    const bool is_q = hh < H, is_k = !is_q && hh < H + KVH;
+    const int slot = slots ? slots[t] : -1;
+    T* dst = nullptr;
+    if (write_kv && slot >= 0 && !is_q) {
+        const int kvh = is_k ? hh - H : hh - H - KVH;
+        dst = (is_k ? k_pool : v_pool) + ((size_t)slot * KVH + kvh) * D;
+    }
+    const int half = rot / 2;
+    if ((is_q || is_k) && cos_t) {
+        const float* c = cos_t + (size_t)positions[t] * half;
+        const float* s = sin_t + (size_t)positions[t] * half;
+        for (int j = threadIdx.x; j < half; j += blockDim.x) {
+            const float x1 = Elem<T>::load(x + j), x2 = Elem<T>::load(x + j + half);
+            const float y1 = x1 * c[j] - x2 * s[j];
+            const float y2 = x2 * c[j] + x1 * s[j];
+            Elem<T>::store(x + j, y1);
+            Elem<T>::store(x + j + half, y2);
+            if (dst) { Elem<T>::store(dst + j, y1); Elem<T>::store(dst + j + half, y2); }
+        }
+        if (dst)
+            for (int j = rot + threadIdx.x; j < D; j += blockDim.x) dst[j] = x[j];
+    } else if (dst) {
+        for (int j = threadIdx.x; j < D; j += blockDim.x) dst[j] = x[j];
+    }
+}
+
+extern "C" int tm_rope_kv_write(void* qkv, int dtype, int T, int H, int KVH, int D, int rot,
+                                const float* cos_t, const float* sin_t, const int* positions,
+                                const int* slots, void* k_pool, void* v_pool, int write_kv,
+                                hipStream_t stream) {
+    if (T <= 0) return TM_OK;
+    if (H <= 0 || KVH <= 0 || D <= 0 || rot < 0 || rot > D || (rot & 1)) return TM_ERR_ARG;
+    if (cos_t && (!sin_t || !positions)) return TM_ERR_ARG;
+    if (write_kv && (!slots || !k_pool || !v_pool)) return TM_ERR_ARG;
+    dim3 grid(T, H + 2 * KVH);
+    if (dtype == TM_F32)
+        rope_kv_write_kernel<float><<<grid, 64, 0, stream>>>((float*)qkv, H, KVH, D, rot, cos_t, sin_t, positions,
+                                                            slots, (float*)k_pool, (float*)v_pool, write_kv);
+    else if (dtype == TM_BF16)
+        rope_kv_write_kernel<bf16_t><<<grid, 64, 0, stream>>>((bf16_t*)qkv, H, KVH, D, rot, cos_t, sin_t,
+                                                             positions, slots, (bf16_t*)k_pool, (bf16_t*)v_pool,
+                                                             write_kv);
+    else
+        return TM_ERR_ARG;
+    TM_CHECK_LAUNCH();
+    return TM_OK;
+}
+
+// ------------------------------------------------------------------------------------------
+// out[t, i] = silu(gu[t, i]) * gu[t, I + i]           (reference src/infer/model/layers.py:164)
+// ------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t total) {
+    for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (size_t)gridDim.x * blockDim.x) {
+        const size_t t = idx / I;
+        const int i = (int)(idx - t * I);
+        const float g = Elem<T>::load(gu + t * 2 * I + i);
+        const float u = Elem<T>::load(gu + t * 2 * I + I + i);
+        Elem<T>::store(out + idx, g / (1.f + expf(-g)) * u);
+    }
+}
+
+extern "C" int tm_silu_mul(const void* gu, void* out, int dtype, int T, int I, hipStream_t stream) {
+    if (T <= 0) return TM_OK;
+    if (I <= 0) return TM_ERR_ARG;
+    const size_t total = (size_t)T * I;
+    size_t want = (total + 255) / 256;
+    const int blocks = (int)(want < 16384 ? want : 16384);
+    if (dtype == TM_F32)
+        silu_mul_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gu, (float*)out, I, total);
+    else if (dtype == TM_BF16)
+        silu_mul_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, I, total);
+    else
+        return TM_ERR_ARG;
+    TM_CHECK_LAUNCH();
+    return TM_OK;
+}
+
+// ------------------------------------------------------------------------------------------
+// type conversion of a flat array
+// ------------------------------------------------------------------------------------------
+template <typename TI, typename TO>
+__global__ void convert_kernel(const TI* __restrict__ in, TO* __restrict__ out, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+        Elem<TO>::store(out + i, Elem<TI>::load(in + i));
+}
+
+extern "C" int tm_convert(const void* in, int in_dtype, void* out, int out_dtype, long long n,
+                          hipStream_t stream) {
+    if (n <= 0) return TM_OK;
+    size_t want = ((size_t)n + 255) / 256;
+    const int blocks = (int)(want < 16384 ? want : 16384);
+    if (in_dtype == TM_BF16 && out_dtype == TM_F32)
+        convert_kernel<bf16_t, float><<<blocks, 256, 0, stream>>>((const bf16_t*)in, (float*)out, (size_t)n);
+    else if (in_dtype == TM_F32 && out_dtype == TM_BF16)
+        convert_kernel<float, bf16_t><<<blocks, 256, 0, stream>>>((const float*)in, (bf16_t*)out, (size_t)n);
+    else
+        return TM_ERR_ARG;
+    TM_CHECK_LAUNCH();
+    return TM_OK;
+}

@@ -1,0 +1,34 @@
+"""From a model folder to a model on the GPU (reference src/infer/model/loader.py:32-41,49-95)."""
+from __future__ import annotations
+
+from pathlib import Path
+
+import torch
+
+from tokenmill_amd.config.registry import load_config
+from tokenmill_amd.weights.loader import read_checkpoint
+
+
+def resolve_dtype(name: str) -> torch.dtype:
+    """auto = bfloat16, the type serving uses (reference src/infer/model/loader.py:32-35 picks the
+    16-bit type on a GPU); float32 = the true 32-bit path."""
+    try:
+        return {"auto": torch.bfloat16, "bfloat16": torch.bfloat16, "float32": torch.float32}[name]
+    except KeyError:
+        raise ValueError(f"dtype '{name}' is not one of auto, bfloat16, float32") from None
+
+
+def resolve_device(name: str) -> torch.device:
+    """There is no CPU path: the device is a GPU or the call fails."""
+    if not torch.cuda.is_available():
+        raise RuntimeError("tokenmill_amd needs a GPU (gfx950); none is visible")
+    return torch.device("cuda:0" if name == "auto" else name)
+
+
+def load_model(model_dir: str | Path, dtype: torch.dtype, device: torch.device, max_positions: int | None = None):
+    """The model that config.json names, with its weights on ``device``."""
+    arch, cfg = load_config(model_dir)
+    model = arch.build_model(cfg, max_positions)
+    tensors = read_checkpoint(model_dir, model.tensor_specs(), dtype, device, model.ignorable)
+    model.load(tensors, dtype, device)
+    return model

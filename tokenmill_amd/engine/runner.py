@@ -1,0 +1,176 @@
+"""The step function: one batch of (request, its next tokens) in, logits at the wanted places out.
+
+It is the reference's ModelRunner.prepare/execute (reference src/infer/engine/model_runner.py:40-97)
+with three differences: any row of the step may ask for logits, not only a request's last; the
+per-step metadata goes to the device in ONE pinned buffer and one copy instead of one per array;
+and attention reads the cache in place, so no per-request segment objects are built.
+
+A step runs only the tokens it is given. Portions of prompts (any length, starting anywhere) and
+single decoded tokens sit side by side in one flat batch; every token carries its absolute
+position in its own request and the flat cache slot its key and value go to.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+import numpy as np
+import torch
+
+from tokenmill_amd.cache.manager import RELEASED, RequestCache
+from tokenmill_amd.cache.pool import CachePools
+from tokenmill_amd.parts.base import GroupStep, StepContext
+
+
+@dataclass
+class StepEntry:
+    """One request's share of a step."""
+    cache: RequestCache              # its block tables and state slot
+    start: int                       # position of tokens[0] = number of its tokens already cached
+    tokens: list[int]
+    want: list[int] = field(default_factory=list)    # indices into ``tokens`` whose logits are wanted
+
+
+class StepError(ValueError):
+    """The batch cannot run as given (an id outside the vocabulary, a position without a page, ...)."""
+
+
+class ModelRunner:
+    def __init__(self, model, pools: CachePools, max_positions: int):
+        self.model = model
+        self.pools = pools
+        self.page_size = pools.page_size
+        self.max_positions = max_positions
+        self.device = model.device
+        self.vocab = model.head.vocab
+        self._pinned = torch.empty(1 << 14, dtype=torch.int32, pin_memory=True)
+        self._copied = torch.cuda.Event()
+        self._copy_pending = False
+
+    # ------------------------------------------------------------------------------------------------
+
+    def _staging(self, n: int) -> np.ndarray:
+        if self._copy_pending:
+            self._copied.synchronize()            # the last step's copy has left the buffer
+            self._copy_pending = False
+        if self._pinned.numel() < n:
+            self._pinned = torch.empty(max(n, 2 * self._pinned.numel()), dtype=torch.int32, pin_memory=True)
+        return self._pinned.numpy()
+
+    def prepare(self, entries: list[StepEntry]) -> tuple[StepContext, list[int]]:
+        """Flatten the entries into device metadata. Returns the context and, for each wanted logit
+        in the caller's order (entries in the given order, ``want`` in its order), its row in the
+        step's logits."""
+        if not entries:
+            raise StepError("a step needs at least one entry")
+        page = self.page_size
+        n_groups = len(self.pools.groups)
+        # prompt portions first, single tokens last (the order the attention kernels split on)
+        order = sorted(range(len(entries)), key=lambda i: len(entries[i].tokens) == 1)
+        S = len(entries)
+        T = sum(len(e.tokens) for e in entries)
+        R = sum(len(e.want) for e in entries)
+        widths = []
+        for e in entries:
+            if not e.tokens:
+                raise StepError(f"{e.cache.request_id}: an entry needs at least one token")
+            if e.start < 0 or e.start + len(e.tokens) > self.max_positions:
+                raise StepError(f"{e.cache.request_id}: positions {e.start}..{e.start + len(e.tokens) - 1} "
+                                f"exceed the model's {self.max_positions}")
+            end = e.start + len(e.tokens)
+            need = -(-end // page)
+            for g in range(n_groups):
+                if len(e.cache.tables[g]) < need:
+                    raise StepError(f"{e.cache.request_id}: {len(e.cache.tables[g])} pages do not hold {end} tokens")
+            widths.append(need)
+            for w in e.want:
+                if not 0 <= w < len(e.tokens):
+                    raise StepError(f"{e.cache.request_id}: wanted place {w} is not among its {len(e.tokens)} tokens")
+        W = max(widths)
+        n_ints = 3 * T + (S + 1) + 2 * S + max(R, 1) + n_groups * (T + S * W)
+        buf = self._staging(n_ints)
+        off = 0
+
+        def take(n):
+            nonlocal off
+            view = buf[off:off + n]
+            span = (off, n)
+            off += n
+            return view, span
+
+        ids, ids_s = take(T)
+        pos, pos_s = take(T)
+        seq_of, seq_s = take(T)
+        cu, cu_s = take(S + 1)
+        ctx_lens, ctx_s = take(S)
+        slots_state, st_s = take(S)
+        rows, rows_s = take(max(R, 1))
+        g_slot, g_tab = [], []
+        for _ in range(n_groups):
+            g_slot.append(take(T))
+            g_tab.append(take(S * W))
+
+        row0 = 0
+        first_row = [0] * S
+        q_lens, starts = [], []
+        cu[0] = 0
+        for s, i in enumerate(order):
+            e = entries[i]
+            n = len(e.tokens)
+            toks = np.asarray(e.tokens, dtype=np.int64)
+            if toks.min() < 0 or toks.max() >= self.vocab:
+                raise StepError(f"{e.cache.request_id}: a token id is outside the vocabulary of {self.vocab}")
+            ids[row0:row0 + n] = toks
+            p = np.arange(e.start, e.start + n, dtype=np.int64)
+            pos[row0:row0 + n] = p
+            seq_of[row0:row0 + n] = s
+            cu[s + 1] = row0 + n
+            ctx_lens[s] = e.start + n
+            slots_state[s] = e.cache.state_slot
+            for g in range(n_groups):
+                table = np.asarray(e.cache.tables[g][:widths[i]], dtype=np.int64)
+                pages = table[p // page]
+                if (pages == RELEASED).any():
+                    raise StepError(f"{e.cache.request_id}: a token would be written to a page already given back")
+                g_slot[g][0][row0:row0 + n] = pages * page + p % page
+                tab = g_tab[g][0][s * W:(s + 1) * W]
+                tab[:widths[i]] = np.where(table == RELEASED, 0, table)   # never read: below the window
+                tab[widths[i]:] = 0                                       # padding: never read either
+            first_row[i] = row0
+            q_lens.append(n)
+            starts.append(e.start)
+            row0 += n
+        r = 0
+        for i, e in enumerate(entries):
+            for w in e.want:
+                rows[r] = first_row[i] + w
+                r += 1
+        if R == 0:
+            rows[0] = 0
+
+        dev = self._pinned[:off].to(self.device, non_blocking=True)
+        self._copied.record()
+        self._copy_pending = True
+
+        def d(span):
+            return dev[span[0]:span[0] + span[1]]
+
+        groups = [GroupStep(block_tables=d(g_tab[g][1]).view(S, W), slot_mapping=d(g_slot[g][1]))
+                  for g in range(n_groups)]
+        ctx = StepContext(
+            num_tokens=T, num_seqs=S, token_ids=d(ids_s), positions=d(pos_s), seq_of_token=d(seq_s),
+            cu_q_lens=d(cu_s), context_lens=d(ctx_s), state_slots=d(st_s), logit_rows=d(rows_s)[:R], groups=groups,
+            q_lens=q_lens, start_positions=starts, max_q_len=max(q_lens),
+            max_context_len=max(s0 + n for s0, n in zip(starts, q_lens)), num_logit_rows=R,
+            num_decode=sum(1 for n in q_lens if n == 1))
+        return ctx, list(range(R))
+
+    @torch.inference_mode()
+    def step(self, entries: list[StepEntry]) -> torch.Tensor:
+        """Run one step. Returns float32 logits [R, vocab] on the device: one row per wanted place,
+        entries in the given order and each entry's ``want`` in its order."""
+        for e in entries:
+            if e.cache.fresh:                     # per-request state starts from zero at (re)admission
+                self.pools.reset_state_slot(e.cache.state_slot)
+                e.cache.fresh = False
+        ctx, _ = self.prepare(entries)
+        return self.model.forward(ctx, self.pools.views)

@@ -1,0 +1,217 @@
+"""Checked calls into the HIP kernels.
+
+Every wrapper checks on the host that the operands are on the GPU, contiguous where the kernel
+assumes it, of a type the kernel has, and of shapes that fit each other and the kernel's limits,
+BEFORE anything is launched; a kernel never sees a size it was not written for. Refusals raise
+``KernelArgumentError`` with the offending value.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_float, c_int, c_longlong, c_void_p
+
+import torch
+
+from tokenmill_amd.hip.library import library
+
+F32, BF16 = 0, 1
+_CODES = {torch.float32: F32, torch.bfloat16: BF16}
+
+
+class KernelArgumentError(ValueError):
+    pass
+
+
+def _need(cond: bool, msg: str) -> None:
+    if not cond:
+        raise KernelArgumentError(msg)
+
+
+def code(dtype: torch.dtype) -> int:
+    _need(dtype in _CODES, f"kernels exist for float32 and bfloat16, not {dtype}")
+    return _CODES[dtype]
+
+
+def _gpu(*tensors: torch.Tensor | None) -> None:
+    for t in tensors:
+        if t is not None:
+            _need(t.is_cuda, "kernel operand is not on the GPU (there is no CPU path)")
+
+
+def _p(t: torch.Tensor | None) -> c_void_p:
+    return c_void_p(0 if t is None else t.data_ptr())
+
+
+def _stream() -> c_void_p:
+    return c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _check(rc: int, name: str) -> None:
+    if rc == 1:
+        raise KernelArgumentError(f"{name}: the kernel refused its arguments")
+    if rc != 0:
+        raise RuntimeError(f"{name}: launch failed (code {rc})")
+
+
+def _ints(t: torch.Tensor, n: int, name: str) -> None:
+    _need(t.dtype == torch.int32 and t.is_contiguous() and t.numel() >= n, f"{name} must be contiguous int32 [{n}]")
+
+
+# --------------------------------------------------------------------------------------------
+
+def embed_gather(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[t] = table[ids[t]] as 32-bit rows. table [V, hidden], ids int32 [T], out float32 [T, hidden]."""
+    _gpu(table, ids, out)
+    T = ids.numel()
+    V, hidden = table.shape
+    _need(table.is_contiguous() and out.is_contiguous(), "embed_gather: operands must be contiguous")
+    _need(out.dtype == torch.float32 and tuple(out.shape) == (T, hidden), "embed_gather: out must be float32 [T, hidden]")
+    _ints(ids, T, "ids")
+    _check(library().tm_embed_gather(_p(table), code(table.dtype), _p(ids), _p(out), c_int(T), c_int(hidden),
+                                     c_int(V), _stream()), "embed_gather")
+    return out
+
+
+def add_rmsnorm(resid: torch.Tensor, delta: torch.Tensor | None, weight: torch.Tensor, eps: float,
+                out: torch.Tensor, rows: torch.Tensor | None = None) -> torch.Tensor:
+    """rows None: resid += delta (in place, 32-bit), out = rmsnorm(resid) * weight, all rows.
+    rows given: out[r] = rmsnorm(resid[rows[r]] + delta[rows[r]]) * weight; resid is not written."""
+    _gpu(resid, delta, weight, out, rows)
+    T, hidden = resid.shape
+    R = T if rows is None else rows.numel()
+    _need(resid.dtype == torch.float32 and resid.is_contiguous(), "add_rmsnorm: the residual stream is contiguous float32")
+    _need(tuple(out.shape) == (R, hidden) and out.is_contiguous(), f"add_rmsnorm: out must be [{R}, {hidden}]")
+    if delta is not None:
+        _need(delta.dtype == out.dtype and tuple(delta.shape) == (T, hidden) and delta.is_contiguous(),
+              "add_rmsnorm: delta must match the residual's shape and out's type")
+    _need(tuple(weight.shape) == (hidden,) and weight.is_contiguous(), "add_rmsnorm: weight must be [hidden]")
+    _need(out.dtype == torch.bfloat16 or weight.dtype == torch.float32, "add_rmsnorm: a float32 output needs float32 weights")
+    if rows is not None:
+        _ints(rows, R, "rows")
+    _need(eps > 0, "add_rmsnorm: eps must be positive")
+    _check(library().tm_add_rmsnorm(_p(resid), _p(delta), _p(rows), _p(weight), code(weight.dtype), _p(out),
+                                    code(out.dtype), c_int(R), c_int(hidden), c_float(eps), _stream()), "add_rmsnorm")
+    return out
+
+
+def rope_kv_write(qkv: torch.Tensor, H: int, KVH: int, D: int, cos: torch.Tensor | None, sin: torch.Tensor | None,
+                  positions: torch.Tensor | None, slots: torch.Tensor | None, k_pool: torch.Tensor | None,
+                  v_pool: torch.Tensor | None) -> None:
+    """Rotate q and k of qkv [T, (H + 2 KVH) D] in place by each token's position and store k, v at
+    the tokens' cache slots. cos/sin float32 [max_pos, rot/2] or None (store only); pools
+    [pages, page, KVH, D] or None (rotate only). A slot < 0 is not stored."""
+    _gpu(qkv, cos, sin, positions, slots, k_pool, v_pool)
+    T = qkv.shape[0]
+    _need(qkv.is_contiguous() and qkv.shape[1] == (H + 2 * KVH) * D, "rope_kv_write: qkv must be contiguous [T, (H+2KVH)D]")
+    rot = 0
+    if cos is not None:
+        _need(sin is not None and positions is not None, "rope_kv_write: cos needs sin and positions")
+        _need(cos.dtype == torch.float32 and sin.dtype == torch.float32 and cos.is_contiguous() and sin.is_contiguous()
+              and cos.shape == sin.shape and cos.dim() == 2, "rope_kv_write: cos/sin must be float32 [max_pos, rot/2]")
+        rot = 2 * cos.shape[1]
+        _need(0 < rot <= D, f"rope_kv_write: rotary width {rot} does not fit head size {D}")
+        _ints(positions, T, "positions")
+    write = k_pool is not None
+    if write:
+        _need(v_pool is not None and slots is not None, "rope_kv_write: a cache write needs both pools and slots")
+        for pool in (k_pool, v_pool):
+            _need(pool.dtype == qkv.dtype and pool.is_contiguous() and pool.dim() == 4 and
+                  tuple(pool.shape[2:]) == (KVH, D), "rope_kv_write: pools must be [pages, page, KVH, D] of qkv's type")
+        _ints(slots, T, "slots")
+    _check(library().tm_rope_kv_write(_p(qkv), code(qkv.dtype), c_int(T), c_int(H), c_int(KVH), c_int(D), c_int(rot),
+                                      _p(cos), _p(sin), _p(positions), _p(slots), _p(k_pool), _p(v_pool),
+                                      c_int(1 if write else 0), _stream()), "rope_kv_write")
+
+
+def silu_mul(gu: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[t, i] = silu(gu[t, i]) * gu[t, I + i]; gu [T, 2I], out [T, I]."""
+    _gpu(gu, out)
+    T, two_i = gu.shape
+    _need(two_i % 2 == 0 and tuple(out.shape) == (T, two_i // 2) and gu.is_contiguous() and out.is_contiguous()
+          and gu.dtype == out.dtype, "silu_mul: gu [T, 2I] and out [T, I] of one type, contiguous")
+    _check(library().tm_silu_mul(_p(gu), _p(out), code(gu.dtype), c_int(T), c_int(two_i // 2), _stream()), "silu_mul")
+    return out
+
+
+def convert(src: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    _gpu(src, out)
+    _need(src.is_contiguous() and out.is_contiguous() and src.numel() == out.numel(), "convert: same size, contiguous")
+    _check(library().tm_convert(_p(src), code(src.dtype), _p(out), code(out.dtype), c_longlong(src.numel()),
+                                _stream()), "convert")
+    return out
+
+
+def gemm_nt_tiled(a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, out: torch.Tensor) -> torch.Tensor:
+    """out[M, N] = a[M, K] @ w[N, K]^T (+ bias[N]) with 32-bit multiply-adds in ascending k.
+    a and out may be row-strided views (unit stride in the last dimension)."""
+    _gpu(a, w, bias, out)
+    M, K = a.shape
+    N = w.shape[0]
+    _need(w.shape[1] == K and w.is_contiguous() and w.dtype == a.dtype, "gemm: w must be contiguous [N, K] of a's type")
+    _need(a.stride(1) == 1 and out.stride(1) == 1 and tuple(out.shape) == (M, N), "gemm: a [M, K], out [M, N], unit inner stride")
+    _need(not (a.dtype == torch.float32 and out.dtype != torch.float32), "gemm: float32 inputs give float32 outputs")
+    if bias is not None:
+        _need(tuple(bias.shape) == (N,) and bias.is_contiguous(), "gemm: bias must be [N]")
+        _need(not (a.dtype == torch.float32 and bias.dtype != torch.float32), "gemm: float32 inputs need a float32 bias")
+    _need(M <= 64 * 65535, "gemm: too many rows for one launch")
+    lda = a.stride(0) if M > 1 else max(K, a.stride(0))
+    ldc = out.stride(0) if M > 1 else max(N, out.stride(0))
+    _check(library().tm_gemm_nt_tiled(_p(a), c_int(lda), _p(w), _p(bias),
+                                      c_int(code(bias.dtype) if bias is not None else -1), _p(out), c_int(ldc),
+                                      c_int(M), c_int(N), c_int(K), code(a.dtype), code(out.dtype), _stream()),
+           "gemm_nt_tiled")
+    return out
+
+
+def attn_paged_generic(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
+                       block_tables: torch.Tensor, seq_of_token: torch.Tensor, positions: torch.Tensor,
+                       H: int, KVH: int, D: int, scale: float, window: int = 0) -> torch.Tensor:
+    """Attention of every token of the step over its request's cached keys (its own included).
+    q: [T, >= H*D] view with unit inner stride (q heads first in each row); out [T, H*D];
+    pools [pages, page, KVH, D]; block_tables int32 [S, W]; seq_of_token, positions int32 [T]."""
+    _gpu(q, out, k_pool, v_pool, block_tables, seq_of_token, positions)
+    T = q.shape[0]
+    _need(q.stride(1) == 1 and q.shape[1] >= H * D and out.is_contiguous() and tuple(out.shape) == (T, H * D),
+          "attention: q [T, >=H*D] unit inner stride, out contiguous [T, H*D]")
+    _need(q.dtype == out.dtype == k_pool.dtype == v_pool.dtype, "attention: q, out and pools share one type")
+    _need(H % KVH == 0 and D % 4 == 0 and 0 < D <= 256, f"attention(generic): head size {D} must be a multiple of 4 up to 256")
+    for pool in (k_pool, v_pool):
+        _need(pool.is_contiguous() and pool.dim() == 4 and tuple(pool.shape[2:]) == (KVH, D),
+              "attention: pools must be contiguous [pages, page, KVH, D]")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous(),
+          "attention: block_tables must be contiguous int32 [S, W]")
+    _ints(seq_of_token, T, "seq_of_token")
+    _ints(positions, T, "positions")
+    _need(window >= 0, "attention: window must be >= 0 (0 = every key)")
+    q_stride = q.stride(0) if T > 1 else max(q.stride(0), H * D)
+    _check(library().tm_attn_paged_generic(_p(q), c_int(q_stride), _p(out), c_int(H * D), _p(k_pool), _p(v_pool),
+                                           _p(block_tables), c_int(block_tables.shape[1]), _p(seq_of_token),
+                                           _p(positions), c_int(T), c_int(H), c_int(KVH), c_int(D),
+                                           c_int(k_pool.shape[1]), c_float(scale), c_int(window), code(q.dtype),
+                                           _stream()), "attn_paged_generic")
+    return out
+
+
+def argmax_rows(logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    _gpu(logits, out)
+    R, V = logits.shape
+    _need(logits.dtype == torch.float32 and logits.is_contiguous(), "argmax: logits must be contiguous float32 [R, V]")
+    _ints(out, R, "out")
+    _check(library().tm_argmax_rows(_p(logits), c_int(R), c_int(V), _p(out), _stream()), "argmax_rows")
+    return out
+
+
+def sample_rows(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
+                u: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """One token per row: argmax where temperature <= 1e-5 or top_k == 1, else the inverse CDF at
+    u of softmax(logits / temperature) after the top-k / top-p filters, in vocabulary order."""
+    _gpu(logits, temperature, top_k, top_p, u, out)
+    R, V = logits.shape
+    _need(logits.dtype == torch.float32 and logits.is_contiguous(), "sample: logits must be contiguous float32 [R, V]")
+    for t, name in ((temperature, "temperature"), (top_p, "top_p"), (u, "u")):
+        _need(t.dtype == torch.float32 and t.is_contiguous() and t.numel() == R, f"sample: {name} must be float32 [R]")
+    _ints(top_k, R, "top_k")
+    _ints(out, R, "out")
+    _check(library().tm_sample_rows(_p(logits), c_int(R), c_int(V), _p(temperature), _p(top_k), _p(top_p), _p(u),
+                                    _p(out), _stream()), "sample_rows")
+    return out

@@ -1,0 +1,125 @@
+"""What every part of a layer looks like to the model that holds it.
+
+A part (mixer, feed-forward, norm, position encoding, embedding, output head) gets its sizes and
+constants as constructor parameters, declares the checkpoint tensors it wants under a prefix,
+takes them in ``load`` and computes in ``forward``. No part knows which model it is in.
+
+Per step, every part sees the same ``StepContext``: the flat batch of tokens with each token's
+absolute position and request, and per cache group the block tables and slot mapping.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+import torch
+
+from tokenmill_amd.weights.loader import TensorSpec
+
+
+# ------------------------------------------------------------------------------------------------
+# what a mixer asks of the cache manager
+# ------------------------------------------------------------------------------------------------
+
+@dataclass(frozen=True)
+class KVCacheSpec:
+    """Keys and values in pages. ``window``: None keeps every token; W keeps the last W."""
+    kv_heads: int
+    head_dim: int
+    window: int | None = None
+
+
+@dataclass(frozen=True)
+class StateSpec:
+    """State of fixed size per request (zeroed when a request is admitted)."""
+    shape: tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+@dataclass
+class KVCacheView:
+    """One cache layer as a mixer sees it."""
+    k: torch.Tensor              # [pages, page_size, kv_heads, head_dim]
+    v: torch.Tensor
+    group: int                   # index into StepContext.groups
+    write: bool = True           # False: this layer reads a cache that another layer writes
+
+
+@dataclass
+class StateView:
+    state: torch.Tensor          # [slots, *shape]; row StepContext.state_slots[s] belongs to request s
+
+
+# ------------------------------------------------------------------------------------------------
+# the step as parts see it
+# ------------------------------------------------------------------------------------------------
+
+@dataclass
+class GroupStep:
+    block_tables: torch.Tensor   # int32 [S, W]: page ids of each request of the step, in this group
+    slot_mapping: torch.Tensor   # int32 [T]: flat cache slot of each token of the step, in this group
+
+
+@dataclass
+class StepContext:
+    num_tokens: int
+    num_seqs: int
+    token_ids: torch.Tensor      # int32 [T]
+    positions: torch.Tensor      # int32 [T]  absolute position of each token in its own request
+    seq_of_token: torch.Tensor   # int32 [T]  index of the token's request in this step
+    cu_q_lens: torch.Tensor      # int32 [S+1] first row of each request's tokens
+    context_lens: torch.Tensor   # int32 [S]  tokens of the request once this step is done
+    state_slots: torch.Tensor    # int32 [S]
+    logit_rows: torch.Tensor     # int32 [R]  rows whose logits are wanted
+    groups: list[GroupStep] = field(default_factory=list)
+    # host-side copies for choosing kernels and grids
+    q_lens: list[int] = field(default_factory=list)
+    start_positions: list[int] = field(default_factory=list)
+    max_q_len: int = 0
+    max_context_len: int = 0
+    num_logit_rows: int = 0
+    # S entries are ordered with the q_len == 1 entries last; this many of them:
+    num_decode: int = 0
+
+
+# ------------------------------------------------------------------------------------------------
+# the part interfaces
+# ------------------------------------------------------------------------------------------------
+
+class Part:
+    """Base of all parts: declares tensors, takes them, computes."""
+
+    def tensor_specs(self, prefix: str) -> dict[str, TensorSpec]:
+        """Checkpoint tensors this part expects, by full name."""
+        return {}
+
+    def load(self, tensors: dict[str, torch.Tensor], prefix: str) -> None:
+        """Take this part's tensors (already on the device, in their storage type)."""
+
+
+class Norm(Part):
+    def add_norm(self, resid: torch.Tensor, delta: torch.Tensor | None, out_dtype: torch.dtype,
+                 rows: torch.Tensor | None = None) -> torch.Tensor:
+        """resid (float32 [T, hidden]) += delta, in place; returns norm(resid) in ``out_dtype``.
+        With ``rows``: only those rows, and resid is left as it is."""
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    def encode_and_store(self, qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
+                         step: StepContext, cache: KVCacheView) -> None:
+        """Encode positions into q and k of ``qkv`` in place and store k, v into the cache."""
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    def cache_spec(self) -> KVCacheSpec | StateSpec | None:
+        return None
+
+    def forward(self, x: torch.Tensor, step: StepContext, cache) -> torch.Tensor:
+        """x: normed [T, hidden] in the compute type -> [T, hidden] to be added to the residual."""
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, x: torch.Tensor, step: StepContext) -> torch.Tensor:
+        raise NotImplementedError

@@ -1,0 +1,62 @@
+"""y = x W^T + b with W stored [out, in] (reference src/infer/model/layers.py:139-140,159-160).
+
+Several checkpoint tensors may be stacked along the output dimension into one matrix at load time
+(q, k, v; gate, up), as the reference's loader does by row ranges
+(reference src/infer/model/loader.py:44-46,68-70,111-116).
+"""
+from __future__ import annotations
+
+import torch
+
+from tokenmill_amd.hip import ops
+from tokenmill_amd.parts.base import Part
+from tokenmill_amd.weights.loader import TensorSpec
+
+
+class Linear(Part):
+    def __init__(self, in_features: int, out_features: list[int] | int, names: list[str] | str,
+                 bias: bool = False):
+        self.in_features = in_features
+        self.out_splits = [out_features] if isinstance(out_features, int) else list(out_features)
+        self.names = [names] if isinstance(names, str) else list(names)
+        assert len(self.names) == len(self.out_splits)
+        self.out_features = sum(self.out_splits)
+        self.has_bias = bias
+        self.weight: torch.Tensor | None = None
+        self.bias: torch.Tensor | None = None
+
+    def tensor_specs(self, prefix: str) -> dict[str, TensorSpec]:
+        specs = {}
+        for name, n in zip(self.names, self.out_splits):
+            specs[f"{prefix}{name}.weight"] = TensorSpec((n, self.in_features))
+            if self.has_bias:
+                specs[f"{prefix}{name}.bias"] = TensorSpec((n,))
+        return specs
+
+    def load(self, tensors, prefix: str) -> None:
+        ws = [tensors[f"{prefix}{name}.weight"] for name in self.names]
+        self.weight = ws[0] if len(ws) == 1 else torch.cat(ws, dim=0).contiguous()
+        if self.has_bias:
+            bs = [tensors[f"{prefix}{name}.bias"] for name in self.names]
+            self.bias = bs[0] if len(bs) == 1 else torch.cat(bs, dim=0).contiguous()
+            if self.weight.dtype == torch.float32 and self.bias.dtype != torch.float32:
+                self.bias = self.bias.float()          # a 32-bit product adds a 32-bit bias
+
+    def use_weight(self, weight: torch.Tensor) -> None:
+        """Share another part's matrix (a tied output head)."""
+        self.weight = weight
+
+    def forward(self, x: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+        """x [M, in] (row-strided views allowed) -> [M, out] in ``out_dtype`` (default: x's type)."""
+        w = self.weight
+        out_dtype = out_dtype or x.dtype
+        if w.dtype != x.dtype:
+            # a matrix the checkpoint stores in 32-bit stays 32-bit: widen the activations for it
+            x = ops.convert(x.contiguous(), torch.empty(x.shape, dtype=w.dtype, device=x.device))
+        inner_dtype = torch.float32 if x.dtype == torch.float32 else out_dtype
+        out = torch.empty((x.shape[0], self.out_features), dtype=inner_dtype, device=x.device)
+        from tokenmill_amd.hip import gemm
+        gemm.linear(x, w, self.bias, out)
+        if out.dtype != out_dtype:
+            out = ops.convert(out, torch.empty(out.shape, dtype=out_dtype, device=out.device))
+        return out

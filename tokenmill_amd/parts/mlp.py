@@ -1,0 +1,29 @@
+"""SwiGLU feed-forward: down(silu(gate(x)) * up(x)), gate and up stacked into one product
+(reference src/infer/model/layers.py:153-164)."""
+from __future__ import annotations
+
+import torch
+
+from tokenmill_amd.hip import ops
+from tokenmill_amd.parts.base import FeedForward, StepContext
+from tokenmill_amd.parts.linear import Linear
+
+
+class SwiGLU(FeedForward):
+    def __init__(self, hidden: int, intermediate: int, bias: bool = False,
+                 names: tuple[str, str, str] = ("gate_proj", "up_proj", "down_proj")):
+        self.hidden, self.intermediate = hidden, intermediate
+        self.gate_up = Linear(hidden, [intermediate, intermediate], list(names[:2]), bias=bias)
+        self.down = Linear(intermediate, hidden, names[2], bias=bias)
+
+    def tensor_specs(self, prefix: str):
+        return {**self.gate_up.tensor_specs(prefix), **self.down.tensor_specs(prefix)}
+
+    def load(self, tensors, prefix: str) -> None:
+        self.gate_up.load(tensors, prefix)
+        self.down.load(tensors, prefix)
+
+    def forward(self, x: torch.Tensor, step: StepContext | None = None) -> torch.Tensor:
+        gu = self.gate_up.forward(x)
+        act = ops.silu_mul(gu, torch.empty((x.shape[0], self.intermediate), dtype=gu.dtype, device=x.device))
+        return self.down.forward(act)
