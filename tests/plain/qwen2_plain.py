@@ -182,14 +182,14 @@ def decoder_layer(x: torch.Tensor, w: dict, i: int, cfg: dict, positions, cos, s
 
 
 def forward_logits(w: dict, cfg: dict, ids: list[int], dt=torch.float32,
-                   windows: list | None = None) -> torch.Tensor:
+                   windows: list | None = None, offset: int = 0) -> torch.Tensor:
     """Logits [T, vocab] (32-bit) at every position of one whole sequence.
 
     reference src/infer/model/qwen2.py:43-52: embedding rows (no scaling), the layers in order,
     the final norm, then hidden @ W_out^T with W_out the embedding table when tied (:39-41)."""
     T = len(ids)
-    positions = torch.arange(T)
-    cos, sin = rope_tables(T, cfg["head_dim"], cfg["theta"])
+    positions = torch.arange(T) + offset        # offset: only for the test that distances alone count
+    cos, sin = rope_tables(T + offset, cfg["head_dim"], cfg["theta"])
     x = rnd(w["model.embed_tokens.weight"], dt)[torch.tensor(ids, dtype=torch.long)]
     for i in range(cfg["layers"]):
         x = decoder_layer(x, w, i, cfg, positions, cos, sin, dt, windows[i] if windows else None)

@@ -1,0 +1,235 @@
+"""Pins of the plain implementation: what fixes each formula beside the reference's text.
+
+The reference is read, not run, and holds no numeric vectors for its layers (its layer tests
+compare with another library's modules, reference tests/test_layers.py:18-93). So each part is
+pinned by special cases that reduce to a torch library routine, by invariants, and by the vectors
+the reference's sampler tests do hold (reference tests/test_sampling.py:11-31). Each check is
+chosen so that a plausible mistake fails it: a wrong sign or pairing in the rotation, a norm whose
+weight multiplies before the rounding, a mask off by one, a kv head mapped by modulo.
+"""
+from __future__ import annotations
+
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from conftest import TINY, random_ids
+from plain import qwen2_plain as P
+
+
+# ----------------------------------------------------------------------------------------------- norm
+
+def test_rmsnorm_is_torchs_rms_norm_in_float32():
+    torch.manual_seed(0)
+    x, w = torch.randn(7, 96) * 3, torch.rand(96) + 0.5
+    for eps in (1e-6, 1e-2):
+        torch.testing.assert_close(P.rms_norm(x, w, eps), F.rms_norm(x, (96,), w, eps), rtol=1e-6, atol=1e-6)
+
+
+def test_rmsnorm_eps_is_inside_the_root_and_no_mean_is_subtracted():
+    x = torch.full((1, 4), 2.0)                       # mean 2, mean of squares 4
+    out = P.rms_norm(x, torch.ones(4), eps=5.0)
+    torch.testing.assert_close(out, torch.full((1, 4), 2.0 / 3.0))      # 2 / sqrt(4 + 5), not 0, not 2/(2+5)
+    # weight used as it is (not 1 + w): zero weight gives zero
+    assert P.rms_norm(x, torch.zeros(4), 1e-6).abs().max() == 0
+
+
+def test_rmsnorm_rounds_before_the_weight_multiplies():
+    """reference tests/test_layers.py:28-37 checks this cast order in 16-bit against the library."""
+    torch.manual_seed(1)
+    x = torch.randn(64, 256) * 4
+    w = (torch.rand(256) + 0.5).bfloat16().float()
+    got = P.rms_norm(x, w, 1e-6, torch.bfloat16)
+    normed = x * torch.rsqrt((x * x).mean(-1, keepdim=True) + 1e-6)
+    first = (w * normed.bfloat16().float()).bfloat16().float()         # round, then weight
+    other = (w * normed).bfloat16().float()                            # weight, then round
+    assert torch.equal(got, first)
+    assert not torch.equal(first, other)                               # the two orders do differ on this input
+
+
+# ----------------------------------------------------------------------------------------------- rope
+
+def test_rope_with_one_pair_is_a_plane_rotation_by_the_position():
+    cos, sin = P.rope_tables(50, 2, theta=12345.0)                     # one frequency: theta^0 = 1
+    x = torch.tensor([[[1.0, 0.0]], [[0.0, 1.0]]])
+    for p in (0, 1, 7, 49):
+        y = P.apply_rope(x, cos, sin, torch.tensor([p, p]))
+        torch.testing.assert_close(y[0, 0], torch.tensor([math.cos(p), math.sin(p)]), rtol=1e-5, atol=1e-6)
+        torch.testing.assert_close(y[1, 0], torch.tensor([-math.sin(p), math.cos(p)]), rtol=1e-5, atol=1e-6)
+
+
+def test_rope_pairs_element_j_with_j_plus_half_at_frequency_theta_pow():
+    D, theta, p = 16, 10000.0, 3
+    cos, sin = P.rope_tables(8, D, theta)
+    for j in range(D // 2):
+        x = torch.zeros(1, 1, D)
+        x[0, 0, j] = 1.0
+        y = P.apply_rope(x, cos, sin, torch.tensor([p]))[0, 0]
+        angle = p * theta ** (-2.0 * j / D)
+        touched = y.nonzero().flatten().tolist()
+        assert set(touched) <= {j, j + D // 2}                         # half-split pairing, not (2j, 2j+1)
+        assert y[j].item() == pytest.approx(math.cos(angle), abs=1e-6)
+        assert y[j + D // 2].item() == pytest.approx(math.sin(angle), abs=1e-6)
+
+
+def test_rope_position_zero_is_identity_norms_stay_and_only_distances_count():
+    torch.manual_seed(2)
+    D = 32
+    cos, sin = P.rope_tables(400, D, 1e6)
+    q, k = torch.randn(1, 3, D), torch.randn(1, 3, D)
+    assert torch.equal(P.apply_rope(q, cos, sin, torch.tensor([0])), q)
+    r = P.apply_rope(q, cos, sin, torch.tensor([123]))
+    torch.testing.assert_close(r.norm(dim=-1), q.norm(dim=-1), rtol=1e-5, atol=1e-5)
+
+    def score(m, n):
+        return (P.apply_rope(q, cos, sin, torch.tensor([m])) * P.apply_rope(k, cos, sin, torch.tensor([n]))).sum(-1)
+
+    torch.testing.assert_close(score(10, 3), score(307, 300), rtol=1e-4, atol=1e-4)
+    assert (score(10, 3) - score(10, 4)).abs().max() > 1e-3
+
+
+# ----------------------------------------------------------------------------------------------- linear
+
+def test_linear_is_torchs_and_stacking_equals_separate_products():
+    torch.manual_seed(3)
+    x, w1, w2, b1, b2 = torch.randn(5, 24), torch.randn(10, 24), torch.randn(6, 24), torch.randn(10), torch.randn(6)
+    torch.testing.assert_close(P.linear(x, w1, b1), F.linear(x, w1, b1))
+    fused = P.linear(x, torch.cat([w1, w2]), torch.cat([b1, b2]))
+    torch.testing.assert_close(fused, torch.cat([P.linear(x, w1, b1), P.linear(x, w2, b2)], dim=-1))
+    assert (P.linear(x, w1, b1) - P.linear(x, w1)).abs().max() > 0.1    # the bias is really added
+
+
+# ----------------------------------------------------------------------------------------------- attention
+
+def test_attention_of_one_whole_prompt_is_torchs_sdpa():
+    torch.manual_seed(4)
+    L, H, KVH, D = 13, 6, 2, 16
+    q, k, v = torch.randn(L, H, D), torch.randn(L, KVH, D), torch.randn(L, KVH, D)
+    got = P.causal_attention(q, k, v, D ** -0.5)
+    want = F.scaled_dot_product_attention(q.transpose(0, 1)[None], k.transpose(0, 1)[None], v.transpose(0, 1)[None],
+                                          is_causal=True, scale=D ** -0.5, enable_gqa=True)[0].transpose(0, 1)
+    torch.testing.assert_close(got, want, rtol=1e-5, atol=1e-5)
+
+
+def test_attention_one_token_returns_v_and_equal_keys_average_the_visible_values():
+    torch.manual_seed(5)
+    D = 8
+    q, k, v = torch.randn(1, 2, D), torch.randn(1, 1, D), torch.randn(1, 1, D)
+    torch.testing.assert_close(P.causal_attention(q, k, v, 1.0), v.expand(1, 2, D))
+    L = 6
+    q, v = torch.randn(L, 1, D), torch.randn(L, 1, D)
+    k = torch.ones(L, 1, D)                                             # equal keys: uniform weights
+    out = P.causal_attention(q, k, v, 0.3)
+    for i in range(L):
+        torch.testing.assert_close(out[i, 0], v[:i + 1, 0].mean(0), rtol=1e-5, atol=1e-6)   # keys 0..i, key i included
+
+
+def test_attention_ignores_later_tokens_and_maps_query_head_h_to_kv_head_h_div_group():
+    torch.manual_seed(6)
+    L, H, KVH, D = 9, 6, 3, 8
+    q, k, v = torch.randn(L, H, D), torch.randn(L, KVH, D), torch.randn(L, KVH, D)
+    a = P.causal_attention(q, k, v, D ** -0.5)
+    k2, v2 = k.clone(), v.clone()
+    k2[5:] += 10.0
+    v2[5:] -= 3.0
+    b = P.causal_attention(q, k2, v2, D ** -0.5)
+    assert torch.equal(a[:5], b[:5]) and not torch.allclose(a[5:], b[5:])
+    vc = torch.zeros(L, KVH, D)
+    for g in range(KVH):
+        vc[:, g] = float(g + 1)                                         # each kv head a constant of its own
+    out = P.causal_attention(q, k, vc, D ** -0.5)
+    for h in range(H):
+        torch.testing.assert_close(out[:, h], torch.full((L, D), float(h // (H // KVH) + 1)))   # not h % KVH
+
+
+def test_attention_window_keeps_the_last_w_keys():
+    torch.manual_seed(7)
+    L, D, W = 10, 4, 3
+    q, v = torch.randn(L, 1, D), torch.randn(L, 1, D)
+    out = P.causal_attention(q, torch.ones(L, 1, D), v, 1.0, window=W)
+    for i in range(L):
+        torch.testing.assert_close(out[i, 0], v[max(0, i - W + 1):i + 1, 0].mean(0), rtol=1e-5, atol=1e-6)
+
+
+# ----------------------------------------------------------------------------------------------- mlp
+
+def test_silu_mul_is_torchs_silu_times_up():
+    torch.manual_seed(8)
+    g, u = torch.randn(4, 10) * 3, torch.randn(4, 10)
+    torch.testing.assert_close(P.silu_mul(g, u), F.silu(g) * u)
+    assert P.silu_mul(torch.zeros(3), torch.randn(3)).abs().max() == 0
+    torch.testing.assert_close(P.silu_mul(torch.tensor([30.0]), torch.tensor([2.0])), torch.tensor([60.0]))
+
+
+# ----------------------------------------------------------------------------------------------- model
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_model_rows_ignore_later_tokens_and_only_distances_count(plains, name):
+    p = plains[name]
+    ids = random_ids(20, p.cfg["vocab"], 11)
+    full = p.logits(ids)
+    torch.testing.assert_close(P.forward_logits(p.w, p.cfg, ids[:12]), full[:12], rtol=1e-5, atol=1e-6)
+    changed = ids[:12] + [(t + 1) % p.cfg["vocab"] for t in ids[12:]]
+    torch.testing.assert_close(P.forward_logits(p.w, p.cfg, changed)[:12], full[:12], rtol=1e-5, atol=1e-6)
+    shifted = P.forward_logits(p.w, p.cfg, ids, offset=37)              # rotary positions: a shift of all changes nothing
+    torch.testing.assert_close(shifted, full, rtol=1e-3, atol=2e-4)
+    assert (shifted - full).abs().max() > 0                             # (it is a different computation)
+
+
+def test_tied_model_multiplies_by_the_embedding_table_itself(plains):
+    p = plains["A"]
+    assert p.cfg["tied"] and "lm_head.weight" not in p.w
+    ids = random_ids(6, p.cfg["vocab"], 12)
+    w2 = dict(p.w)
+    w2["model.embed_tokens.weight"] = p.w["model.embed_tokens.weight"] * 2       # doubles the input rows AND the output matrix
+    a, b = p.logits(ids), P.forward_logits(w2, p.cfg, ids)
+    assert (a - b).abs().max() > 1e-3
+    untied = dict(p.cfg, tied=False)
+    w3 = dict(p.w)
+    w3["lm_head.weight"] = p.w["model.embed_tokens.weight"]
+    torch.testing.assert_close(P.forward_logits(w3, untied, ids), a)
+
+
+def test_bfloat16_mode_stays_close_to_float32_and_differs_from_it(plains):
+    p = plains["B"]
+    ids = random_ids(30, p.cfg["vocab"], 13)
+    a, b = p.logits(ids), p.logits(ids, torch.bfloat16)
+    err = (a - b).abs().max().item()
+    assert 0 < err < 2e-2 * max(1.0, a.abs().max().item())
+
+
+# ----------------------------------------------------------------------------------------------- sampler
+
+def test_greedy_is_argmax_on_the_references_vector():
+    """reference tests/test_sampling.py:11-13"""
+    for row, want in (([0.1, 3.0, 2.0], 1), ([5.0, -1.0, 4.9], 0)):
+        assert P.sample_token(torch.tensor(row), 0.0, -1, 1.0, 0, 0)[0] == want
+        assert P.sample_token(torch.tensor(row), 0.7, 1, 1.0, 0, 0)[0] == want      # top_k == 1 is greedy too
+
+
+def test_filters_on_the_references_vectors():
+    """reference tests/test_sampling.py:16-31"""
+    out = P.filter_top_k_top_p(torch.tensor([1.0, 4.0, 3.0, 2.0]), 2, 1.0)
+    assert torch.isinf(out[[0, 3]]).all() and torch.isfinite(out[[1, 2]]).all()
+    out = P.filter_top_k_top_p(torch.tensor([0.5, 0.3, 0.15, 0.05]).log(), -1, 0.7)
+    assert torch.isfinite(out[:2]).all() and torch.isinf(out[2:]).all()
+    out = P.filter_top_k_top_p(torch.tensor([10.0, 0.0]), -1, 1e-6)
+    assert torch.isfinite(out[0]) and torch.isinf(out[1])
+
+
+def test_random_stream_and_inverse_cdf():
+    us = [P.uniform_from_counter(1234, i) for i in range(2000)]
+    assert all(0.0 <= u < 1.0 for u in us) and len(set(us)) > 1990
+    assert us[:5] == [P.uniform_from_counter(1234, i) for i in range(5)]
+    assert us[:5] != [P.uniform_from_counter(1235, i) for i in range(5)]
+    assert abs(sum(us) / len(us) - 0.5) < 0.03
+    logits = torch.tensor([2.0, 1.0, 0.0])
+
+    def frac_top(t):
+        return sum(P.sample_token(logits, t, -1, 1.0, 9, i)[0] == 0 for i in range(3000)) / 3000
+
+    want = torch.softmax(logits, -1)[0].item()
+    assert abs(frac_top(1.0) - want) < 0.03                             # temperature row = softmax(logits / t)
+    assert frac_top(0.3) > frac_top(1.0) > 0.4                          # reference tests/test_sampling.py:52-62
