@@ -1,0 +1,174 @@
+"""Generation through the engine's entry points on the GPU, checked against the plain
+implementation: every token the engine produced must be the plain implementation's choice at that
+place of the engine's own sequence (or lie within the tolerance of a near-tie)."""
+from __future__ import annotations
+
+import json
+import subprocess
+import sys
+
+import pytest
+import torch
+
+from conftest import ROOT, TINY, random_ids
+from plain import qwen2_plain as P
+from tolerances import REL
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+def make_engine(model_dir, dtype_name, **kw):
+    from tokenmill_amd import EngineConfig, LLMEngine
+    base = dict(model=str(model_dir), dtype=dtype_name, block_size=16, kv_cache_mb=8, max_model_len=256,
+                max_num_seqs=32, max_num_batched_tokens=512, watermark=0.0)
+    base.update(kw)
+    return LLMEngine(EngineConfig(**base))
+
+
+def verify(plain, prompt, out, dt, params=None, seed=0):
+    """Every generated token is what the plain implementation picks after the same tokens."""
+    logits = plain.logits(list(prompt) + list(out), dt)[len(prompt) - 1:-1]
+    scale = max(1.0, float(logits.abs().max()))
+    gap = 2 * REL[dt] * scale
+    exempt = 0
+    for n, (row, tok) in enumerate(zip(logits, out)):
+        if params is None or params.greedy:
+            assert row[tok] >= row.max() - gap, f"token {n}: {tok} is not the argmax ({row[tok]} vs {row.max()})"
+            exempt += int(tok != int(row.argmax()))
+        else:
+            want, margin = P.sample_token(row, params.temperature, params.top_k, params.top_p, seed, n)
+            assert tok == want or margin < 20 * REL[dt], f"token {n}: sampled {tok}, plain {want} (margin {margin})"
+            exempt += int(tok != want)
+    return exempt
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_greedy_generation_whole_prompts(model_dirs, plains, dtype_name):
+    """BASELINE configuration A: prompts of 5 / 17 / 33 ids, whole-prompt prefill, 16 greedy tokens."""
+    from tokenmill_amd import SamplingParams
+    eng = make_engine(model_dirs["A"], dtype_name)
+    prompts = [random_ids(n, 256, 20 + i) for i, n in enumerate((5, 17, 33))]
+    outs = eng.generate(prompts, SamplingParams(max_tokens=16, ignore_eos=True))
+    assert [len(o) for o in outs] == [16, 16, 16]
+    flips = sum(verify(plains["A"], p, o, DTYPES[dtype_name]) for p, o in zip(prompts, outs))
+    assert flips == 0 or dtype_name == "bfloat16"
+    assert not eng.scheduler.running and eng.cache.num_free_pages == eng.cache.num_pages
+    assert eng.stats["prefill_steps"] == 1 and eng.stats["decode_steps"] == 15
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_sampled_generation_chunked_and_mixed(model_dirs, plains, dtype_name):
+    """BASELINE configuration B: page size 8, prefill in portions of 12 mixed with decodes,
+    temperature 0.8 with a fixed seed, prompts of 1 / 9 / 24 / 40 ids, 20 tokens."""
+    from tokenmill_amd import SamplingParams
+    eng = make_engine(model_dirs["B"], dtype_name, block_size=8, enable_chunked_prefill=True,
+                      max_num_batched_tokens=12)
+    prompts = [random_ids(n, 384, 30 + i) for i, n in enumerate((1, 9, 24, 40))]
+    params = [SamplingParams(max_tokens=20, temperature=0.8, seed=100 + i, ignore_eos=True) for i in range(4)]
+    outs = eng.generate(prompts, params)
+    assert [len(o) for o in outs] == [20] * 4
+    for i, (p, o) in enumerate(zip(prompts, outs)):
+        verify(plains["B"], p, o, DTYPES[dtype_name], params[i], seed=100 + i)
+    assert len({tuple(o) for o in outs}) == 4
+    assert eng.cache.num_free_pages == eng.cache.num_pages
+    # the same request alone gives the same tokens: a request's draws do not depend on its batch-mates
+    alone = make_engine(model_dirs["B"], dtype_name, block_size=8).generate([prompts[2]], params[2])[0]
+    if dtype_name == "float32":
+        assert alone == outs[2]
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+@pytest.mark.parametrize("chunked", [False, True])
+def test_same_tokens_under_every_cutting_and_a_starved_pool(model_dirs, plains, dtype_name, chunked):
+    """16 prompts at once (reference tests/test_engine_greedy.py:25-88): small pages, small budgets,
+    and so few pages that requests are preempted and recomputed."""
+    from tokenmill_amd import SamplingParams
+    lengths = [1, 2, 3, 4, 5, 7, 8, 9, 13, 16, 17, 31, 40, 64, 3, 11]
+    prompts = [random_ids(n, 307, 50 + i) for i, n in enumerate(lengths)]
+    sp = SamplingParams(max_tokens=24, ignore_eos=True)
+    dt = DTYPES[dtype_name]
+    roomy = make_engine(model_dirs["C"], dtype_name, block_size=16, enable_chunked_prefill=chunked,
+                        max_num_batched_tokens=16 if chunked else 40)
+    base = roomy.generate(prompts, sp)
+    for p, o in zip(prompts, base):
+        verify(plains["C"], p, o, dt)
+    starved = make_engine(model_dirs["C"], dtype_name, block_size=4, kv_cache_mb=None, num_blocks=40,
+                          enable_chunked_prefill=chunked, max_num_batched_tokens=12 if chunked else 512)
+    outs = starved.generate(prompts, sp)
+    assert starved.scheduler.num_preemptions > 0
+    assert starved.cache.num_free_pages == starved.cache.num_pages and not starved.scheduler.running
+    starved.cache.check_invariants()
+    for p, o in zip(prompts, outs):
+        assert len(o) == 24
+        verify(plains["C"], p, o, dt)
+    if dtype_name == "float32":
+        assert outs == base
+
+
+def test_stop_rules_abort_and_rejections(model_dirs):
+    from tokenmill_amd import RequestRejected, SamplingParams
+    eng = make_engine(model_dirs["A"], "float32", max_model_len=40)
+    prompt = random_ids(10, 256, 70)
+    free_run = eng.generate([prompt], SamplingParams(max_tokens=12, ignore_eos=True))[0]
+    # max_model_len stops generation with "length" (reference tests/test_engine_greedy.py:203-208)
+    s = eng.add_request("long", random_ids(35, 256, 71), SamplingParams(max_tokens=100, ignore_eos=True))
+    while eng.has_unfinished():
+        eng.step()
+    assert s.finish_reason == "length" and s.length == 40
+    # an end-of-sequence token stops with "stop" and stays in the output
+    eng.eos_ids = {free_run[4]}
+    stopped = eng.generate([prompt], SamplingParams(max_tokens=12))[0]
+    first = free_run.index(free_run[4])
+    assert stopped == free_run[:first + 1]
+    assert eng.generate([prompt], SamplingParams(max_tokens=12, ignore_eos=True))[0] == free_run
+    # abort mid-run gives every page back (reference tests/test_engine_greedy.py:174-184)
+    eng.add_request("x", prompt, SamplingParams(max_tokens=50, ignore_eos=True))
+    eng.add_request("y", random_ids(20, 256, 72), SamplingParams(max_tokens=50, ignore_eos=True))
+    for _ in range(3):
+        eng.step()
+    out = eng.abort_request("x")
+    assert out.finished and out.finish_reason == "abort"
+    eng.abort_request("y")
+    assert not eng.has_unfinished() and eng.cache.num_free_pages == eng.cache.num_pages
+    assert eng.abort_request("nobody") is None
+    for bad in ([], list(range(40))):
+        with pytest.raises(RequestRejected):
+            eng.add_request("bad", bad, SamplingParams())
+    with pytest.raises(RequestRejected):
+        eng.add_request("vocab", [0, 256], SamplingParams())
+    eng.add_request("dup", prompt, SamplingParams(max_tokens=1))
+    with pytest.raises(RequestRejected):
+        eng.add_request("dup", prompt, SamplingParams(max_tokens=1))
+    # a prompt that can never fit the pool is finished with an error, not left waiting
+    tiny_pool = make_engine(model_dirs["A"], "float32", kv_cache_mb=None, num_blocks=2, max_model_len=200)
+    tiny_pool.add_request("big", random_ids(60, 256, 73), SamplingParams(max_tokens=4))
+    outs = tiny_pool.step()
+    assert outs[0].finished and outs[0].error == "prompt does not fit in the KV cache"
+
+
+def test_long_decoding_and_the_first_tokens_of_a_sequence(model_dirs, plains):
+    """A 2-token prompt decoded for 230 tokens across many pages; and 1-token prompts."""
+    from tokenmill_amd import SamplingParams
+    for dtype_name in ("float32", "bfloat16"):
+        eng = make_engine(model_dirs["B"], dtype_name, block_size=8)
+        prompts = [random_ids(2, 384, 80), [5], [0]]
+        outs = eng.generate(prompts, [SamplingParams(max_tokens=230, ignore_eos=True),
+                                      SamplingParams(max_tokens=3, ignore_eos=True),
+                                      SamplingParams(max_tokens=3, ignore_eos=True)])
+        assert len(outs[0]) == 230
+        for p, o in zip(prompts, outs):
+            verify(plains["B"], p, o, DTYPES[dtype_name])
+
+
+def test_command_line(model_dirs, plains):
+    r = subprocess.run([sys.executable, "-m", "tokenmill_amd.generate", "--model", str(model_dirs["A"]), "--dtype",
+                        "float32", "--prompt-ids", "1,2,3;4,5", "--max-tokens", "6", "--ignore-eos",
+                        "--kv-cache-mb", "4", "--max-model-len", "64", "--block-size", "8"],
+                       capture_output=True, text=True, cwd=ROOT, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = [json.loads(ln) for ln in r.stdout.splitlines() if ln.startswith("{")]
+    assert [ln["prompt_tokens"] for ln in lines] == [3, 2]
+    verify(plains["A"], [1, 2, 3], lines[0]["output_ids"], torch.float32)
+    verify(plains["A"], [4, 5], lines[1]["output_ids"], torch.float32)

@@ -1,0 +1,315 @@
+"""Each HIP kernel alone against a plain torch reference on the CPU, at sizes other than the tiny
+models': widths and vocabularies that are no powers of two, head sizes in steps of 16, odd numbers
+of heads and groups, row counts that do not fill a tile."""
+from __future__ import annotations
+
+import math
+
+import pytest
+import torch
+
+from plain import qwen2_plain as P
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+DTS = [torch.float32, torch.bfloat16]
+
+
+def tol(dt):
+    return dict(rtol=1e-5, atol=1e-5) if dt == torch.float32 else dict(rtol=1.6e-2, atol=1e-2)
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from tokenmill_amd.hip import ops as o
+    from tokenmill_amd.hip.library import library
+    library()
+    return o
+
+
+def q(x, dt):
+    """values representable in dt, as float32"""
+    return x.to(dt).float()
+
+
+@pytest.mark.parametrize("dt", DTS)
+def test_embed_gather(ops, dt):
+    torch.manual_seed(0)
+    table = q(torch.randn(307, 120), dt)
+    ids = torch.randint(0, 307, (33,), dtype=torch.int32)
+    out = torch.empty(33, 120, dtype=torch.float32, device=DEV)
+    ops.embed_gather(table.to(dt).to(DEV), ids.to(DEV), out)
+    assert torch.equal(out.cpu(), table[ids.long()])
+
+
+@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("hidden", [64, 120, 896, 5000])
+def test_add_rmsnorm(ops, dt, hidden):
+    torch.manual_seed(1)
+    T, eps = 7, 1e-5
+    resid, delta, w = torch.randn(T, hidden) * 3, q(torch.randn(T, hidden), dt), q(torch.rand(hidden) + 0.5, dt)
+    want_resid = resid + delta
+    want = P.rms_norm(want_resid, w, eps, dt)
+    r = resid.to(DEV)
+    out = torch.empty(T, hidden, dtype=dt, device=DEV)
+    ops.add_rmsnorm(r, delta.to(dt).to(DEV), w.to(dt).to(DEV), eps, out)
+    torch.testing.assert_close(r.cpu(), want_resid, rtol=0, atol=0)            # the 32-bit sum is exact
+    torch.testing.assert_close(out.float().cpu(), want, **tol(dt))
+    # no delta; and rows picked (the residual is then left alone)
+    r2 = resid.to(DEV)
+    ops.add_rmsnorm(r2, None, w.to(dt).to(DEV), eps, out)
+    torch.testing.assert_close(out.float().cpu(), P.rms_norm(resid, w, eps, dt), **tol(dt))
+    rows = torch.tensor([5, 0, 5, 2], dtype=torch.int32)
+    out_r = torch.empty(4, hidden, dtype=dt, device=DEV)
+    ops.add_rmsnorm(r2, delta.to(dt).to(DEV), w.to(dt).to(DEV), eps, out_r, rows.to(DEV))
+    torch.testing.assert_close(out_r.float().cpu(), want[rows.long()], **tol(dt))
+    assert torch.equal(r2.cpu(), resid)
+    if dt == torch.bfloat16:                                                    # a weight stored in 32-bit stays so
+        w32 = torch.rand(hidden) + 0.5
+        ops.add_rmsnorm(resid.to(DEV), None, w32.to(DEV), eps, out)
+        normed = q(resid * torch.rsqrt((resid * resid).mean(-1, keepdim=True) + eps), dt)
+        torch.testing.assert_close(out.float().cpu(), q(w32 * normed, dt), **tol(dt))
+
+
+@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("H,KVH,D,rot", [(5, 1, 16, 16), (6, 3, 48, 48), (4, 2, 128, 64), (3, 3, 80, 80)])
+def test_rope_and_cache_write(ops, dt, H, KVH, D, rot):
+    torch.manual_seed(2)
+    T, max_pos, pages, page = 9, 700, 12, 4
+    qkv = q(torch.randn(T, (H + 2 * KVH) * D), dt)
+    positions = torch.tensor([0, 1, 5, 17, 300, 699, 2, 3, 4], dtype=torch.int32)   # absolute, not contiguous
+    slots = torch.randperm(pages * page)[:T].to(torch.int32)
+    slots[3] = -1                                                               # a padding row: not stored
+    theta = 1e6
+    inv = 1.0 / (theta ** (torch.arange(0, rot, 2, dtype=torch.int64).float() / rot))
+    fr = torch.outer(torch.arange(max_pos).float(), inv)
+    cos_h, sin_h = fr.cos(), fr.sin()
+    cos, sin = P.rope_tables(max_pos, rot, theta)
+    qq = qkv[:, :H * D].view(T, H, D).clone()
+    kk = qkv[:, H * D:(H + KVH) * D].view(T, KVH, D).clone()
+    vv = qkv[:, (H + KVH) * D:].view(T, KVH, D)
+    qq[..., :rot] = P.apply_rope(qq[..., :rot], cos, sin, positions.long(), dt)
+    kk[..., :rot] = P.apply_rope(kk[..., :rot], cos, sin, positions.long(), dt)
+    dq = qkv.to(dt).to(DEV)
+    kp = torch.full((pages, page, KVH, D), 7.0, dtype=dt, device=DEV)
+    vp = torch.full((pages, page, KVH, D), 7.0, dtype=dt, device=DEV)
+    ops.rope_kv_write(dq, H, KVH, D, cos_h.to(DEV), sin_h.to(DEV), positions.to(DEV), slots.to(DEV), kp, vp)
+    got = dq.float().cpu()
+    torch.testing.assert_close(got[:, :H * D].view(T, H, D), qq, **tol(dt))
+    torch.testing.assert_close(got[:, H * D:(H + KVH) * D].view(T, KVH, D), kk, **tol(dt))
+    assert torch.equal(got[:, (H + KVH) * D:].view(T, KVH, D), vv)              # v is not rotated
+    kflat, vflat = kp.float().cpu().view(-1, KVH, D), vp.float().cpu().view(-1, KVH, D)
+    written = torch.zeros(pages * page, dtype=torch.bool)
+    for t in range(T):
+        if slots[t] >= 0:
+            written[slots[t]] = True
+            assert torch.equal(kflat[slots[t]], got[t, H * D:(H + KVH) * D].view(KVH, D))
+            assert torch.equal(vflat[slots[t]], vv[t])
+    assert (kflat[~written] == 7.0).all() and (vflat[~written] == 7.0).all()   # nothing else is touched
+
+
+@pytest.mark.parametrize("dt", DTS)
+def test_silu_mul(ops, dt):
+    torch.manual_seed(3)
+    gu = q(torch.randn(5, 2 * 203) * 4, dt)
+    out = torch.empty(5, 203, dtype=dt, device=DEV)
+    ops.silu_mul(gu.to(dt).to(DEV), out)
+    torch.testing.assert_close(out.float().cpu(), P.silu_mul(gu[:, :203], gu[:, 203:], dt), **tol(dt))
+
+
+@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("M,N,K", [(1, 307, 120), (7, 64, 64), (65, 130, 17), (130, 96, 300), (3, 1152, 896)])
+def test_gemm_tiled(ops, dt, M, N, K):
+    torch.manual_seed(4)
+    a, w, b = q(torch.randn(M, K), dt), q(torch.randn(N, K) * 0.1, dt), q(torch.randn(N), dt)
+    want = a @ w.t() + b
+    out = torch.empty(M, N, dtype=dt, device=DEV)
+    ops.gemm_nt_tiled(a.to(dt).to(DEV), w.to(dt).to(DEV), b.to(dt).to(DEV), out)
+    torch.testing.assert_close(out.float().cpu(), q(want, dt), **tol(dt))
+    out32 = torch.empty(M, N, dtype=torch.float32, device=DEV)                  # 32-bit result, no bias
+    ops.gemm_nt_tiled(a.to(dt).to(DEV), w.to(dt).to(DEV), None, out32)
+    torch.testing.assert_close(out32.cpu(), a @ w.t(), rtol=1e-5, atol=2e-5)
+    # a row-strided input (the q part of a qkv row) and a row's result that does not depend on the other rows
+    wide = torch.zeros(M, K + 13, dtype=dt, device=DEV)
+    wide[:, :K] = a.to(dt).to(DEV)
+    out_s = torch.empty(M, N, dtype=torch.float32, device=DEV)
+    ops.gemm_nt_tiled(wide[:, :K], w.to(dt).to(DEV), None, out_s)
+    assert torch.equal(out_s, out32)
+    one = torch.empty(1, N, dtype=torch.float32, device=DEV)
+    ops.gemm_nt_tiled(a[M - 1:].to(dt).to(DEV), w.to(dt).to(DEV), None, one)
+    assert torch.equal(one[0], out32[M - 1])
+
+
+def paged_case(dt, lens, q_lens, H, KVH, D, page, seed, spike=None):
+    """Random requests laid out in shuffled pages. Returns device operands and the CPU truth."""
+    g = torch.Generator().manual_seed(seed)
+    S = len(lens)
+    n_pages = sum(-(-n // page) for n in lens) + 3
+    perm = torch.randperm(n_pages, generator=g).tolist()
+    W = max(-(-n // page) for n in lens)
+    tables = torch.zeros(S, W, dtype=torch.int32)
+    kp = torch.randn(n_pages, page, KVH, D, generator=g).to(dt)        # stale values everywhere
+    vp = torch.randn(n_pages, page, KVH, D, generator=g).to(dt)
+    qs, ks, vs, seq_of, pos = [], [], [], [], []
+    used = 0
+    for s, (n, ql) in enumerate(zip(lens, q_lens)):
+        k = torch.randn(n, KVH, D, generator=g).to(dt)
+        v = torch.randn(n, KVH, D, generator=g).to(dt)
+        qq = torch.randn(n, H, D, generator=g).to(dt)
+        if spike and spike[0] == s:                                  # one far key that must dominate the last query
+            _, far = spike
+            k[far] *= 0.0
+            k[far, :, 0] = 12.0
+            qq[n - 1] *= 0.0
+            qq[n - 1, :, 0] = 12.0
+        for i in range(-(-n // page)):
+            tables[s, i] = perm[used]
+            lo, hi = i * page, min(n, (i + 1) * page)
+            kp[perm[used], :hi - lo] = k[lo:hi]
+            vp[perm[used], :hi - lo] = v[lo:hi]
+            used += 1
+        qs.append(qq)
+        ks.append(k)
+        vs.append(v)
+        seq_of += [s] * ql
+        pos += list(range(n - ql, n))
+    q_rows = torch.cat([qq[n - ql:] for qq, n, ql in zip(qs, lens, q_lens)])   # [T, H, D]
+    return dict(q=q_rows, k=ks, v=vs, qfull=qs, tables=tables, kp=kp, vp=vp,
+                seq_of=torch.tensor(seq_of, dtype=torch.int32), pos=torch.tensor(pos, dtype=torch.int32))
+
+
+def paged_truth(case, lens, q_lens, scale, dt, window=None):
+    outs = []
+    for qq, k, v, n, ql in zip(case["qfull"], case["k"], case["v"], lens, q_lens):
+        full = P.causal_attention(qq.float(), k.float(), v.float(), scale, dt, window)
+        outs.append(full[n - ql:])
+    return torch.cat(outs)
+
+
+@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("H,KVH,D,page", [(4, 2, 16, 16), (6, 1, 32, 8), (14, 2, 64, 16), (5, 5, 48, 4), (3, 1, 128, 16),
+                                           (8, 2, 80, 16)])
+def test_paged_attention_generic(ops, dt, H, KVH, D, page):
+    lens = [1, 37, 130, 64, 5, 200]
+    q_lens = [1, 37, 2, 1, 3, 1]                 # whole prompts, portions that start mid-page, single tokens
+    case = paged_case(dt, lens, q_lens, H, KVH, D, page, seed=5, spike=(5, 3))
+    scale = D ** -0.5
+    T = case["q"].shape[0]
+    out = torch.empty(T, H * D, dtype=dt, device=DEV)
+    # q sits in the first H*D columns of a wider row, as in a fused qkv product
+    wide = torch.zeros(T, (H + 2 * KVH) * D, dtype=dt, device=DEV)
+    wide[:, :H * D] = case["q"].reshape(T, H * D).to(DEV)
+    ops.attn_paged_generic(wide, out, case["kp"].to(DEV), case["vp"].to(DEV), case["tables"].to(DEV),
+                           case["seq_of"].to(DEV), case["pos"].to(DEV), H, KVH, D, scale, 0)
+    want = paged_truth(case, lens, q_lens, scale, dt).reshape(T, H * D)
+    torch.testing.assert_close(out.float().cpu(), want, **tol(dt))
+    # the spiked far key carries the last query's output: it equals that key's value almost exactly
+    v_far = case["v"][5][3].float()
+    got_last = out.float().cpu()[-1].view(H, D)
+    for h in range(H):
+        torch.testing.assert_close(got_last[h], v_far[h // (H // KVH)], rtol=0, atol=5e-2)
+
+
+@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("window", [1, 7, 16, 50])
+def test_paged_attention_generic_window(ops, dt, window):
+    H, KVH, D, page = 6, 2, 32, 8
+    lens, q_lens = [60, 9, 33], [60, 1, 5]
+    case = paged_case(dt, lens, q_lens, H, KVH, D, page, seed=6)
+    # poison every page wholly behind the window of the queries run here: it must never be read
+    for s, (n, ql) in enumerate(zip(lens, q_lens)):
+        first_query = n - ql
+        for i in range(max(0, first_query - window + 1) // page):
+            case["kp"][case["tables"][s, i]] = float("nan")
+            case["vp"][case["tables"][s, i]] = float("nan")
+    T = case["q"].shape[0]
+    out = torch.empty(T, H * D, dtype=dt, device=DEV)
+    ops.attn_paged_generic(case["q"].reshape(T, H * D).to(DEV), out, case["kp"].to(DEV), case["vp"].to(DEV),
+                           case["tables"].to(DEV), case["seq_of"].to(DEV), case["pos"].to(DEV), H, KVH, D,
+                           D ** -0.5, window)
+    want = paged_truth(case, lens, q_lens, D ** -0.5, dt, window).reshape(T, H * D)
+    torch.testing.assert_close(out.float().cpu(), want, **tol(dt))
+
+
+def test_kernels_refuse_what_they_cannot_run(ops):
+    from tokenmill_amd.hip.ops import KernelArgumentError
+    x = torch.zeros(4, 8, device=DEV)
+    with pytest.raises(KernelArgumentError):
+        ops.silu_mul(x.cpu(), torch.zeros(4, 4))                      # no CPU path
+    with pytest.raises(KernelArgumentError):
+        ops.silu_mul(x.double(), torch.zeros(4, 4, device=DEV).double())
+    with pytest.raises(KernelArgumentError):
+        ops.attn_paged_generic(torch.zeros(1, 6, device=DEV), torch.zeros(1, 6, device=DEV),
+                               torch.zeros(1, 4, 1, 6, device=DEV), torch.zeros(1, 4, 1, 6, device=DEV),
+                               torch.zeros(1, 1, dtype=torch.int32, device=DEV),
+                               torch.zeros(1, dtype=torch.int32, device=DEV),
+                               torch.zeros(1, dtype=torch.int32, device=DEV), 1, 1, 6, 1.0)   # head size 6
+    with pytest.raises(KernelArgumentError):
+        ops.gemm_nt_tiled(torch.zeros(2, 8, device=DEV), torch.zeros(4, 9, device=DEV), None,
+                          torch.zeros(2, 4, device=DEV))
+
+
+# ----------------------------------------------------------------------------------------------- sampling
+
+def test_argmax_rows(ops):
+    torch.manual_seed(7)
+    logits = torch.randn(9, 151936 // 8 + 5)
+    logits[3, 100] = logits[3, 7000] = 50.0                           # a tie: the first maximum wins
+    out = torch.empty(9, dtype=torch.int32, device=DEV)
+    ops.argmax_rows(logits.to(DEV), out)
+    assert out.cpu().tolist() == logits.argmax(-1).tolist() and out[3].item() == 100
+    two = torch.tensor([[0.1, 3.0, 2.0], [5.0, -1.0, 4.9]])          # reference tests/test_sampling.py:11-13
+    out = torch.empty(2, dtype=torch.int32, device=DEV)
+    ops.argmax_rows(two.to(DEV), out)
+    assert out.cpu().tolist() == [1, 0]
+
+
+def sample(ops, logits, temps, ks, ps, us):
+    R = logits.shape[0]
+    out = torch.empty(R, dtype=torch.int32, device=DEV)
+    f = lambda x: torch.tensor(x, dtype=torch.float32, device=DEV)    # noqa: E731
+    ops.sample_rows(logits.to(DEV), f(temps), torch.tensor(ks, dtype=torch.int32, device=DEV), f(ps), f(us), out)
+    return out.cpu().tolist()
+
+
+def test_sample_rows_against_the_plain_sampler(ops):
+    torch.manual_seed(8)
+    V = 1000
+    logits = torch.randn(64, V) * 2
+    cases = [(0.8, -1, 1.0), (1.0, 20, 1.0), (0.7, -1, 0.9), (1.3, 50, 0.8), (0.0, -1, 1.0), (0.9, 1, 1.0),
+             (1.0, 5000, 0.999), (0.5, 3, 0.5)]
+    temps, ks, ps, us, want, margins = [], [], [], [], [], []
+    for r in range(64):
+        t, k, p = cases[r % len(cases)]
+        temps.append(t), ks.append(k), ps.append(p)
+        u = P.uniform_from_counter(99, r)
+        us.append(u)
+        # the plain sampler draws from (seed, index); index r here
+        tok, margin = P.sample_token(logits[r], t, k, p, 99, r)
+        want.append(tok), margins.append(margin)
+    got = sample(ops, logits, temps, ks, ps, us)
+    for r in range(64):
+        assert got[r] == want[r] or margins[r] < 1e-4, f"row {r} {cases[r % len(cases)]}: {got[r]} != {want[r]}"
+    assert sum(g == w for g, w in zip(got, want)) >= 62
+
+
+def test_sample_rows_filters_on_the_references_vectors(ops):
+    """reference tests/test_sampling.py:16-31: what top-k and top-p keep."""
+    draws = [i / 64 + 1 / 128 for i in range(64)]
+    row = torch.tensor([1.0, 4.0, 3.0, 2.0]).repeat(64, 1)
+    got = set(sample(ops, row, [1.0] * 64, [2] * 64, [1.0] * 64, draws))
+    assert got == {1, 2}
+    row = torch.tensor([0.5, 0.3, 0.15, 0.05]).log().repeat(64, 1)
+    assert set(sample(ops, row, [1.0] * 64, [-1] * 64, [0.7] * 64, draws)) == {0, 1}
+    row = torch.tensor([10.0, 0.0]).repeat(64, 1)
+    assert set(sample(ops, row, [1.0] * 64, [-1] * 64, [1e-6] * 64, draws)) == {0}
+    # temperature row = softmax(logits / t): frequencies over a fine grid of u
+    n = 4096
+    row = torch.tensor([2.0, 1.0, 0.0]).repeat(n, 1)
+    grid = [(i + 0.5) / n for i in range(n)]
+    for t in (1.0, 0.3):
+        got = sample(ops, row, [t] * n, [-1] * n, [1.0] * n, grid)
+        want = torch.softmax(torch.tensor([2.0, 1.0, 0.0]) / t, -1)
+        for tok in range(3):
+            assert abs(got.count(tok) / n - want[tok].item()) < 2e-3

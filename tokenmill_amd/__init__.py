@@ -6,3 +6,16 @@ manager, one step function, a scheduler, a sampler and hand-written HIP kernels.
 """
 
 __version__ = "0.1.0"
+
+
+def __getattr__(name):          # the public names, imported on first use (torch loads slowly)
+    if name in ("LLMEngine", "RequestRejected"):
+        from tokenmill_amd.engine import engine
+        return getattr(engine, name)
+    if name == "EngineConfig":
+        from tokenmill_amd.config.engine_config import EngineConfig
+        return EngineConfig
+    if name == "SamplingParams":
+        from tokenmill_amd.sampling.sampler import SamplingParams
+        return SamplingParams
+    raise AttributeError(name)

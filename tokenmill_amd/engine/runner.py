@@ -45,6 +45,7 @@ class ModelRunner:
         self._pinned = torch.empty(1 << 14, dtype=torch.int32, pin_memory=True)
         self._copied = torch.cuda.Event()
         self._copy_pending = False
+        self.graphs = None                        # DecodeGraphs when the engine runs with --hip-graphs
 
     # ------------------------------------------------------------------------------------------------
 

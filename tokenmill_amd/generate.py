@@ -1,0 +1,63 @@
+"""Offline generation from the command line, in the manner of the reference's one CLI entry point
+(``python -m infer.serve`` with the engine flags, reference src/infer/serve.py:1-44): the same
+engine flags, plus where the prompts come from and how to sample.
+
+    python -m tokenmill_amd.generate --model DIR --prompt-ids "1,2,3;4,5" --max-tokens 16
+    python -m tokenmill_amd.generate --model DIR --prompt-lens 5,17,33 --prompt-seed 0 --temperature 0.8
+
+Token ids in, token ids out (one JSON line per prompt).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import logging
+import sys
+
+from tokenmill_amd.config.engine_config import add_engine_args, engine_config_from_args
+
+
+def main(argv=None) -> int:
+    parser = argparse.ArgumentParser(description="tokenmill_amd: continuous-batching generation on one MI355X")
+    add_engine_args(parser)
+    parser.add_argument("--prompt-ids", default=None, help='prompts as token ids: "1,2,3;4,5"')
+    parser.add_argument("--prompt-lens", default=None, help="lengths of uniform-random prompts: 5,17,33")
+    parser.add_argument("--prompt-seed", type=int, default=0)
+    parser.add_argument("--max-tokens", type=int, default=256)
+    parser.add_argument("--temperature", type=float, default=0.0)
+    parser.add_argument("--top-k", type=int, default=-1)
+    parser.add_argument("--top-p", type=float, default=1.0)
+    parser.add_argument("--sample-seed", type=int, default=None)
+    parser.add_argument("--ignore-eos", action="store_true")
+    parser.add_argument("--log-level", default="warning")
+    args = parser.parse_args(argv)
+    logging.basicConfig(level=args.log_level.upper(), format="%(asctime)s %(levelname)s %(name)s: %(message)s")
+    if args.debug_steps:
+        logging.getLogger("tokenmill_amd.engine").setLevel(logging.INFO)
+    if not args.model:
+        parser.error("--model DIR is required")
+    if (args.prompt_ids is None) == (args.prompt_lens is None):
+        parser.error("give exactly one of --prompt-ids and --prompt-lens")
+
+    import torch
+
+    from tokenmill_amd.engine.engine import LLMEngine
+    from tokenmill_amd.sampling.sampler import SamplingParams
+
+    engine = LLMEngine(engine_config_from_args(args))
+    if args.prompt_ids is not None:
+        prompts = [[int(t) for t in part.split(",") if t.strip()] for part in args.prompt_ids.split(";") if part.strip()]
+    else:
+        g = torch.Generator().manual_seed(args.prompt_seed)
+        vocab = engine.runner.vocab
+        prompts = [torch.randint(0, vocab, (int(n),), generator=g).tolist() for n in args.prompt_lens.split(",")]
+    params = SamplingParams(max_tokens=args.max_tokens, temperature=args.temperature, top_k=args.top_k,
+                            top_p=args.top_p, seed=args.sample_seed, ignore_eos=args.ignore_eos)
+    outputs = engine.generate(prompts, params)
+    for i, (p, o) in enumerate(zip(prompts, outputs)):
+        print(json.dumps({"prompt": i, "prompt_tokens": len(p), "output_ids": o}))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
