@@ -1,0 +1,169 @@
+"""Headline benchmark: decode tokens/s and prefill tokens/s at the Qwen2.5-0.5B shape, random
+weights, synthetic token ids, on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype bfloat16|float32] [--layers L]
+
+A "step" is one decode step of the engine (scheduling, metadata upload, the forward pass and greedy
+sampling) with a batch of 8 requests, each holding a 2,048-token prompt. One JSON line is printed.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import statistics
+import sys
+import time
+from pathlib import Path
+
+sys.path.insert(0, str(Path(__file__).resolve().parent))
+
+# BASELINE configuration 3: the Qwen2.5-0.5B shape
+SHAPE = {"architectures": ["Qwen2ForCausalLM"], "num_hidden_layers": 24, "hidden_size": 896,
+         "num_attention_heads": 14, "num_key_value_heads": 2, "intermediate_size": 4864, "vocab_size": 151936,
+         "rope_theta": 1e6, "rms_norm_eps": 1e-6, "tie_word_embeddings": True, "max_position_embeddings": 32768,
+         "use_sliding_window": False}
+MAX_MODEL_LEN = 4096
+PROMPT_LEN = 2048
+BLOCK_SIZE = 16
+
+# MI355X published peaks
+PEAK_HBM_GBS = 8000.0
+PEAK_FLOPS = {"bfloat16": 2.5e15, "float32": 157.3e12}
+
+
+def matmul_params(c: dict) -> int:
+    """Parameters of the matrices one token passes through in the layers (no embedding, no head)."""
+    h, d = c["hidden_size"], c["hidden_size"] // c["num_attention_heads"]
+    q, kv, i = c["num_attention_heads"] * d, c["num_key_value_heads"] * d, c["intermediate_size"]
+    return c["num_hidden_layers"] * (h * (q + 2 * kv) + q * h + 3 * h * i)
+
+
+def decode_bytes(c: dict, batch: int, context: int, elem: int) -> float:
+    """Bytes a decode step has to read: every weight it uses once, and the cache of the live requests."""
+    h, d = c["hidden_size"], c["hidden_size"] // c["num_attention_heads"]
+    q, kv = c["num_attention_heads"] * d, c["num_key_value_heads"] * d
+    weights = matmul_params(c) + c["vocab_size"] * h + c["num_hidden_layers"] * (q + 2 * kv + 2 * h) + h
+    cache = 2 * c["num_hidden_layers"] * kv * context * batch
+    return float((weights + cache) * elem)
+
+
+def prefill_flops(c: dict, T: int) -> float:
+    """Projections 2 * parameters * T, causal attention 2 * T^2 * D * H per layer, one row of logits."""
+    d = c["hidden_size"] // c["num_attention_heads"]
+    attn = c["num_hidden_layers"] * 2.0 * T * T * d * c["num_attention_heads"]
+    return 2.0 * matmul_params(c) * T + attn + 2.0 * c["hidden_size"] * c["vocab_size"]
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (named in config)")
+    ap.add_argument("--no-graphs", action="store_true", help="launch decode steps kernel by kernel")
+    ap.add_argument("--skip-points", action="store_true", help="only the headline batch and the prefill")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+
+    import torch
+
+    from tokenmill_amd import EngineConfig, LLMEngine, SamplingParams
+    from tokenmill_amd.engine.loading import load_random_model
+
+    torch.cuda.set_device(0)
+    device = torch.device("cuda:0")
+    dtype = {"bfloat16": torch.bfloat16, "float32": torch.float32}[args.dtype]
+    shape = dict(SHAPE)
+    layers_full = shape["num_hidden_layers"]
+    if args.layers:
+        shape["num_hidden_layers"] = args.layers
+    model = load_random_model(shape, seed=0, dtype=dtype, device=device, max_positions=MAX_MODEL_LEN)
+    elem = 2 if dtype == torch.bfloat16 else 4
+    gen = torch.Generator().manual_seed(0)
+
+    def prompts(n):
+        return [torch.randint(0, shape["vocab_size"], (PROMPT_LEN,), generator=gen).tolist() for _ in range(n)]
+
+    def engine_for(batch):
+        pages = batch * (-(-(PROMPT_LEN + args.steps + args.warmup + 64) // BLOCK_SIZE)) + 8
+        cfg = EngineConfig(dtype=args.dtype, block_size=BLOCK_SIZE, num_blocks=pages, max_model_len=MAX_MODEL_LEN,
+                           max_num_seqs=max(batch, 1), max_num_batched_tokens=max(PROMPT_LEN, batch),
+                           watermark=0.0, hip_graphs=not args.no_graphs)
+        return LLMEngine(cfg, model=model)
+
+    def time_decode(batch, steps, warmup):
+        eng = engine_for(batch)
+        sp = SamplingParams(max_tokens=steps + warmup + 8, ignore_eos=True)
+        for i, p in enumerate(prompts(batch)):
+            eng.add_request(f"d{i}", p, sp)
+        while eng.scheduler.waiting or any(s.num_new_tokens > 1 for s in eng.scheduler.running):
+            eng.step()                                   # prefills (one prompt a step: budget = 2,048 tokens)
+        for _ in range(warmup):
+            eng.step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            outs = eng.step()
+            assert len(outs) == batch
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        context = PROMPT_LEN + warmup + steps // 2
+        for s in list(eng.seqs):
+            eng.abort_request(s)
+        del eng
+        return dt / steps, context
+
+    def time_prefill(reps=5):
+        eng = engine_for(1)
+        times = []
+        for r in range(reps + 1):
+            p = prompts(1)[0]
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            eng.add_request(f"p{r}", p, SamplingParams(max_tokens=1, ignore_eos=True))
+            outs = eng.step()                            # the whole prompt in one step, first token sampled
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+            assert outs and outs[0].finished
+        return statistics.median(times[1:])              # the first run warms up
+
+    step_s, context = time_decode(args.batch, args.steps, args.warmup)
+    value = args.batch / step_s
+    prefill_s = time_prefill()
+    points = {}
+    if not args.skip_points:
+        for b in (1, 64):
+            s, _ = time_decode(b, max(16, args.steps // 2), max(4, args.warmup // 2))
+            points[f"decode_b{b}"] = round(b / s, 1)
+    nbytes = decode_bytes(shape, args.batch, context, elem)
+    achieved = nbytes / step_s / 1e9
+    flops = prefill_flops(shape, PROMPT_LEN)
+    line = {
+        "metric": "decode tok/s at batch 8, context 2048 (Qwen2.5-0.5B shape); prefill and batch 1/64 alongside",
+        "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if dtype == torch.bfloat16 else "fp32", "data": "synthetic token ids, random weights",
+        "config": {"model": "Qwen2.5-0.5B shape", "layers": shape["num_hidden_layers"], "layers_full": layers_full,
+                   "hidden": shape["hidden_size"], "q_heads": shape["num_attention_heads"],
+                   "kv_heads": shape["num_key_value_heads"],
+                   "head_dim": shape["hidden_size"] // shape["num_attention_heads"],
+                   "intermediate": shape["intermediate_size"], "vocab": shape["vocab_size"], "tied": True,
+                   "global_batch": args.batch, "seq_len": PROMPT_LEN, "context": context,
+                   "max_model_len": MAX_MODEL_LEN, "block_size": BLOCK_SIZE, "parallelism": "single GPU",
+                   "hip_graphs": not args.no_graphs},
+        "prefill": {"value": round(PROMPT_LEN / prefill_s, 1), "tokens": PROMPT_LEN, "ms": round(prefill_s * 1e3, 3),
+                    "frac": round(flops / prefill_s / PEAK_FLOPS[args.dtype], 4)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(achieved / PEAK_HBM_GBS, 4)},
+        "points": points,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

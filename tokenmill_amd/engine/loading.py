@@ -32,3 +32,30 @@ def load_model(model_dir: str | Path, dtype: torch.dtype, device: torch.device, 
     tensors = read_checkpoint(model_dir, model.tensor_specs(), dtype, device, model.ignorable)
     model.load(tensors, dtype, device)
     return model
+
+
+def load_random_model(config: dict, seed: int, dtype: torch.dtype, device: torch.device,
+                      max_positions: int | None = None, std: float = 0.02, norm_std: float = 0.0):
+    """The model that ``config`` (config.json contents) names, with random weights drawn on the
+    device: the random-weights mode without the trip through a file, for large shapes."""
+    from tokenmill_amd.config.registry import architecture_name, get_architecture
+    from tokenmill_amd.weights.loader import storage_dtype
+
+    arch = get_architecture(architecture_name(config))
+    model = arch.build_model(arch.config_from_dict(config, None), max_positions)
+    g = torch.Generator(device=device).manual_seed(seed)
+    tensors = {}
+    for name, spec in sorted(model.tensor_specs().items()):
+        if spec.kind == "int":
+            t = torch.arange(int(torch.tensor(spec.shape).prod()), dtype=torch.int32, device=device).reshape(spec.shape)
+        elif spec.init == "ones":
+            t = torch.ones(spec.shape, dtype=torch.float32, device=device)
+            if norm_std:
+                t += torch.randn(spec.shape, generator=g, dtype=torch.float32, device=device) * norm_std
+        elif spec.init == "zeros":
+            t = torch.zeros(spec.shape, dtype=torch.float32, device=device)
+        else:
+            t = torch.randn(spec.shape, generator=g, dtype=torch.float32, device=device) * std
+        tensors[name] = t if spec.kind == "int" else t.to(storage_dtype(torch.bfloat16, spec.kind, dtype))
+    model.load(tensors, dtype, device)
+    return model
