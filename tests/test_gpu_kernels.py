@@ -33,6 +33,11 @@ def q(x, dt):
     return x.to(dt).float()
 
 
+def v_layout(vp):
+    """[pages, page, KVH, D] (how the tests fill it) -> the engine's V pool [pages, KVH, D, page]."""
+    return vp.permute(0, 2, 3, 1).contiguous()
+
+
 @pytest.mark.parametrize("dt", DTS)
 def test_embed_gather(ops, dt):
     torch.manual_seed(0)
@@ -93,13 +98,14 @@ def test_rope_and_cache_write(ops, dt, H, KVH, D, rot):
     kk[..., :rot] = P.apply_rope(kk[..., :rot], cos, sin, positions.long(), dt)
     dq = qkv.to(dt).to(DEV)
     kp = torch.full((pages, page, KVH, D), 7.0, dtype=dt, device=DEV)
-    vp = torch.full((pages, page, KVH, D), 7.0, dtype=dt, device=DEV)
+    vp = torch.full((pages, KVH, D, page), 7.0, dtype=dt, device=DEV)
     ops.rope_kv_write(dq, H, KVH, D, cos_h.to(DEV), sin_h.to(DEV), positions.to(DEV), slots.to(DEV), kp, vp)
     got = dq.float().cpu()
     torch.testing.assert_close(got[:, :H * D].view(T, H, D), qq, **tol(dt))
     torch.testing.assert_close(got[:, H * D:(H + KVH) * D].view(T, KVH, D), kk, **tol(dt))
     assert torch.equal(got[:, (H + KVH) * D:].view(T, KVH, D), vv)              # v is not rotated
-    kflat, vflat = kp.float().cpu().view(-1, KVH, D), vp.float().cpu().view(-1, KVH, D)
+    kflat = kp.float().cpu().view(-1, KVH, D)
+    vflat = vp.float().cpu().permute(0, 3, 1, 2).reshape(-1, KVH, D)
     written = torch.zeros(pages * page, dtype=torch.bool)
     for t in range(T):
         if slots[t] >= 0:
@@ -200,7 +206,7 @@ def test_paged_attention_generic(ops, dt, H, KVH, D, page):
     # q sits in the first H*D columns of a wider row, as in a fused qkv product
     wide = torch.zeros(T, (H + 2 * KVH) * D, dtype=dt, device=DEV)
     wide[:, :H * D] = case["q"].reshape(T, H * D).to(DEV)
-    ops.attn_paged_generic(wide, out, case["kp"].to(DEV), case["vp"].to(DEV), case["tables"].to(DEV),
+    ops.attn_paged_generic(wide, out, case["kp"].to(DEV), v_layout(case["vp"]).to(DEV), case["tables"].to(DEV),
                            case["seq_of"].to(DEV), case["pos"].to(DEV), H, KVH, D, scale, 0)
     want = paged_truth(case, lens, q_lens, scale, dt).reshape(T, H * D)
     torch.testing.assert_close(out.float().cpu(), want, **tol(dt))
@@ -225,7 +231,7 @@ def test_paged_attention_generic_window(ops, dt, window):
             case["vp"][case["tables"][s, i]] = float("nan")
     T = case["q"].shape[0]
     out = torch.empty(T, H * D, dtype=dt, device=DEV)
-    ops.attn_paged_generic(case["q"].reshape(T, H * D).to(DEV), out, case["kp"].to(DEV), case["vp"].to(DEV),
+    ops.attn_paged_generic(case["q"].reshape(T, H * D).to(DEV), out, case["kp"].to(DEV), v_layout(case["vp"]).to(DEV),
                            case["tables"].to(DEV), case["seq_of"].to(DEV), case["pos"].to(DEV), H, KVH, D,
                            D ** -0.5, window)
     want = paged_truth(case, lens, q_lens, D ** -0.5, dt, window).reshape(T, H * D)
@@ -313,3 +319,82 @@ def test_sample_rows_filters_on_the_references_vectors(ops):
         want = torch.softmax(torch.tensor([2.0, 1.0, 0.0]) / t, -1)
         for tok in range(3):
             assert abs(got.count(tok) / n - want[tok].item()) < 2e-3
+
+
+# ----------------------------------------------------------------------------------------------- MFMA kernels
+
+@pytest.mark.parametrize("M,N,K", [(1, 307, 120), (8, 1152, 896), (8, 896, 4864), (17, 1000, 64), (64, 896, 896),
+                                   (33, 16 * 2048 + 5, 72), (48, 130, 2056), (5, 16, 8)])
+def test_gemm_skinny(ops, M, N, K):
+    torch.manual_seed(9)
+    dt = torch.bfloat16
+    a, w, b = q(torch.randn(M, K), dt), q(torch.randn(N, K) * 0.1, dt), q(torch.randn(N), dt)
+    want = a @ w.t()
+    da, dw = a.to(dt).to(DEV), w.to(dt).to(DEV)
+    out = torch.empty(M, N, dtype=dt, device=DEV)
+    ops.gemm_skinny(da, dw, b.to(dt).to(DEV), out)
+    torch.testing.assert_close(out.float().cpu(), q(want + b, dt), **tol(dt))
+    out32 = torch.empty(M, N, dtype=torch.float32, device=DEV)
+    ops.gemm_skinny(da, dw, b.to(DEV), out32)                                   # a bias stored in 32-bit
+    torch.testing.assert_close(out32.cpu(), want + b, rtol=1e-4, atol=1e-4 * K ** 0.5)
+    ops.gemm_skinny(da, dw, None, out32)
+    torch.testing.assert_close(out32.cpu(), want, rtol=1e-4, atol=1e-4 * K ** 0.5)
+    # a row's result does not depend on the other rows of the call, nor on a strided input
+    one = torch.empty(1, N, dtype=torch.float32, device=DEV)
+    ops.gemm_skinny(da[M - 1:], dw, None, one)
+    assert torch.equal(one[0], out32[M - 1])
+    wide = torch.zeros(M, K + 24, dtype=dt, device=DEV)
+    wide[:, :K] = da
+    out_s = torch.empty(M, N, dtype=torch.float32, device=DEV)
+    ops.gemm_skinny(wide[:, :K], dw, None, out_s)
+    assert torch.equal(out_s, out32)
+
+
+@pytest.mark.parametrize("M,I,K", [(1, 128, 64), (8, 4864, 896), (40, 200, 120), (64, 320, 192)])
+def test_gemm_skinny_with_silu_epilogue(ops, M, I, K):
+    torch.manual_seed(10)
+    dt = torch.bfloat16
+    a, w = q(torch.randn(M, K), dt), q(torch.randn(2 * I, K) * 0.2, dt)
+    gu = q(a @ w.t(), dt)
+    want = P.silu_mul(gu[:, :I], gu[:, I:], dt)
+    out = torch.empty(M, I, dtype=dt, device=DEV)
+    ops.gemm_skinny(a.to(dt).to(DEV), w.to(dt).to(DEV), None, out, silu=True)
+    torch.testing.assert_close(out.float().cpu(), want, rtol=2e-2, atol=2e-2)
+    assert ((out.float().cpu() - want).abs() > 1e-2).float().mean() < 0.01      # a rounding flip of gate or up now and then
+
+
+@pytest.mark.parametrize("H,KVH,D,page", [(14, 2, 64, 16), (6, 1, 32, 16), (5, 5, 128, 32), (16, 1, 64, 16),
+                                           (8, 2, 96, 16), (4, 2, 64, 64)])
+@pytest.mark.parametrize("window", [0, 40])
+def test_paged_attention_decode_mfma(ops, H, KVH, D, page, window):
+    dt = torch.bfloat16
+    lens = [1, 2, 16, 17, 255, 256, 257, 700, 64, 1000]
+    q_lens = [1] * len(lens)
+    case = paged_case(dt, lens, q_lens, H, KVH, D, page, seed=11, spike=(7, 2) if not window else None)
+    if window:                                   # pages wholly behind the window must never be read
+        for s, n in enumerate(lens):
+            for i in range(max(0, n - 1 - window + 1) // page):
+                case["kp"][case["tables"][s, i]] = float("nan")
+                case["vp"][case["tables"][s, i]] = float("nan")
+    S = len(lens)
+    scale = D ** -0.5
+    wide = torch.zeros(S, (H + 2 * KVH) * D, dtype=dt, device=DEV)
+    wide[:, :H * D] = case["q"].reshape(S, H * D).to(DEV)
+    out = torch.full((S, H * D), 3.0, dtype=dt, device=DEV)
+    ctx = torch.tensor(lens, dtype=torch.int32, device=DEV)
+    ops.attn_decode_mfma(wide, out, case["kp"].to(DEV), v_layout(case["vp"]).to(DEV), case["tables"].to(DEV), ctx,
+                         H, KVH, D, scale, window, max(lens))
+    want = paged_truth(case, lens, q_lens, scale, dt, window or None).reshape(S, H * D)
+    torch.testing.assert_close(out.float().cpu(), want, **tol(dt))
+    if not window:                               # the spiked far key (position 2 of 700) carries its request's output
+        v_far = case["v"][7][2].float()
+        got = out.float().cpu()[7].view(H, D)
+        for h in range(H):
+            torch.testing.assert_close(got[h], v_far[h // (H // KVH)], rtol=0, atol=5e-2)
+    # the same requests in another batch composition give the same bits
+    sub = [7, 3]
+    out2 = torch.empty(2, H * D, dtype=dt, device=DEV)
+    ops.attn_decode_mfma(wide[sub].contiguous(), out2, case["kp"].to(DEV), v_layout(case["vp"]).to(DEV),
+                         case["tables"][sub].contiguous().to(DEV), ctx[sub].contiguous(), H, KVH, D, scale, window,
+                         max(lens))
+    assert torch.equal(out2, out[sub])

@@ -1,8 +1,11 @@
 """The cache memory on the device.
 
-Per group one tensor [cache layers of the group, 2 (K, V), pages, page_size, kv_heads, head_dim] in
-the model's storage type, the reference's layout (reference src/infer/kv/paged_cache.py:1-6,28-34)
-for each group; per state-holding layer one tensor [slots, *shape].
+Per group two tensors in the model's storage type: keys [cache layers of the group, pages,
+page_size, kv_heads, head_dim], the reference's layout (reference
+src/infer/kv/paged_cache.py:1-6,28-34), and values [cache layers, pages, kv_heads, head_dim,
+page_size]: inside a page the values lie key-contiguous for each (head, d), which is the operand
+layout of the MFMA attention kernels (no transposition through LDS). Per state-holding layer one
+tensor [slots, *shape].
 """
 from __future__ import annotations
 
@@ -35,13 +38,15 @@ class CachePools:
         for j, g in enumerate(group_of_call):
             if g is not None:
                 members[g].append(j)
-        self.kv = [torch.zeros((len(members[g]), 2, counts[g], page_size, s.kv_heads, s.head_dim), dtype=dtype,
-                               device=device) for g, s in enumerate(self.groups)]
+        self.k = [torch.zeros((len(members[g]), counts[g], page_size, s.kv_heads, s.head_dim), dtype=dtype,
+                              device=device) for g, s in enumerate(self.groups)]
+        self.v = [torch.zeros((len(members[g]), counts[g], s.kv_heads, s.head_dim, page_size), dtype=dtype,
+                              device=device) for g, s in enumerate(self.groups)]
         self.states: dict[int, torch.Tensor] = {}
         views: list = [None] * len(specs)
         for g, calls in enumerate(members):
             for idx, j in enumerate(calls):
-                views[j] = KVCacheView(self.kv[g][idx, 0], self.kv[g][idx, 1], g, True)
+                views[j] = KVCacheView(self.k[g][idx], self.v[g][idx], g, True)
         for j, spec in enumerate(specs):
             if isinstance(spec, StateSpec):
                 self.states[j] = torch.zeros((num_state_slots, *spec.shape), dtype=spec.dtype, device=device)
@@ -62,7 +67,7 @@ class CachePools:
 
     @property
     def nbytes(self) -> int:
-        return sum(t.numel() * t.element_size() for t in self.kv) + \
+        return sum(t.numel() * t.element_size() for t in self.k + self.v) + \
             sum(t.numel() * t.element_size() for t in self.states.values())
 
     @staticmethod

@@ -14,7 +14,7 @@ int tm_add_rmsnorm(float* resid, const void* delta, const int* rows, const void*
 
 int tm_rope_kv_write(void* qkv, int dtype, int T, int H, int KVH, int D, int rot, const float* cos_t,
                      const float* sin_t, const int* positions, const int* slots, void* k_pool, void* v_pool,
-                     int write_kv, hipStream_t stream);
+                     int page, int write_kv, hipStream_t stream);
 
 int tm_silu_mul(const void* gu, void* out, int dtype, int T, int I, hipStream_t stream);
 
@@ -27,6 +27,14 @@ int tm_attn_paged_generic(const void* q, int q_stride, void* out, int out_stride
                           const void* v_pool, const int* block_tables, int table_width, const int* seq_of_token,
                           const int* positions, int T, int H, int KVH, int D, int page, float scale, int window,
                           int dtype, hipStream_t stream);
+
+int tm_gemm_skinny(const void* A, int lda, const void* W, const void* bias, int bias_dtype, void* C, int ldc, int M,
+                   int N, int K, int out_dtype, int silu, hipStream_t stream);
+
+int tm_attn_decode_mfma(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
+                        const void* v_pool, const int* block_tables, int table_width, const int* context_lens,
+                        float* part_o, float* part_ml, int max_chunks, int S, int H, int KVH, int D, int page,
+                        float scale, int window, hipStream_t stream);
 
 int tm_argmax_rows(const float* logits, int R, int V, int* out, hipStream_t stream);
 

@@ -1,0 +1,251 @@
+// Paged attention for single decoded tokens on MFMA (bfloat16), split over the context.
+//
+//   One token per request; its G = H / KVH query heads that share a kv head are the 16 columns of
+//   one MFMA tile, so the keys and values of a kv head are read once for all of them
+//   (the reference folds the group into query rows the same way: src/infer/model/layers.py:110-124).
+//   The context is cut into chunks of 256 positions, fixed by position alone; each block of four
+//   wavefronts takes one chunk of one (request, kv head), each wavefront 64 keys of it, and writes
+//   an unnormalised partial (max, sum, weighted values) in 32-bit; attn_decode_merge adds the
+//   partials of a request in ascending chunk order. What a request gets therefore does not depend
+//   on which other requests are in the batch.
+//
+//   Operand layouts need no LDS: keys K[page][slot][kvh][d] give the A operand of S^T = K Q^T
+//   (16 keys x 32 d per instruction), values V[page][kvh][d][slot] give the A operand of
+//   O^T = V^T P^T (16 d x 32 keys), and P^T comes straight from the S^T accumulators.
+#include "common.h"
+#include "api.h"
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+#define AD_CHUNK 256        // keys per block
+#define AD_WKEYS 64         // keys per wavefront
+
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
+    return (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16);
+}
+
+union Bf16x8Bits {
+    u32x4_t u;
+    bf16x8_t b;
+};
+
+// D = head size (multiple of 32, at most 128); page % 16 == 0; G <= 16.
+template <int D>
+__global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
+    const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_pool,
+    const bf16_t* __restrict__ v_pool, const int* __restrict__ block_tables, int table_width,
+    const int* __restrict__ context_lens, float* __restrict__ part_o, float* __restrict__ part_ml,
+    int max_chunks, int H, int KVH, int page, float scale, int window) {
+    constexpr int NDC = D / 32;          // 32-wide d chunks of the q.k product
+    constexpr int NDT = D / 16;          // 16-wide d tiles of the output
+    __shared__ float s_m[4][16], s_l[4][16];
+    __shared__ float s_o[4][16][D + 1];
+
+    const int s = blockIdx.x, kvh = blockIdx.y, chunk = blockIdx.z;
+    const int G = H / KVH;
+    const int ctx = context_lens[s];
+    const int p = ctx - 1;
+    const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+    const int chunk_lo = chunk * AD_CHUNK;
+    if (chunk_lo >= ctx || chunk_lo + AD_CHUNK <= lo) return;       // nothing of this chunk is visible
+
+    const int wave = threadIdx.x / TM_WAVE, lane = threadIdx.x % TM_WAVE;
+    const int r = lane % 16, g = lane / 16;
+    const int* table = block_tables + (size_t)s * table_width;
+
+    // Q^T operand: column r = query head kvh*G + r, rows d = 32c + 8g .. +7
+    Bf16x8Bits qreg[NDC];
+#pragma unroll
+    for (int c = 0; c < NDC; ++c) {
+        if (r < G)
+            qreg[c].u = *(const u32x4_t*)(q + (size_t)s * q_stride + (size_t)(kvh * G + r) * D + 32 * c + 8 * g);
+        else
+            qreg[c].u = u32x4_t{0, 0, 0, 0};
+    }
+
+    const int wbase = chunk_lo + wave * AD_WKEYS;                   // first key of this wavefront
+    float sc[4][4];                                                 // [16-key tile][key 4g+i] for head r
+    int tile_page[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        const int tile0 = wbase + 16 * t;
+        f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+        tile_page[t] = -1;
+        if (tile0 < ctx && tile0 + 16 > lo) {                       // wave-uniform
+            tile_page[t] = table[tile0 / page];
+            const int kj = tile0 + r;                               // this lane's key row of the A operand
+            const bf16_t* kr = k_pool + (((size_t)tile_page[t] * page + (kj % page)) * KVH + kvh) * D + 8 * g;
+#pragma unroll
+            for (int c = 0; c < NDC; ++c) {
+                Bf16x8Bits kreg;
+                kreg.u = (kj < ctx) ? *(const u32x4_t*)(kr + 32 * c) : u32x4_t{0, 0, 0, 0};
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg.b, qreg[c].b, acc, 0, 0, 0);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int kj = tile0 + 4 * g + i;
+            sc[t][i] = (kj < ctx && kj >= lo) ? acc[i] * scale : -INFINITY;
+        }
+    }
+    // softmax pieces of this wavefront's 64 keys, per head r: combine the four key groups g
+    float m = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) m = fmaxf(m, sc[t][i]);
+    m = fmaxf(m, __shfl_xor(m, 16, TM_WAVE));
+    m = fmaxf(m, __shfl_xor(m, 32, TM_WAVE));
+    float l = 0.f;
+    float pr[4][4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            pr[t][i] = (sc[t][i] == -INFINITY) ? 0.f : expf(sc[t][i] - m);
+            l += pr[t][i];
+        }
+    l += __shfl_xor(l, 16, TM_WAVE);
+    l += __shfl_xor(l, 32, TM_WAVE);
+
+    // O^T[d][head] += V^T[d][keys] P^T[keys][head], 32 keys (tiles 2b, 2b+1) per instruction
+    f32x4_t o[NDT];
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) o[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+        if (tile_page[2 * b] < 0 && tile_page[2 * b + 1] < 0) continue;
+        Bf16x8Bits pt;
+        pt.u = u32x4_t{pack_bf16(pr[2 * b][0], pr[2 * b][1]), pack_bf16(pr[2 * b][2], pr[2 * b][3]),
+                       pack_bf16(pr[2 * b + 1][0], pr[2 * b + 1][1]), pack_bf16(pr[2 * b + 1][2], pr[2 * b + 1][3])};
+        // which of this lane's 4 + 4 keys exist (a value beyond the context may hold anything)
+        uint32_t keep[4];
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            const int k0 = wbase + 16 * (2 * b + half) + 4 * g;
+#pragma unroll
+            for (int w2 = 0; w2 < 2; ++w2) {
+                const int ka = k0 + 2 * w2, kb = ka + 1;
+                keep[half * 2 + w2] = ((ka < ctx && ka >= lo) ? 0x0000ffffu : 0u) | ((kb < ctx && kb >= lo) ? 0xffff0000u : 0u);
+            }
+        }
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt) {
+            Bf16x8Bits vreg;
+            vreg.u = u32x4_t{0, 0, 0, 0};
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                const int t = 2 * b + half;
+                if (tile_page[t] >= 0) {
+                    const int in_page = (wbase + 16 * t) % page + 4 * g;
+                    const bf16_t* vr = v_pool + (((size_t)tile_page[t] * KVH + kvh) * D + 16 * dt + r) * page + in_page;
+                    const u32x2_t v2 = *(const u32x2_t*)vr;
+                    vreg.u[half * 2 + 0] = v2[0] & keep[half * 2 + 0];
+                    vreg.u[half * 2 + 1] = v2[1] & keep[half * 2 + 1];
+                }
+            }
+            o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg.b, pt.b, o[dt], 0, 0, 0);
+        }
+    }
+
+    // the four wavefronts of the block -> one partial, added in wavefront order
+    if (g == 0) {
+        s_m[wave][r] = m;
+        s_l[wave][r] = l;
+    }
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) s_o[wave][r][16 * dt + 4 * g + i] = o[dt][i];
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < G * D; idx += 256) {
+        const int n = idx / D, d = idx % D;
+        float mm = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) mm = fmaxf(mm, s_m[w][n]);
+        float ll = 0.f, oo = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const float f = (s_m[w][n] == -INFINITY) ? 0.f : expf(s_m[w][n] - mm);
+            ll += s_l[w][n] * f;
+            oo += s_o[w][n][d] * f;
+        }
+        const size_t slot = ((size_t)s * H + kvh * G + n) * max_chunks + chunk;
+        part_o[slot * D + d] = oo;
+        if (d == 0) {
+            part_ml[slot * 2 + 0] = mm;
+            part_ml[slot * 2 + 1] = ll;
+        }
+    }
+}
+
+// out[s, h, :] = sum over the visible chunks (ascending) of partial values, normalised.
+__global__ void attn_decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                         const int* __restrict__ context_lens, bf16_t* __restrict__ out,
+                                         int out_stride, int max_chunks, int H, int D, int window) {
+    const int s = blockIdx.x, h = blockIdx.y;
+    const int ctx = context_lens[s];
+    const int p = ctx - 1;
+    const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+    const int c0 = lo / AD_CHUNK, c1 = (ctx - 1) / AD_CHUNK;
+    const size_t base = ((size_t)s * H + h) * max_chunks;
+    float mm = -INFINITY;
+    for (int c = c0; c <= c1; ++c) mm = fmaxf(mm, part_ml[(base + c) * 2]);
+    for (int d = threadIdx.x; d < D; d += blockDim.x) {
+        float ll = 0.f, oo = 0.f;
+        for (int c = c0; c <= c1; ++c) {
+            const float mc = part_ml[(base + c) * 2];
+            const float f = (mc == -INFINITY) ? 0.f : expf(mc - mm);
+            ll += part_ml[(base + c) * 2 + 1] * f;
+            oo += part_o[(base + c) * D + d] * f;
+        }
+        out[(size_t)s * out_stride + (size_t)h * D + d] = f32_to_bf16(oo / ll);
+    }
+}
+
+template <int D>
+static int launch_decode(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
+                         const void* v_pool, const int* block_tables, int table_width, const int* context_lens,
+                         float* part_o, float* part_ml, int max_chunks, int S, int H, int KVH, int page,
+                         float scale, int window, hipStream_t stream) {
+    dim3 grid(S, KVH, max_chunks);
+    attn_decode_mfma_kernel<D><<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)k_pool,
+                                                         (const bf16_t*)v_pool, block_tables, table_width,
+                                                         context_lens, part_o, part_ml, max_chunks, H, KVH, page,
+                                                         scale, window);
+    TM_CHECK_LAUNCH();
+    attn_decode_merge_kernel<<<dim3(S, H), 64, 0, stream>>>(part_o, part_ml, context_lens, (bf16_t*)out, out_stride,
+                                                            max_chunks, H, D, window);
+    TM_CHECK_LAUNCH();
+    return TM_OK;
+}
+
+// q: first decode row (one row per request, rows q_stride apart); out likewise; block_tables and
+// context_lens: first decode request. part_o: float [S, H, max_chunks, D]; part_ml: [S, H, max_chunks, 2].
+extern "C" int tm_attn_decode_mfma(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
+                                   const void* v_pool, const int* block_tables, int table_width,
+                                   const int* context_lens, float* part_o, float* part_ml, int max_chunks, int S,
+                                   int H, int KVH, int D, int page, float scale, int window, hipStream_t stream) {
+    if (S <= 0) return TM_OK;
+    if (H <= 0 || KVH <= 0 || H % KVH || H / KVH > 16 || page <= 0 || page % 16 || max_chunks <= 0 ||
+        max_chunks > 65535 || KVH > 65535 || window < 0 || table_width <= 0 || (q_stride % 8) ||
+        ((uintptr_t)q % 16) || q_stride < H * D || out_stride < H * D)
+        return TM_ERR_ARG;
+#define TM_DECODE_CASE(DD)                                                                                        \
+    case DD:                                                                                                      \
+        return launch_decode<DD>(q, q_stride, out, out_stride, k_pool, v_pool, block_tables, table_width,         \
+                                 context_lens, part_o, part_ml, max_chunks, S, H, KVH, page, scale, window, stream)
+    switch (D) {
+        TM_DECODE_CASE(32);
+        TM_DECODE_CASE(64);
+        TM_DECODE_CASE(96);
+        TM_DECODE_CASE(128);
+        default:
+            return TM_ERR_ARG;
+    }
+#undef TM_DECODE_CASE
+}

@@ -8,6 +8,7 @@
 //   keys and values are read in place through the request's block table
 //                               (flat slot of position p = table[p / page] * page + p % page,
 //                                reference src/infer/kv/paged_cache.py:4-5,90-91)
+//   K pool [pages, page, KVH, D]; V pool [pages, KVH, D, page] (key-contiguous per head and d)
 //
 // It takes every head size that is a multiple of 4 up to 256 and any q length and start position,
 // in 32-bit and in bfloat16; it is the attention of the true 32-bit path, and the bfloat16 path
@@ -76,11 +77,11 @@ __global__ __launch_bounds__(AG_WAVES * TM_WAVE) void attn_paged_generic_kernel(
         for (int jj = 0; jj < n; ++jj) {
             const float pj = __shfl(pr_v, jj, TM_WAVE);
             const long long rj = __shfl(row, jj, TM_WAVE);
-            const T* vr = v_pool + ((size_t)rj * KVH + kvh) * D;
+            const T* vr = v_pool + ((size_t)(rj / page) * KVH + kvh) * D * page + (rj % page);
 #pragma unroll
             for (int i = 0; i < AG_MAXD / TM_WAVE; ++i) {
                 const int d = lane + i * TM_WAVE;
-                if (d < D) acc[i] = fmaf(pj, Elem<T>::load(vr + d), acc[i]);
+                if (d < D) acc[i] = fmaf(pj, Elem<T>::load(vr + (size_t)d * page), acc[i]);
             }
         }
     }

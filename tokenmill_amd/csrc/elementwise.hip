@@ -95,58 +95,65 @@ extern "C" int tm_add_rmsnorm(float* resid, const void* delta, const int* rows, 
 //                                                    (reference src/infer/model/layers.py:55-64;
 //                                                     cache write: src/infer/kv/paged_cache.py:40-43)
 //   cos/sin: [max_pos, rot/2] 32-bit; cos == nullptr means no rotation (cache write only).
-//   slot < 0: the token's k and v are not stored (padding rows).
+//   slot = page * page_size + place in the page; slot < 0: k and v are not stored (padding rows).
+//   K pool [pages, page_size, KVH, D]; V pool [pages, KVH, D, page_size]: the values of one page
+//   lie key-contiguous for each (head, d), which is how the MFMA attention kernels read them.
 // ------------------------------------------------------------------------------------------
 template <typename T>
 __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int H, int KVH, int D, int rot,
                                      const float* __restrict__ cos_t, const float* __restrict__ sin_t,
                                      const int* __restrict__ positions, const int* __restrict__ slots,
-                                     T* __restrict__ k_pool, T* __restrict__ v_pool, int write_kv) {
+                                     T* __restrict__ k_pool, T* __restrict__ v_pool, int page, int write_kv) {
     const int t = blockIdx.x, hh = blockIdx.y;
     const int width = (H + 2 * KVH) * D;
     T* x = qkv + (size_t)t * width + (size_t)hh * D;
     const bool is_q = hh < H, is_k = !is_q && hh < H + KVH;
     const int slot = slots ? slots[t] : -1;
-    T* dst = nullptr;
-    if (write_kv && slot >= 0 && !is_q) {
-        const int kvh = is_k ? hh - H : hh - H - KVH;
-        dst = (is_k ? k_pool : v_pool) + ((size_t)slot * KVH + kvh) * D;
-    }
-    const int half = rot / 2;
-    if ((is_q || is_k) && cos_t) {
-        const float* c = cos_t + (size_t)positions[t] * half;
-        const float* s = sin_t + (size_t)positions[t] * half;
-        for (int j = threadIdx.x; j < half; j += blockDim.x) {
-            const float x1 = Elem<T>::load(x + j), x2 = Elem<T>::load(x + j + half);
-            const float y1 = x1 * c[j] - x2 * s[j];
-            const float y2 = x2 * c[j] + x1 * s[j];
-            Elem<T>::store(x + j, y1);
-            Elem<T>::store(x + j + half, y2);
-            if (dst) { Elem<T>::store(dst + j, y1); Elem<T>::store(dst + j + half, y2); }
+    const bool store = write_kv && slot >= 0 && !is_q;
+    if (is_q || is_k) {
+        T* dst = nullptr;
+        if (store) dst = k_pool + ((size_t)slot * KVH + (hh - H)) * D;
+        const int half = rot / 2;
+        if (cos_t) {
+            const float* c = cos_t + (size_t)positions[t] * half;
+            const float* s = sin_t + (size_t)positions[t] * half;
+            for (int j = threadIdx.x; j < half; j += blockDim.x) {
+                const float x1 = Elem<T>::load(x + j), x2 = Elem<T>::load(x + j + half);
+                const float y1 = x1 * c[j] - x2 * s[j];
+                const float y2 = x2 * c[j] + x1 * s[j];
+                Elem<T>::store(x + j, y1);
+                Elem<T>::store(x + j + half, y2);
+                if (dst) { Elem<T>::store(dst + j, y1); Elem<T>::store(dst + j + half, y2); }
+            }
+            if (dst)
+                for (int j = rot + threadIdx.x; j < D; j += blockDim.x) dst[j] = x[j];
+        } else if (dst) {
+            for (int j = threadIdx.x; j < D; j += blockDim.x) dst[j] = x[j];
         }
-        if (dst)
-            for (int j = rot + threadIdx.x; j < D; j += blockDim.x) dst[j] = x[j];
-    } else if (dst) {
-        for (int j = threadIdx.x; j < D; j += blockDim.x) dst[j] = x[j];
+    } else if (store) {
+        const int kvh = hh - H - KVH;
+        const int pg = slot / page, in_page = slot % page;
+        T* dst = v_pool + ((size_t)pg * KVH + kvh) * D * page + in_page;
+        for (int j = threadIdx.x; j < D; j += blockDim.x) dst[(size_t)j * page] = x[j];
     }
 }
 
 extern "C" int tm_rope_kv_write(void* qkv, int dtype, int T, int H, int KVH, int D, int rot,
                                 const float* cos_t, const float* sin_t, const int* positions,
-                                const int* slots, void* k_pool, void* v_pool, int write_kv,
+                                const int* slots, void* k_pool, void* v_pool, int page, int write_kv,
                                 hipStream_t stream) {
     if (T <= 0) return TM_OK;
     if (H <= 0 || KVH <= 0 || D <= 0 || rot < 0 || rot > D || (rot & 1)) return TM_ERR_ARG;
     if (cos_t && (!sin_t || !positions)) return TM_ERR_ARG;
-    if (write_kv && (!slots || !k_pool || !v_pool)) return TM_ERR_ARG;
+    if (write_kv && (!slots || !k_pool || !v_pool || page <= 0)) return TM_ERR_ARG;
     dim3 grid(T, H + 2 * KVH);
     if (dtype == TM_F32)
         rope_kv_write_kernel<float><<<grid, 64, 0, stream>>>((float*)qkv, H, KVH, D, rot, cos_t, sin_t, positions,
-                                                            slots, (float*)k_pool, (float*)v_pool, write_kv);
+                                                            slots, (float*)k_pool, (float*)v_pool, page, write_kv);
     else if (dtype == TM_BF16)
         rope_kv_write_kernel<bf16_t><<<grid, 64, 0, stream>>>((bf16_t*)qkv, H, KVH, D, rot, cos_t, sin_t,
                                                              positions, slots, (bf16_t*)k_pool, (bf16_t*)v_pool,
-                                                             write_kv);
+                                                             page, write_kv);
     else
         return TM_ERR_ARG;
     TM_CHECK_LAUNCH();

@@ -1,0 +1,208 @@
+// C[M, N] = A[M, K] * W[N, K]^T (+ bias) for few rows (M <= 64) on MFMA, bfloat16 in, 32-bit sums.
+//
+// With so few rows the product is bound by reading W once. Each wavefront streams a strip of 16
+// rows of W (16-byte loads straight into the MFMA A operand: 16 rows x 32 k per instruction) and
+// multiplies it with all M activations rows (B operand, 16 tokens per tile). The result tile holds,
+// per lane, four consecutive output features of one token.
+//
+//   split mode : the WAVES wavefronts of a block share one strip and split K between them; their
+//                partial sums are added through LDS in wavefront order (for matrices with few rows,
+//                so that enough wavefronts are in flight).
+//   row mode   : each of the 4 wavefronts of a block has a strip of its own (matrices with many
+//                rows, such as the output head).
+//
+// The K range of each wavefront and the order of all additions depend only on K and the mode,
+// never on M: a token's result does not depend on how many other tokens the call holds.
+// Fused epilogues: bias; silu(gate) * up for a stacked [gate; up] matrix (reference
+// src/infer/model/layers.py:163-164), with gate and up rounded to bfloat16 first as if stored.
+#include "common.h"
+#include "api.h"
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+union Frag {
+    u32x4_t u;
+    bf16x8_t b;
+};
+
+__device__ __forceinline__ Frag load_frag(const bf16_t* row, int k, int K, bool row_ok) {
+    Frag f;
+    if (row_ok && k < K)
+        f.u = *(const u32x4_t*)(row + k);
+    else
+        f.u = u32x4_t{0, 0, 0, 0};
+    return f;
+}
+
+template <typename TC>
+__device__ __forceinline__ void store4(TC* dst, const float v[4], int n_left);
+
+template <>
+__device__ __forceinline__ void store4<float>(float* dst, const float v[4], int n_left) {
+    if (n_left >= 4 && ((uintptr_t)dst % 16) == 0) {
+        *(f32x4_t*)dst = f32x4_t{v[0], v[1], v[2], v[3]};
+    } else {
+        for (int i = 0; i < 4 && i < n_left; ++i) dst[i] = v[i];
+    }
+}
+
+template <>
+__device__ __forceinline__ void store4<bf16_t>(bf16_t* dst, const float v[4], int n_left) {
+    if (n_left >= 4 && ((uintptr_t)dst % 8) == 0) {
+        uint2 pk;
+        pk.x = (uint32_t)f32_to_bf16(v[0]) | ((uint32_t)f32_to_bf16(v[1]) << 16);
+        pk.y = (uint32_t)f32_to_bf16(v[2]) | ((uint32_t)f32_to_bf16(v[3]) << 16);
+        *(uint2*)dst = pk;
+    } else {
+        for (int i = 0; i < 4 && i < n_left; ++i) dst[i] = f32_to_bf16(v[i]);
+    }
+}
+
+__device__ __forceinline__ float bias_at(const void* bias, int bias_f32, int n) {
+    return bias_f32 ? ((const float*)bias)[n] : bf16_to_f32(((const bf16_t*)bias)[n]);
+}
+
+// NT: tiles of 16 tokens. WAVES: wavefronts per block. SPLIT: they share a strip and split K.
+// SILU: W is [2 * N, K] = [gate; up] and the output is silu(gate) * up, N wide.
+template <int NT, int WAVES, bool SPLIT, bool SILU, typename TC>
+__global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ A, int lda,
+                                                                 const bf16_t* __restrict__ W,
+                                                                 const void* __restrict__ bias, int bias_f32,
+                                                                 TC* __restrict__ C, int ldc, int M, int N, int K) {
+    constexpr int NACC = SILU ? 2 : 1;
+    __shared__ float red[SPLIT ? WAVES : 1][64][4 + 1];        // one accumulator tile at a time
+    const int wave = threadIdx.x / TM_WAVE, lane = threadIdx.x % TM_WAVE;
+    const int r = lane % 16, g = lane / 16;
+    const int strip = SPLIT ? blockIdx.x : blockIdx.x * WAVES + wave;
+    const int n0 = strip * 16;
+    // K range of this wavefront, in steps of 32
+    const int ksteps = (K + 31) / 32;
+    int ks0 = 0, ks1 = ksteps;
+    if (SPLIT) {
+        const int per = (ksteps + WAVES - 1) / WAVES;
+        ks0 = wave * per;
+        ks1 = ks0 + per < ksteps ? ks0 + per : ksteps;
+    }
+    const bool w_ok = n0 + r < N;
+    const bf16_t* wrow = W + (size_t)(n0 + r) * K + 8 * g;
+    const bf16_t* urow = SILU ? W + (size_t)(N + n0 + r) * K + 8 * g : nullptr;
+    const bf16_t* arow[NT];
+    bool a_ok[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        a_ok[t] = 16 * t + r < M;
+        arow[t] = A + (size_t)(16 * t + r) * lda + 8 * g;
+    }
+    f32x4_t acc[NACC][NT];
+#pragma unroll
+    for (int a = 0; a < NACC; ++a)
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[a][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    if (n0 < N) {
+#pragma unroll 4
+        for (int ks = ks0; ks < ks1; ++ks) {
+            const int k = ks * 32;
+            const Frag wf = load_frag(wrow, k, K - 8 * g, w_ok);
+            Frag uf;
+            if (SILU) uf = load_frag(urow, k, K - 8 * g, w_ok);
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                const Frag af = load_frag(arow[t], k, K - 8 * g, a_ok[t]);
+                acc[0][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf.b, af.b, acc[0][t], 0, 0, 0);
+                if (SILU) acc[1][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf.b, af.b, acc[1][t], 0, 0, 0);
+            }
+        }
+    }
+    if (SPLIT) {
+#pragma unroll
+        for (int a = 0; a < NACC; ++a)
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) red[wave][lane][i] = acc[a][t][i];
+                __syncthreads();
+                if (wave == 0) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        float v = red[0][lane][i];
+                        for (int w = 1; w < WAVES; ++w) v += red[w][lane][i];
+                        acc[a][t][i] = v;
+                    }
+                }
+                __syncthreads();
+            }
+        if (wave != 0) return;
+    }
+    if (n0 >= N) return;
+    // lane: output features n0 + 4g + i (i = 0..3) of token 16t + r
+    const int nf = n0 + 4 * g;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        const int tok = 16 * t + r;
+        if (tok >= M || nf >= N) continue;
+        float v[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float x = acc[0][t][i];
+            if (bias && nf + i < N) x += bias_at(bias, bias_f32, nf + i);
+            if (SILU) {
+                const float gt = bf16_to_f32(f32_to_bf16(x));
+                const float up = bf16_to_f32(f32_to_bf16(acc[1][t][i]));
+                x = gt / (1.f + expf(-gt)) * up;
+            }
+            v[i] = x;
+        }
+        store4<TC>(C + (size_t)tok * ldc + nf, v, N - nf);
+    }
+}
+
+template <int NT, bool SILU, typename TC>
+static int launch_skinny(const void* A, int lda, const void* W, const void* bias, int bias_f32, void* C, int ldc,
+                         int M, int N, int K, hipStream_t stream) {
+    const int strips = (N + 15) / 16;
+    if (strips >= 2048) {                      // many rows: a strip per wavefront
+        gemm_skinny_kernel<NT, 4, false, SILU, TC><<<(strips + 3) / 4, 256, 0, stream>>>(
+            (const bf16_t*)A, lda, (const bf16_t*)W, bias, bias_f32, (TC*)C, ldc, M, N, K);
+    } else if (strips >= 256 || K < 2048) {    // a block of 4 wavefronts per strip
+        gemm_skinny_kernel<NT, 4, true, SILU, TC><<<strips, 256, 0, stream>>>(
+            (const bf16_t*)A, lda, (const bf16_t*)W, bias, bias_f32, (TC*)C, ldc, M, N, K);
+    } else {                                   // few rows, long K: 16 wavefronts per strip
+        gemm_skinny_kernel<NT, 16, true, SILU, TC><<<strips, 1024, 0, stream>>>(
+            (const bf16_t*)A, lda, (const bf16_t*)W, bias, bias_f32, (TC*)C, ldc, M, N, K);
+    }
+    TM_CHECK_LAUNCH();
+    return TM_OK;
+}
+
+template <bool SILU, typename TC>
+static int launch_skinny_nt(const void* A, int lda, const void* W, const void* bias, int bias_f32, void* C, int ldc,
+                            int M, int N, int K, hipStream_t stream) {
+    switch ((M + 15) / 16) {
+        case 1: return launch_skinny<1, SILU, TC>(A, lda, W, bias, bias_f32, C, ldc, M, N, K, stream);
+        case 2: return launch_skinny<2, SILU, TC>(A, lda, W, bias, bias_f32, C, ldc, M, N, K, stream);
+        case 3: return launch_skinny<3, SILU, TC>(A, lda, W, bias, bias_f32, C, ldc, M, N, K, stream);
+        case 4: return launch_skinny<4, SILU, TC>(A, lda, W, bias, bias_f32, C, ldc, M, N, K, stream);
+        default: return TM_ERR_ARG;
+    }
+}
+
+// silu == 0: C[M, N] = A W^T + bias, W [N, K].   silu == 1: C[M, N] = silu(A Wg^T) * (A Wu^T), W = [Wg; Wu] [2N, K].
+// A, W bfloat16; C bfloat16 (out_dtype 1) or float32 (0); bias bfloat16 or float32 or null.
+// Needs M <= 64, K % 8 == 0, lda % 8 == 0 and 16-byte aligned A and W.
+extern "C" int tm_gemm_skinny(const void* A, int lda, const void* W, const void* bias, int bias_dtype, void* C,
+                              int ldc, int M, int N, int K, int out_dtype, int silu, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return TM_OK;
+    if (M > 64 || K <= 0 || (K % 8) || (lda % 8) || lda < K || ldc < N || ((uintptr_t)A % 16) || ((uintptr_t)W % 16))
+        return TM_ERR_ARG;
+    if (silu && bias) return TM_ERR_ARG;
+    const int bias_f32 = bias_dtype == TM_F32;
+    if (out_dtype == TM_BF16)
+        return silu ? launch_skinny_nt<true, bf16_t>(A, lda, W, bias, bias_f32, C, ldc, M, N, K, stream)
+                    : launch_skinny_nt<false, bf16_t>(A, lda, W, bias, bias_f32, C, ldc, M, N, K, stream);
+    if (out_dtype == TM_F32 && !silu)
+        return launch_skinny_nt<false, float>(A, lda, W, bias, bias_f32, C, ldc, M, N, K, stream);
+    return TM_ERR_ARG;
+}

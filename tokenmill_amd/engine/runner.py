@@ -162,7 +162,8 @@ class ModelRunner:
             cu_q_lens=d(cu_s), context_lens=d(ctx_s), state_slots=d(st_s), logit_rows=d(rows_s)[:R], groups=groups,
             q_lens=q_lens, start_positions=starts, max_q_len=max(q_lens),
             max_context_len=max(s0 + n for s0, n in zip(starts, q_lens)), num_logit_rows=R,
-            num_decode=sum(1 for n in q_lens if n == 1))
+            num_decode=sum(1 for n in q_lens if n == 1),
+            max_decode_context=max([s0 + 1 for s0, n in zip(starts, q_lens) if n == 1], default=0))
         return ctx, list(range(R))
 
     @torch.inference_mode()

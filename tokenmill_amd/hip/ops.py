@@ -53,6 +53,17 @@ def _check(rc: int, name: str) -> None:
         raise RuntimeError(f"{name}: launch failed (code {rc})")
 
 
+def _check_pools(k_pool: torch.Tensor, v_pool: torch.Tensor, KVH: int, D: int, dtype, who: str) -> int:
+    """K pool [pages, page, KVH, D], V pool [pages, KVH, D, page]; returns the page size."""
+    _need(k_pool.dim() == 4 and v_pool.dim() == 4 and k_pool.is_contiguous() and v_pool.is_contiguous(),
+          f"{who}: the cache pools must be contiguous 4-d tensors")
+    pages, page = k_pool.shape[0], k_pool.shape[1]
+    _need(tuple(k_pool.shape) == (pages, page, KVH, D), f"{who}: k_pool must be [pages, page, {KVH}, {D}]")
+    _need(tuple(v_pool.shape) == (pages, KVH, D, page), f"{who}: v_pool must be [pages, {KVH}, {D}, page]")
+    _need(k_pool.dtype == dtype and v_pool.dtype == dtype, f"{who}: the cache pools must have the type {dtype}")
+    return page
+
+
 def _ints(t: torch.Tensor, n: int, name: str) -> None:
     _need(t.dtype == torch.int32 and t.is_contiguous() and t.numel() >= n, f"{name} must be contiguous int32 [{n}]")
 
@@ -98,8 +109,9 @@ def rope_kv_write(qkv: torch.Tensor, H: int, KVH: int, D: int, cos: torch.Tensor
                   positions: torch.Tensor | None, slots: torch.Tensor | None, k_pool: torch.Tensor | None,
                   v_pool: torch.Tensor | None) -> None:
     """Rotate q and k of qkv [T, (H + 2 KVH) D] in place by each token's position and store k, v at
-    the tokens' cache slots. cos/sin float32 [max_pos, rot/2] or None (store only); pools
-    [pages, page, KVH, D] or None (rotate only). A slot < 0 is not stored."""
+    the tokens' cache slots. cos/sin float32 [max_pos, rot/2] or None (store only); k_pool
+    [pages, page, KVH, D] and v_pool [pages, KVH, D, page], or None (rotate only). A slot < 0 is
+    not stored."""
     _gpu(qkv, cos, sin, positions, slots, k_pool, v_pool)
     T = qkv.shape[0]
     _need(qkv.is_contiguous() and qkv.shape[1] == (H + 2 * KVH) * D, "rope_kv_write: qkv must be contiguous [T, (H+2KVH)D]")
@@ -112,15 +124,14 @@ def rope_kv_write(qkv: torch.Tensor, H: int, KVH: int, D: int, cos: torch.Tensor
         _need(0 < rot <= D, f"rope_kv_write: rotary width {rot} does not fit head size {D}")
         _ints(positions, T, "positions")
     write = k_pool is not None
+    page = 0
     if write:
         _need(v_pool is not None and slots is not None, "rope_kv_write: a cache write needs both pools and slots")
-        for pool in (k_pool, v_pool):
-            _need(pool.dtype == qkv.dtype and pool.is_contiguous() and pool.dim() == 4 and
-                  tuple(pool.shape[2:]) == (KVH, D), "rope_kv_write: pools must be [pages, page, KVH, D] of qkv's type")
+        page = _check_pools(k_pool, v_pool, KVH, D, qkv.dtype, "rope_kv_write")
         _ints(slots, T, "slots")
     _check(library().tm_rope_kv_write(_p(qkv), code(qkv.dtype), c_int(T), c_int(H), c_int(KVH), c_int(D), c_int(rot),
                                       _p(cos), _p(sin), _p(positions), _p(slots), _p(k_pool), _p(v_pool),
-                                      c_int(1 if write else 0), _stream()), "rope_kv_write")
+                                      c_int(page), c_int(1 if write else 0), _stream()), "rope_kv_write")
 
 
 def silu_mul(gu: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
@@ -168,16 +179,15 @@ def attn_paged_generic(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor,
                        H: int, KVH: int, D: int, scale: float, window: int = 0) -> torch.Tensor:
     """Attention of every token of the step over its request's cached keys (its own included).
     q: [T, >= H*D] view with unit inner stride (q heads first in each row); out [T, H*D];
-    pools [pages, page, KVH, D]; block_tables int32 [S, W]; seq_of_token, positions int32 [T]."""
+    k_pool [pages, page, KVH, D], v_pool [pages, KVH, D, page]; block_tables int32 [S, W];
+    seq_of_token, positions int32 [T]."""
     _gpu(q, out, k_pool, v_pool, block_tables, seq_of_token, positions)
     T = q.shape[0]
     _need(q.stride(1) == 1 and q.shape[1] >= H * D and out.is_contiguous() and tuple(out.shape) == (T, H * D),
           "attention: q [T, >=H*D] unit inner stride, out contiguous [T, H*D]")
-    _need(q.dtype == out.dtype == k_pool.dtype == v_pool.dtype, "attention: q, out and pools share one type")
+    _need(q.dtype == out.dtype, "attention: q and out share one type")
     _need(H % KVH == 0 and D % 4 == 0 and 0 < D <= 256, f"attention(generic): head size {D} must be a multiple of 4 up to 256")
-    for pool in (k_pool, v_pool):
-        _need(pool.is_contiguous() and pool.dim() == 4 and tuple(pool.shape[2:]) == (KVH, D),
-              "attention: pools must be contiguous [pages, page, KVH, D]")
+    _check_pools(k_pool, v_pool, KVH, D, q.dtype, "attention")
     _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous(),
           "attention: block_tables must be contiguous int32 [S, W]")
     _ints(seq_of_token, T, "seq_of_token")
@@ -214,4 +224,73 @@ def sample_rows(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Te
     _ints(out, R, "out")
     _check(library().tm_sample_rows(_p(logits), c_int(R), c_int(V), _p(temperature), _p(top_k), _p(top_p), _p(u),
                                     _p(out), _stream()), "sample_rows")
+    return out
+
+
+def gemm_skinny(a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, out: torch.Tensor,
+                silu: bool = False) -> torch.Tensor:
+    """MFMA product for at most 64 rows of bfloat16 activations: out[M, N] = a @ w^T (+ bias), or with
+    ``silu`` out[M, N] = silu(a @ w[:N]^T) * (a @ w[N:]^T) for a stacked [gate; up] matrix w [2N, K].
+    out is bfloat16 or float32 (float32 not with silu)."""
+    _gpu(a, w, bias, out)
+    M, K = a.shape
+    N = out.shape[1]
+    _need(a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_skinny: bfloat16 inputs")
+    _need(0 < M <= 64, f"gemm_skinny: at most 64 rows, got {M}")
+    _need(w.is_contiguous() and tuple(w.shape) == ((2 * N if silu else N), K), "gemm_skinny: w must be contiguous [N, K]")
+    _need(a.stride(1) == 1 and out.stride(1) == 1 and out.shape[0] == M, "gemm_skinny: unit inner strides")
+    lda = a.stride(0) if M > 1 else max(K, a.stride(0))
+    ldc = out.stride(0) if M > 1 else max(N, out.stride(0))
+    _need(K % 8 == 0 and lda % 8 == 0 and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0,
+          "gemm_skinny: K and the row stride must be multiples of 8 and the operands 16-byte aligned")
+    _need(out.dtype in (torch.bfloat16, torch.float32) and not (silu and out.dtype != torch.bfloat16),
+          "gemm_skinny: out is bfloat16, or float32 without silu")
+    if bias is not None:
+        _need(not silu and tuple(bias.shape) == (N,) and bias.is_contiguous(), "gemm_skinny: bias must be [N], not with silu")
+    _check(library().tm_gemm_skinny(_p(a), c_int(lda), _p(w), _p(bias),
+                                    c_int(code(bias.dtype) if bias is not None else -1), _p(out), c_int(ldc),
+                                    c_int(M), c_int(N), c_int(K), code(out.dtype), c_int(1 if silu else 0),
+                                    _stream()), "gemm_skinny")
+    return out
+
+
+DECODE_CHUNK = 256          # keys per block of the split decode attention
+
+
+def attn_decode_mfma_supported(dtype, H: int, KVH: int, D: int, page: int) -> bool:
+    return dtype == torch.bfloat16 and D in (32, 64, 96, 128) and page % 16 == 0 and H % KVH == 0 and H // KVH <= 16
+
+
+def attn_decode_mfma(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
+                     block_tables: torch.Tensor, context_lens: torch.Tensor, H: int, KVH: int, D: int, scale: float,
+                     window: int, max_context: int, workspace: tuple[torch.Tensor, torch.Tensor] | None = None):
+    """Attention of one new token per request over its cache (the token's own key included).
+    q: [S, >= H*D] rows (unit inner stride), out [S, H*D] view; block_tables int32 [S, W];
+    context_lens int32 [S] (new token counted); max_context >= every context length."""
+    _gpu(q, out, k_pool, v_pool, block_tables, context_lens)
+    S = q.shape[0]
+    page = _check_pools(k_pool, v_pool, KVH, D, torch.bfloat16, "attn_decode")
+    _need(attn_decode_mfma_supported(q.dtype, H, KVH, D, page), "attn_decode: unsupported head size, group or page size")
+    _need(q.stride(1) == 1 and out.stride(1) == 1 and out.dtype == torch.bfloat16 and out.shape[0] == S
+          and q.shape[1] >= H * D and out.shape[1] >= H * D, "attn_decode: q, out [S, >= H*D] with unit inner stride")
+    q_stride = q.stride(0) if S > 1 else max(q.stride(0), H * D)
+    out_stride = out.stride(0) if S > 1 else max(out.stride(0), H * D)
+    _need(q_stride % 8 == 0 and q.data_ptr() % 16 == 0, "attn_decode: q rows must be 16-byte aligned")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.shape[0] >= S
+          and block_tables.stride(1) == 1, "attn_decode: block_tables must be int32 [S, W]")
+    W = block_tables.shape[1]
+    _need(block_tables.stride(0) == W or S == 1, "attn_decode: block_tables rows must be contiguous")
+    _ints(context_lens, S, "context_lens")
+    _need(0 < max_context <= W * page, "attn_decode: max_context exceeds what the block tables hold")
+    chunks = -(-max_context // DECODE_CHUNK)
+    if workspace is None:
+        workspace = (torch.empty((S, H, chunks, D), dtype=torch.float32, device=q.device),
+                     torch.empty((S, H, chunks, 2), dtype=torch.float32, device=q.device))
+    part_o, part_ml = workspace
+    _need(part_o.numel() >= S * H * chunks * D and part_ml.numel() >= S * H * chunks * 2
+          and part_o.dtype == torch.float32 and part_ml.dtype == torch.float32, "attn_decode: workspace too small")
+    _check(library().tm_attn_decode_mfma(_p(q), c_int(q_stride), _p(out), c_int(out_stride), _p(k_pool), _p(v_pool),
+                                         _p(block_tables), c_int(W), _p(context_lens), _p(part_o), _p(part_ml),
+                                         c_int(chunks), c_int(S), c_int(H), c_int(KVH), c_int(D), c_int(page),
+                                         c_float(scale), c_int(window), _stream()), "attn_decode_mfma")
     return out

@@ -39,7 +39,7 @@ class StateSpec:
 class KVCacheView:
     """One cache layer as a mixer sees it."""
     k: torch.Tensor              # [pages, page_size, kv_heads, head_dim]
-    v: torch.Tensor
+    v: torch.Tensor              # [pages, kv_heads, head_dim, page_size]
     group: int                   # index into StepContext.groups
     write: bool = True           # False: this layer reads a cache that another layer writes
 
@@ -79,6 +79,7 @@ class StepContext:
     num_logit_rows: int = 0
     # S entries are ordered with the q_len == 1 entries last; this many of them:
     num_decode: int = 0
+    max_decode_context: int = 0      # longest context among them (new token counted)
 
 
 # ------------------------------------------------------------------------------------------------

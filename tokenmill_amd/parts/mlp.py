@@ -4,7 +4,7 @@ from __future__ import annotations
 
 import torch
 
-from tokenmill_amd.hip import ops
+from tokenmill_amd.hip import gemm, ops
 from tokenmill_amd.parts.base import FeedForward, StepContext
 from tokenmill_amd.parts.linear import Linear
 
@@ -24,6 +24,8 @@ class SwiGLU(FeedForward):
         self.down.load(tensors, prefix)
 
     def forward(self, x: torch.Tensor, step: StepContext | None = None) -> torch.Tensor:
-        gu = self.gate_up.forward(x)
-        act = ops.silu_mul(gu, torch.empty((x.shape[0], self.intermediate), dtype=gu.dtype, device=x.device))
+        act = torch.empty((x.shape[0], self.intermediate), dtype=x.dtype, device=x.device)
+        w = self.gate_up.weight
+        if not (w.dtype == x.dtype and self.gate_up.bias is None and gemm.gate_up_silu(x, w, act)):
+            ops.silu_mul(self.gate_up.forward(x), act)
         return self.down.forward(act)
