@@ -172,3 +172,30 @@ def test_command_line(model_dirs, plains):
     assert [ln["prompt_tokens"] for ln in lines] == [3, 2]
     verify(plains["A"], [1, 2, 3], lines[0]["output_ids"], torch.float32)
     verify(plains["A"], [4, 5], lines[1]["output_ids"], torch.float32)
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_decode_steps_replayed_from_hip_graphs(model_dirs, plains, dtype_name):
+    """Graph replays between eager prefill steps, batch sizes that change as requests come and go:
+    every replay gives what the eager engine gives."""
+    from tokenmill_amd import SamplingParams
+    lengths = [3, 30, 17, 9, 1, 40, 22]
+    prompts = [random_ids(n, 384, 90 + i) for i, n in enumerate(lengths)]
+    params = [SamplingParams(max_tokens=6 + 5 * i, ignore_eos=True) for i in range(len(lengths))]
+    outs = {}
+    for graphs in (False, True):
+        eng = make_engine(model_dirs["B"], dtype_name, block_size=16, hip_graphs=graphs, max_num_seqs=6,
+                          max_num_batched_tokens=48)
+        seqs = [eng.add_request(f"r{i}", p, sp) for i, (p, sp) in enumerate(zip(prompts[:4], params[:4]))]
+        for _ in range(4):
+            eng.step()
+        seqs += [eng.add_request(f"r{i + 4}", p, sp) for i, (p, sp) in enumerate(zip(prompts[4:], params[4:]))]
+        while eng.has_unfinished():
+            eng.step()
+        outs[graphs] = [s.output_ids for s in seqs]
+        if graphs:
+            assert eng.runner.graphs.replays > 20 and len(eng.runner.graphs.buckets) >= 3
+        assert eng.cache.num_free_pages == eng.cache.num_pages
+    for p, o in zip(prompts, outs[True]):
+        verify(plains["B"], p, o, DTYPES[dtype_name])
+    assert outs[True] == outs[False]

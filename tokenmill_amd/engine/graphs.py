@@ -1,0 +1,147 @@
+"""HIP graphs for decode steps.
+
+A step in which every request decodes one token launches the same kernels with the same grids
+whatever the requests are, once the batch is padded to a bucket size and the block tables to the
+width of the longest request the engine allows. Such a step is captured once per bucket and then
+replayed: one graph launch instead of a few hundred kernel launches from the host. (The reference
+has the same device for the same reason: reference src/infer/engine/cuda_graphs.py:88-115, and its
+profile of where an eager decode step's time goes, bench/results/profile/decode_breakdown_b32.json.)
+
+Padding rows carry token 0 at position 0, a context of one key, and cache slot -1, which the cache
+write skips; their logits are never looked at. The graphs hold no memset node.
+"""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from tokenmill_amd.cache.manager import RELEASED
+from tokenmill_amd.parts.base import GroupStep, StepContext
+
+
+class _Bucket:
+    def __init__(self, runner, B: int, W: int):
+        self.B, self.W = B, W
+        n_groups = len(runner.pools.groups)
+        self.n_ints = 3 * B + (B + 1) + 3 * B + n_groups * (B + B * W)
+        self.pinned = torch.zeros(self.n_ints, dtype=torch.int32, pin_memory=True)
+        self.dev = torch.zeros(self.n_ints, dtype=torch.int32, device=runner.device)
+        off = 0
+
+        def take(n):
+            nonlocal off
+            span = (off, off + n)
+            off += n
+            return span
+
+        self.ids, self.pos, self.seq_of = take(B), take(B), take(B)
+        self.cu, self.ctx, self.state, self.rows = take(B + 1), take(B), take(B), take(B)
+        self.g_slot = [take(B) for _ in range(n_groups)]
+        self.g_tab = [take(B * W) for _ in range(n_groups)]
+        host = self.pinned.numpy()
+        host[self.seq_of[0]:self.seq_of[1]] = np.arange(B)
+        host[self.cu[0]:self.cu[1]] = np.arange(B + 1)
+        host[self.rows[0]:self.rows[1]] = np.arange(B)
+        self.graph: torch.cuda.CUDAGraph | None = None
+        self.logits: torch.Tensor | None = None
+
+    def view(self, span):
+        return self.dev[span[0]:span[1]]
+
+    def context(self, max_positions: int) -> StepContext:
+        B, W = self.B, self.W
+        groups = [GroupStep(block_tables=self.view(t).view(B, W), slot_mapping=self.view(s))
+                  for s, t in zip(self.g_slot, self.g_tab)]
+        return StepContext(num_tokens=B, num_seqs=B, token_ids=self.view(self.ids), positions=self.view(self.pos),
+                           seq_of_token=self.view(self.seq_of), cu_q_lens=self.view(self.cu),
+                           context_lens=self.view(self.ctx), state_slots=self.view(self.state),
+                           logit_rows=self.view(self.rows), groups=groups, q_lens=[1] * B, start_positions=[0] * B,
+                           max_q_len=1, max_context_len=max_positions, num_logit_rows=B, num_decode=B,
+                           max_decode_context=max_positions)
+
+
+class DecodeGraphs:
+    def __init__(self, runner, cfg, max_batch: int = 256):
+        self.runner = runner
+        self.page = runner.page_size
+        self.max_positions = runner.max_positions
+        self.W = -(-runner.max_positions // self.page)
+        top = min(cfg.max_num_seqs, max_batch)
+        self.sizes = [b for b in (1, 2, 4, 8, 16, 32, 64, 128, 256) if b < top] + [top]
+        self.buckets: dict[int, _Bucket] = {}
+        self.replays = 0
+        self._copied = torch.cuda.Event()
+
+    def can_run(self, entries) -> bool:
+        return (0 < len(entries) <= self.sizes[-1] and all(len(e.tokens) == 1 for e in entries)
+                and not self.runner.pools.states)
+
+    def _bucket(self, n: int) -> _Bucket:
+        B = next(b for b in self.sizes if b >= n)
+        if B not in self.buckets:
+            self.buckets[B] = _Bucket(self.runner, B, self.W)
+        return self.buckets[B]
+
+    @torch.inference_mode()
+    def run(self, entries) -> torch.Tensor:
+        """Float32 logits [wanted, vocab], entries in the given order (each wants place 0 or nothing)."""
+        runner = self.runner
+        bk = self._bucket(len(entries))
+        B, W, page = bk.B, bk.W, self.page
+        self._copied.synchronize()                          # the last replay's copy has left the pinned buffer
+        host = bk.pinned.numpy()
+        n = len(entries)
+        ids = np.zeros(B, dtype=np.int64)
+        pos = np.zeros(B, dtype=np.int64)
+        for i, e in enumerate(entries):
+            ids[i], pos[i] = e.tokens[0], e.start
+        if ids.min() < 0 or ids.max() >= runner.vocab:
+            raise ValueError("a token id is outside the vocabulary")
+        if pos.max() >= self.max_positions:
+            raise ValueError(f"a position exceeds the model's {self.max_positions}")
+        host[bk.ids[0]:bk.ids[1]] = ids
+        host[bk.pos[0]:bk.pos[1]] = pos
+        ctx = pos + 1
+        ctx[n:] = 1
+        host[bk.ctx[0]:bk.ctx[1]] = ctx
+        state = host[bk.state[0]:bk.state[1]]
+        state[:] = 0
+        for i, e in enumerate(entries):
+            state[i] = e.cache.state_slot
+        for g in range(len(runner.pools.groups)):
+            slots = host[bk.g_slot[g][0]:bk.g_slot[g][1]]
+            tabs = host[bk.g_tab[g][0]:bk.g_tab[g][1]].reshape(B, W)
+            slots[:] = -1
+            for i, e in enumerate(entries):
+                table = e.cache.tables[g]
+                need = e.start // page + 1
+                if len(table) < need or table[need - 1] == RELEASED:
+                    raise ValueError(f"{e.cache.request_id}: no page for position {e.start}")
+                row = np.asarray(table[:need], dtype=np.int64)
+                tabs[i, :need] = np.where(row == RELEASED, 0, row)
+                slots[i] = table[need - 1] * page + e.start % page
+        bk.dev.copy_(bk.pinned, non_blocking=True)
+        self._copied.record()
+        if bk.graph is None:
+            self._capture(bk)
+        bk.graph.replay()
+        self.replays += 1
+        wanted = [i for i, e in enumerate(entries) if e.want]
+        if wanted == list(range(n)):
+            return bk.logits[:n]
+        return bk.logits[torch.tensor(wanted, dtype=torch.long, device=bk.logits.device)]
+
+    def _capture(self, bk: _Bucket) -> None:
+        runner = self.runner
+        step = bk.context(self.max_positions)
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):                       # a first run outside the graph: lazy set-up happens here
+            runner.model.forward(step, runner.pools.views)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            bk.logits = runner.model.forward(step, runner.pools.views)
+        bk.graph = graph

@@ -174,5 +174,7 @@ class ModelRunner:
             if e.cache.fresh:                     # per-request state starts from zero at (re)admission
                 self.pools.reset_state_slot(e.cache.state_slot)
                 e.cache.fresh = False
+        if self.graphs is not None and self.graphs.can_run(entries):
+            return self.graphs.run(entries)
         ctx, _ = self.prepare(entries)
         return self.model.forward(ctx, self.pools.views)
