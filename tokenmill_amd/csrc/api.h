@@ -36,6 +36,10 @@ int tm_attn_decode_mfma(const void* q, int q_stride, void* out, int out_stride, 
                         float* part_o, float* part_ml, int max_chunks, int S, int H, int KVH, int D, int page,
                         float scale, int window, hipStream_t stream);
 
+int tm_attn_prefill_mfma(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
+                         const void* v_pool, const int* block_tables, int table_width, const int* tiles, int n_tiles,
+                         int H, int KVH, int D, int page, float scale, int window, hipStream_t stream);
+
 int tm_argmax_rows(const float* logits, int R, int V, int* out, hipStream_t stream);
 
 int tm_sample_rows(const float* logits, int R, int V, const float* temperature, const int* top_k,

@@ -87,7 +87,8 @@ class ModelRunner:
                 if not 0 <= w < len(e.tokens):
                     raise StepError(f"{e.cache.request_id}: wanted place {w} is not among its {len(e.tokens)} tokens")
         W = max(widths)
-        n_ints = 3 * T + (S + 1) + 2 * S + max(R, 1) + n_groups * (T + S * W)
+        n_tiles = sum(-(-len(e.tokens) // 16) for e in entries if len(e.tokens) > 1)
+        n_ints = 3 * T + (S + 1) + 2 * S + max(R, 1) + n_groups * (T + S * W) + 4 * n_tiles
         buf = self._staging(n_ints)
         off = 0
 
@@ -110,6 +111,8 @@ class ModelRunner:
             g_slot.append(take(T))
             g_tab.append(take(S * W))
 
+        tiles, tiles_s = take(4 * n_tiles)
+        tile_i = 0
         row0 = 0
         first_row = [0] * S
         q_lens, starts = [], []
@@ -136,6 +139,10 @@ class ModelRunner:
                 tab = g_tab[g][0][s * W:(s + 1) * W]
                 tab[:widths[i]] = np.where(table == RELEASED, 0, table)   # never read: below the window
                 tab[widths[i]:] = 0                                       # padding: never read either
+            if n > 1:
+                for j in range(0, n, 16):
+                    tiles[4 * tile_i:4 * tile_i + 4] = (s, row0 + j, min(16, n - j), e.start + j)
+                    tile_i += 1
             first_row[i] = row0
             q_lens.append(n)
             starts.append(e.start)
@@ -163,7 +170,8 @@ class ModelRunner:
             q_lens=q_lens, start_positions=starts, max_q_len=max(q_lens),
             max_context_len=max(s0 + n for s0, n in zip(starts, q_lens)), num_logit_rows=R,
             num_decode=sum(1 for n in q_lens if n == 1),
-            max_decode_context=max([s0 + 1 for s0, n in zip(starts, q_lens) if n == 1], default=0))
+            max_decode_context=max([s0 + 1 for s0, n in zip(starts, q_lens) if n == 1], default=0),
+            prefill_tiles=d(tiles_s).view(n_tiles, 4))
         return ctx, list(range(R))
 
     @torch.inference_mode()

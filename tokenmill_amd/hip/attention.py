@@ -1,8 +1,9 @@
 """Which attention kernels a step runs.
 
-The step's entries are ordered with the single-token entries last. In bfloat16 those go to the
-split-context MFMA decode kernel when it takes the head size, group and page size; everything
-else (prompt portions, the true 32-bit path, unusual shapes) goes to the generic kernel.
+The step's entries are ordered with the single-token entries last. In bfloat16, when the head
+size and page size allow, prompt portions go to the flash-style MFMA kernel and single tokens to
+the split-context MFMA decode kernel; everything else (the true 32-bit path, unusual shapes) goes
+to the generic kernel.
 """
 from __future__ import annotations
 
@@ -17,14 +18,23 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, cache: KVCacheView, st
     """q = the first H*D columns of qkv; keys and values come from the cache (this step's included)."""
     g = step.groups[cache.group]
     T, S, nd = step.num_tokens, step.num_seqs, step.num_decode
+    tp = T - nd
     page = cache.k.shape[1]
+    done_prefill = done_decode = False
+    if tp and step.prefill_tiles is not None and ops.attn_prefill_mfma_supported(qkv.dtype, H, KVH, D, page):
+        ops.attn_prefill_mfma(qkv, out, cache.k, cache.v, g.block_tables, step.prefill_tiles, H, KVH, D, scale, window)
+        done_prefill = True
     if nd and ops.attn_decode_mfma_supported(qkv.dtype, H, KVH, D, page):
-        tp = T - nd
-        if tp:
-            ops.attn_paged_generic(qkv[:tp], out[:tp], cache.k, cache.v, g.block_tables, step.seq_of_token[:tp],
-                                   step.positions[:tp], H, KVH, D, scale, window)
         ops.attn_decode_mfma(qkv[tp:], out[tp:], cache.k, cache.v, g.block_tables[S - nd:], step.context_lens[S - nd:],
                              H, KVH, D, scale, window, step.max_decode_context)
-        return out
-    return ops.attn_paged_generic(qkv, out, cache.k, cache.v, g.block_tables, step.seq_of_token, step.positions,
-                                  H, KVH, D, scale, window)
+        done_decode = True
+    if tp and not done_prefill and nd and not done_decode:
+        return ops.attn_paged_generic(qkv, out, cache.k, cache.v, g.block_tables, step.seq_of_token, step.positions,
+                                      H, KVH, D, scale, window)
+    if tp and not done_prefill:
+        ops.attn_paged_generic(qkv[:tp], out[:tp], cache.k, cache.v, g.block_tables, step.seq_of_token[:tp],
+                               step.positions[:tp], H, KVH, D, scale, window)
+    if nd and not done_decode:
+        ops.attn_paged_generic(qkv[tp:], out[tp:], cache.k, cache.v, g.block_tables, step.seq_of_token[tp:],
+                               step.positions[tp:], H, KVH, D, scale, window)
+    return out

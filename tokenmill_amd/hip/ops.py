@@ -294,3 +294,37 @@ def attn_decode_mfma(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v
                                          c_int(chunks), c_int(S), c_int(H), c_int(KVH), c_int(D), c_int(page),
                                          c_float(scale), c_int(window), _stream()), "attn_decode_mfma")
     return out
+
+
+PREFILL_TILE = 16           # query tokens per tile of the MFMA prefill attention
+
+
+def attn_prefill_mfma_supported(dtype, H: int, KVH: int, D: int, page: int) -> bool:
+    return dtype == torch.bfloat16 and D in (32, 64, 96, 128) and page % 16 == 0 and H % KVH == 0
+
+
+def attn_prefill_mfma(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
+                      block_tables: torch.Tensor, tiles: torch.Tensor, H: int, KVH: int, D: int, scale: float,
+                      window: int) -> torch.Tensor:
+    """Attention of prompt portions over the cache. q: [T, >= H*D] rows, out [T, H*D]; tiles int32
+    [n, 4] = (request index, first row, tokens (1..16), position of the first token) cover the rows
+    to compute; every row of a tile belongs to one request at consecutive positions."""
+    _gpu(q, out, k_pool, v_pool, block_tables, tiles)
+    T = q.shape[0]
+    page = _check_pools(k_pool, v_pool, KVH, D, torch.bfloat16, "attn_prefill")
+    _need(attn_prefill_mfma_supported(q.dtype, H, KVH, D, page), "attn_prefill: unsupported head size or page size")
+    _need(q.stride(1) == 1 and out.stride(1) == 1 and out.dtype == torch.bfloat16 and out.shape[0] == T
+          and q.shape[1] >= H * D and out.shape[1] >= H * D, "attn_prefill: q, out [T, >= H*D] with unit inner stride")
+    q_stride = q.stride(0) if T > 1 else max(q.stride(0), H * D)
+    out_stride = out.stride(0) if T > 1 else max(out.stride(0), H * D)
+    _need(q_stride % 8 == 0 and q.data_ptr() % 16 == 0 and out_stride % 4 == 0 and out.data_ptr() % 8 == 0,
+          "attn_prefill: q rows must be 16-byte aligned and out rows 8-byte aligned")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous(),
+          "attn_prefill: block_tables must be contiguous int32 [S, W]")
+    _need(tiles.dtype == torch.int32 and tiles.dim() == 2 and tiles.shape[1] == 4 and tiles.is_contiguous(),
+          "attn_prefill: tiles must be contiguous int32 [n, 4]")
+    _check(library().tm_attn_prefill_mfma(_p(q), c_int(q_stride), _p(out), c_int(out_stride), _p(k_pool), _p(v_pool),
+                                          _p(block_tables), c_int(block_tables.shape[1]), _p(tiles),
+                                          c_int(tiles.shape[0]), c_int(H), c_int(KVH), c_int(D), c_int(page),
+                                          c_float(scale), c_int(window), _stream()), "attn_prefill_mfma")
+    return out

@@ -80,6 +80,9 @@ class StepContext:
     # S entries are ordered with the q_len == 1 entries last; this many of them:
     num_decode: int = 0
     max_decode_context: int = 0      # longest context among them (new token counted)
+    # the q_len > 1 entries cut into tiles of at most 16 tokens: int32 [n, 4] =
+    # (request index, first row, tokens, position of the first token)
+    prefill_tiles: torch.Tensor | None = None
 
 
 # ------------------------------------------------------------------------------------------------
