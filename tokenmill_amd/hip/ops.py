@@ -300,7 +300,8 @@ PREFILL_TILE = 16           # query tokens per tile of the MFMA prefill attentio
 
 
 def attn_prefill_mfma_supported(dtype, H: int, KVH: int, D: int, page: int) -> bool:
-    return dtype == torch.bfloat16 and D in (32, 64, 96, 128) and page % 16 == 0 and H % KVH == 0
+    return (dtype == torch.bfloat16 and D in (32, 64, 96, 128) and page >= 16 and page & (page - 1) == 0
+            and H % KVH == 0)
 
 
 def attn_prefill_mfma(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
@@ -317,8 +318,8 @@ def attn_prefill_mfma(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, 
           and q.shape[1] >= H * D and out.shape[1] >= H * D, "attn_prefill: q, out [T, >= H*D] with unit inner stride")
     q_stride = q.stride(0) if T > 1 else max(q.stride(0), H * D)
     out_stride = out.stride(0) if T > 1 else max(out.stride(0), H * D)
-    _need(q_stride % 8 == 0 and q.data_ptr() % 16 == 0 and out_stride % 4 == 0 and out.data_ptr() % 8 == 0,
-          "attn_prefill: q rows must be 16-byte aligned and out rows 8-byte aligned")
+    _need(q_stride % 8 == 0 and q.data_ptr() % 16 == 0 and out_stride % 2 == 0 and out.data_ptr() % 4 == 0,
+          "attn_prefill: q rows must be 16-byte aligned and out rows 4-byte aligned")
     _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous(),
           "attn_prefill: block_tables must be contiguous int32 [S, W]")
     _need(tiles.dtype == torch.int32 and tiles.dim() == 2 and tiles.shape[1] == 4 and tiles.is_contiguous(),
