@@ -24,8 +24,13 @@ typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 #define AD_CHUNK 256        // keys per block
 #define AD_WKEYS 64         // keys per wavefront
 
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+
+// two floats -> packed bfloat16 (round to nearest even, one instruction on gfx950)
 __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
-    return (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16);
+    const bf16x2_t v = __builtin_convertvector(f32x2_t{a, b}, bf16x2_t);
+    return *(const uint32_t*)&v;
 }
 
 union Bf16x8Bits {
@@ -33,13 +38,14 @@ union Bf16x8Bits {
     bf16x8_t b;
 };
 
-// D = head size (multiple of 32, at most 128); page % 16 == 0; G <= 16.
+// D = head size (multiple of 32, at most 128); page a power of two >= 16; G <= 16.
+// Scores are kept as score * scale * log2(e) so that the exponentials are single exp2 instructions.
 template <int D>
 __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_pool,
     const bf16_t* __restrict__ v_pool, const int* __restrict__ block_tables, int table_width,
     const int* __restrict__ context_lens, float* __restrict__ part_o, float* __restrict__ part_ml,
-    int max_chunks, int H, int KVH, int page, float scale, int window) {
+    int max_chunks, int H, int KVH, int page_shift, float scale_log2, int window) {
     constexpr int NDC = D / 32;          // 32-wide d chunks of the q.k product
     constexpr int NDT = D / 16;          // 16-wide d tiles of the output
     __shared__ float s_m[4][16], s_l[4][16];
@@ -56,7 +62,16 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
     const int wave = threadIdx.x / TM_WAVE, lane = threadIdx.x % TM_WAVE;
     const int r = lane % 16, g = lane / 16;
     const int* table = block_tables + (size_t)s * table_width;
+    const int page_mask = (1 << page_shift) - 1;
+    const int wbase = chunk_lo + wave * AD_WKEYS;                   // first key of this wavefront
 
+    // every load of the wavefront is issued before the first product
+    int tile_page[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        const int tile0 = wbase + 16 * t;
+        tile_page[t] = (tile0 < ctx && tile0 + 16 > lo) ? table[tile0 >> page_shift] : -1;      // wave-uniform
+    }
     // Q^T operand: column r = query head kvh*G + r, rows d = 32c + 8g .. +7
     Bf16x8Bits qreg[NDC];
 #pragma unroll
@@ -66,30 +81,35 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
         else
             qreg[c].u = u32x4_t{0, 0, 0, 0};
     }
-
-    const int wbase = chunk_lo + wave * AD_WKEYS;                   // first key of this wavefront
-    float sc[4][4];                                                 // [16-key tile][key 4g+i] for head r
-    int tile_page[4];
+    Bf16x8Bits kreg[4][NDC];
+    u32x2_t vreg[NDT][4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
         const int tile0 = wbase + 16 * t;
-        f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
-        tile_page[t] = -1;
-        if (tile0 < ctx && tile0 + 16 > lo) {                       // wave-uniform
-            tile_page[t] = table[tile0 / page];
-            const int kj = tile0 + r;                               // this lane's key row of the A operand
-            const bf16_t* kr = k_pool + (((size_t)tile_page[t] * page + (kj % page)) * KVH + kvh) * D + 8 * g;
+        const int in_page = tile0 & page_mask;
+        const bool have = tile_page[t] >= 0;
+        const size_t pg = have ? (size_t)tile_page[t] : 0;
+        const bf16_t* kr = k_pool + (((pg << page_shift) + in_page + r) * KVH + kvh) * D + 8 * g;
+        const bf16_t* vr = v_pool + (((pg * KVH + kvh) * D + r) << page_shift) + in_page + 4 * g;
 #pragma unroll
-            for (int c = 0; c < NDC; ++c) {
-                Bf16x8Bits kreg;
-                kreg.u = (kj < ctx) ? *(const u32x4_t*)(kr + 32 * c) : u32x4_t{0, 0, 0, 0};
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg.b, qreg[c].b, acc, 0, 0, 0);
-            }
-        }
+        for (int c = 0; c < NDC; ++c)
+            kreg[t][c].u = (have && tile0 + r < ctx) ? *(const u32x4_t*)(kr + 32 * c) : u32x4_t{0, 0, 0, 0};
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt)
+            vreg[dt][t] = have ? *(const u32x2_t*)(vr + ((size_t)(16 * dt) << page_shift)) : u32x2_t{0, 0};
+    }
+
+    float sc[4][4];                                                 // [16-key tile][key 4g+i] for head r
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c = 0; c < NDC; ++c)
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[t][c].b, qreg[c].b, acc, 0, 0, 0);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const int kj = tile0 + 4 * g + i;
-            sc[t][i] = (kj < ctx && kj >= lo) ? acc[i] * scale : -INFINITY;
+            const int kj = wbase + 16 * t + 4 * g + i;
+            sc[t][i] = (kj < ctx && kj >= lo) ? acc[i] * scale_log2 : -INFINITY;
         }
     }
     // softmax pieces of this wavefront's 64 keys, per head r: combine the four key groups g
@@ -100,13 +120,14 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
         for (int i = 0; i < 4; ++i) m = fmaxf(m, sc[t][i]);
     m = fmaxf(m, __shfl_xor(m, 16, TM_WAVE));
     m = fmaxf(m, __shfl_xor(m, 32, TM_WAVE));
+    const float neg_m = (m == -INFINITY) ? 0.f : -m;
     float l = 0.f;
     float pr[4][4];
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            pr[t][i] = (sc[t][i] == -INFINITY) ? 0.f : expf(sc[t][i] - m);
+            pr[t][i] = __builtin_amdgcn_exp2f(sc[t][i] + neg_m);
             l += pr[t][i];
         }
     l += __shfl_xor(l, 16, TM_WAVE);
@@ -135,20 +156,10 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
         }
 #pragma unroll
         for (int dt = 0; dt < NDT; ++dt) {
-            Bf16x8Bits vreg;
-            vreg.u = u32x4_t{0, 0, 0, 0};
-#pragma unroll
-            for (int half = 0; half < 2; ++half) {
-                const int t = 2 * b + half;
-                if (tile_page[t] >= 0) {
-                    const int in_page = (wbase + 16 * t) % page + 4 * g;
-                    const bf16_t* vr = v_pool + (((size_t)tile_page[t] * KVH + kvh) * D + 16 * dt + r) * page + in_page;
-                    const u32x2_t v2 = *(const u32x2_t*)vr;
-                    vreg.u[half * 2 + 0] = v2[0] & keep[half * 2 + 0];
-                    vreg.u[half * 2 + 1] = v2[1] & keep[half * 2 + 1];
-                }
-            }
-            o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg.b, pt.b, o[dt], 0, 0, 0);
+            Bf16x8Bits vf;
+            vf.u = u32x4_t{vreg[dt][2 * b][0] & keep[0], vreg[dt][2 * b][1] & keep[1],
+                           vreg[dt][2 * b + 1][0] & keep[2], vreg[dt][2 * b + 1][1] & keep[3]};
+            o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.b, pt.b, o[dt], 0, 0, 0);
         }
     }
 
@@ -170,7 +181,7 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
         float ll = 0.f, oo = 0.f;
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
-            const float f = (s_m[w][n] == -INFINITY) ? 0.f : expf(s_m[w][n] - mm);
+            const float f = (s_m[w][n] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(s_m[w][n] - mm);
             ll += s_l[w][n] * f;
             oo += s_o[w][n][d] * f;
         }
@@ -199,7 +210,7 @@ __global__ void attn_decode_merge_kernel(const float* __restrict__ part_o, const
         float ll = 0.f, oo = 0.f;
         for (int c = c0; c <= c1; ++c) {
             const float mc = part_ml[(base + c) * 2];
-            const float f = (mc == -INFINITY) ? 0.f : expf(mc - mm);
+            const float f = (mc == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mc - mm);
             ll += part_ml[(base + c) * 2 + 1] * f;
             oo += part_o[(base + c) * D + d] * f;
         }
@@ -212,11 +223,14 @@ static int launch_decode(const void* q, int q_stride, void* out, int out_stride,
                          const void* v_pool, const int* block_tables, int table_width, const int* context_lens,
                          float* part_o, float* part_ml, int max_chunks, int S, int H, int KVH, int page,
                          float scale, int window, hipStream_t stream) {
+    int page_shift = 0;
+    while ((1 << page_shift) < page) ++page_shift;
+    const float scale_log2 = scale * 1.4426950408889634f;
     dim3 grid(S, KVH, max_chunks);
     attn_decode_mfma_kernel<D><<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)k_pool,
                                                          (const bf16_t*)v_pool, block_tables, table_width,
-                                                         context_lens, part_o, part_ml, max_chunks, H, KVH, page,
-                                                         scale, window);
+                                                         context_lens, part_o, part_ml, max_chunks, H, KVH,
+                                                         page_shift, scale_log2, window);
     TM_CHECK_LAUNCH();
     attn_decode_merge_kernel<<<dim3(S, H), 64, 0, stream>>>(part_o, part_ml, context_lens, (bf16_t*)out, out_stride,
                                                             max_chunks, H, D, window);
@@ -231,7 +245,8 @@ extern "C" int tm_attn_decode_mfma(const void* q, int q_stride, void* out, int o
                                    const int* context_lens, float* part_o, float* part_ml, int max_chunks, int S,
                                    int H, int KVH, int D, int page, float scale, int window, hipStream_t stream) {
     if (S <= 0) return TM_OK;
-    if (H <= 0 || KVH <= 0 || H % KVH || H / KVH > 16 || page <= 0 || page % 16 || max_chunks <= 0 ||
+    if (H <= 0 || KVH <= 0 || H % KVH || H / KVH > 16 || page < 16 || (page & (page - 1)) || max_chunks <= 0 ||
+        !(scale > 0.f) ||
         max_chunks > 65535 || KVH > 65535 || window < 0 || table_width <= 0 || (q_stride % 8) ||
         ((uintptr_t)q % 16) || q_stride < H * D || out_stride < H * D)
         return TM_ERR_ARG;

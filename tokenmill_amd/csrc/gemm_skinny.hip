@@ -72,6 +72,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
                                                                  const void* __restrict__ bias, int bias_f32,
                                                                  TC* __restrict__ C, int ldc, int M, int N, int K) {
     constexpr int NACC = SILU ? 2 : 1;
+    // k-steps in flight per wavefront (fewer where 16 wavefronts share the register file)
+    constexpr int KCH = (WAVES > 4 && SILU && NT > 2) ? 4 : ((WAVES > 4 || NT > 2 || SILU) ? 8 : 16);
     __shared__ float red[SPLIT ? WAVES : 1][64][4 + 1];        // one accumulator tile at a time
     const int wave = threadIdx.x / TM_WAVE, lane = threadIdx.x % TM_WAVE;
     const int r = lane % 16, g = lane / 16;
@@ -102,17 +104,25 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
         for (int t = 0; t < NT; ++t) acc[a][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
     if (n0 < N) {
-#pragma unroll 4
-        for (int ks = ks0; ks < ks1; ++ks) {
-            const int k = ks * 32;
-            const Frag wf = load_frag(wrow, k, K - 8 * g, w_ok);
-            Frag uf;
-            if (SILU) uf = load_frag(urow, k, K - 8 * g, w_ok);
+        // KCH k-steps at a time with every load issued before the first product: a wavefront's whole
+        // K range is at most one or two such groups, so it waits for memory once or twice, not per step.
+        for (int base = ks0; base < ks1; base += KCH) {
+            Frag wf[KCH], uf[SILU ? KCH : 1];
 #pragma unroll
-            for (int t = 0; t < NT; ++t) {
-                const Frag af = load_frag(arow[t], k, K - 8 * g, a_ok[t]);
-                acc[0][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf.b, af.b, acc[0][t], 0, 0, 0);
-                if (SILU) acc[1][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf.b, af.b, acc[1][t], 0, 0, 0);
+            for (int j = 0; j < KCH; ++j) {
+                const bool in = base + j < ks1;
+                wf[j] = load_frag(wrow, (base + j) * 32, K - 8 * g, w_ok && in);
+                if (SILU) uf[j] = load_frag(urow, (base + j) * 32, K - 8 * g, w_ok && in);
+            }
+#pragma unroll
+            for (int j = 0; j < KCH; ++j) {
+                const bool in = base + j < ks1;
+#pragma unroll
+                for (int t = 0; t < NT; ++t) {
+                    const Frag af = load_frag(arow[t], (base + j) * 32, K - 8 * g, a_ok[t] && in);
+                    acc[0][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[j].b, af.b, acc[0][t], 0, 0, 0);
+                    if (SILU) acc[1][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[j].b, af.b, acc[1][t], 0, 0, 0);
+                }
             }
         }
     }

@@ -258,7 +258,8 @@ DECODE_CHUNK = 256          # keys per block of the split decode attention
 
 
 def attn_decode_mfma_supported(dtype, H: int, KVH: int, D: int, page: int) -> bool:
-    return dtype == torch.bfloat16 and D in (32, 64, 96, 128) and page % 16 == 0 and H % KVH == 0 and H // KVH <= 16
+    return (dtype == torch.bfloat16 and D in (32, 64, 96, 128) and page >= 16 and page & (page - 1) == 0
+            and H % KVH == 0 and H // KVH <= 16)
 
 
 def attn_decode_mfma(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
