@@ -446,3 +446,93 @@ def test_paged_attention_prefill_mfma(ops, H, KVH, D, page, window):
                       [(s, first + 77 + j, min(16, 123 - j), 77 + j) for j in range(0, 123, 16)], dtype=torch.int32)
     ops.attn_prefill_mfma(wide, out2, k_dev, v_dev, case["tables"].to(DEV), t2.to(DEV), H, KVH, D, scale, window)
     assert torch.equal(out2[first:first + 200], out[first:first + 200])
+
+
+# ----------------------------------------------------------------------------------------------- fused decode kernels
+
+@pytest.mark.parametrize("M,K,H,KVH,D,page", [(8, 896, 14, 2, 64, 16), (1, 192, 6, 1, 32, 16), (16, 3584, 4, 4, 128, 32),
+                                               (5, 120, 3, 1, 96, 64)])
+def test_fused_norm_qkv_rope(ops, M, K, H, KVH, D, page):
+    torch.manual_seed(13)
+    dt = torch.bfloat16
+    eps, theta, max_pos, pages = 1e-5, 1e6, 500, 9
+    rows = (H + 2 * KVH) * D
+    resid = torch.randn(M, K) * 2
+    nw, W, b = q(torch.rand(K) + 0.5, dt), q(torch.randn(rows, K) * 0.05, dt), q(torch.randn(rows) * 0.5, dt)
+    positions = torch.randint(0, max_pos, (M,), dtype=torch.int32)
+    slots = torch.randperm(pages * page)[:M].to(torch.int32)
+    if M > 2:
+        slots[1] = -1
+    # the unfused chain on the CPU
+    h = P.rms_norm(resid, nw, eps, dt)
+    qkv = P.linear(h, W, b, dt)
+    cos, sin = P.rope_tables(max_pos, D, theta)
+    qq = P.apply_rope(qkv[:, :H * D].view(M, H, D), cos, sin, positions.long(), dt)
+    kk = P.apply_rope(qkv[:, H * D:(H + KVH) * D].view(M, KVH, D), cos, sin, positions.long(), dt)
+    vv = qkv[:, (H + KVH) * D:].view(M, KVH, D)
+    half = cos[:, :D // 2].contiguous(), sin[:, :D // 2].contiguous()
+    kp = torch.full((pages, page, KVH, D), 7.0, dtype=dt, device=DEV)
+    vp = torch.full((pages, KVH, D, page), 7.0, dtype=dt, device=DEV)
+    q_out = torch.empty(M, H * D, dtype=dt, device=DEV)
+    r_dev = resid.to(DEV)
+    ops.fused_norm_qkv_rope(r_dev, nw.to(dt).to(DEV), eps, W.to(dt).to(DEV), b.to(dt).to(DEV), q_out, H, KVH, D,
+                            half[0].to(DEV), half[1].to(DEV), positions.to(DEV), slots.to(DEV), kp, vp)
+    assert torch.equal(r_dev.cpu(), resid)                              # the residual is only read
+    torch.testing.assert_close(q_out.float().cpu().view(M, H, D), qq, **tol(dt))
+    kflat = kp.float().cpu().view(-1, KVH, D)
+    vflat = vp.float().cpu().permute(0, 3, 1, 2).reshape(-1, KVH, D)
+    written = torch.zeros(pages * page, dtype=torch.bool)
+    for t in range(M):
+        if slots[t] >= 0:
+            written[slots[t]] = True
+            torch.testing.assert_close(kflat[slots[t]], kk[t], **tol(dt))
+            torch.testing.assert_close(vflat[slots[t]], vv[t], **tol(dt))
+    assert (kflat[~written] == 7.0).all() and (vflat[~written] == 7.0).all()
+    # a norm weight stored in 32-bit
+    nw32 = torch.rand(K) + 0.5
+    ops.fused_norm_qkv_rope(r_dev, nw32.to(DEV), eps, W.to(dt).to(DEV), None, q_out, H, KVH, D, half[0].to(DEV),
+                            half[1].to(DEV), positions.to(DEV), None, None, None)
+    normed = q(resid * torch.rsqrt((resid * resid).mean(-1, keepdim=True) + eps), dt)
+    qkv2 = P.linear(q(nw32 * normed, dt), W, None, dt)
+    qq2 = P.apply_rope(qkv2[:, :H * D].view(M, H, D), cos, sin, positions.long(), dt)
+    torch.testing.assert_close(q_out.float().cpu().view(M, H, D), qq2, **tol(dt))
+
+
+@pytest.mark.parametrize("M,K,I", [(8, 896, 4864), (1, 64, 128), (16, 192, 320), (3, 120, 200)])
+def test_fused_norm_gate_up_silu(ops, M, K, I):
+    torch.manual_seed(14)
+    dt = torch.bfloat16
+    eps = 1e-6
+    resid = torch.randn(M, K) * 3
+    nw, W = q(torch.rand(K) + 0.5, dt), q(torch.randn(2 * I, K) * 0.1, dt)
+    h = P.rms_norm(resid, nw, eps, dt)
+    gu = P.linear(h, W, None, dt)
+    want = P.silu_mul(gu[:, :I], gu[:, I:], dt)
+    out = torch.empty(M, I, dtype=dt, device=DEV)
+    ops.fused_norm_gate_up_silu(resid.to(DEV), nw.to(dt).to(DEV), eps, W.to(dt).to(DEV), out)
+    torch.testing.assert_close(out.float().cpu(), want, rtol=2e-2, atol=2e-2)
+    assert ((out.float().cpu() - want).abs() > 1e-2).float().mean() < 0.01
+
+
+@pytest.mark.parametrize("M,N,K", [(8, 896, 4864), (1, 64, 128), (40, 200, 120), (64, 896, 896)])
+def test_gemm_skinny_adds_into_the_residual(ops, M, N, K):
+    torch.manual_seed(15)
+    dt = torch.bfloat16
+    a, w, b = q(torch.randn(M, K), dt), q(torch.randn(N, K) * 0.1, dt), q(torch.randn(N), dt)
+    resid = torch.randn(M, N) * 5
+    acc = resid.to(DEV)
+    ops.gemm_skinny(a.to(dt).to(DEV), w.to(dt).to(DEV), b.to(dt).to(DEV), None, accum=acc)
+    out = torch.empty(M, N, dtype=dt, device=DEV)
+    ops.gemm_skinny(a.to(dt).to(DEV), w.to(dt).to(DEV), b.to(dt).to(DEV), out)
+    assert torch.equal(acc.cpu(), resid + out.float().cpu())            # the rounded product, added in 32-bit
+
+
+def test_argmax_over_a_wide_vocabulary(ops):
+    torch.manual_seed(16)
+    logits = torch.randn(70, 151936)
+    logits[5, 150000] = logits[5, 20] = 60.0                            # a tie across chunks: the first maximum
+    logits[6, :] = float("-inf")
+    logits[6, 151935] = -3.0
+    out = torch.empty(70, dtype=torch.int32, device=DEV)
+    ops.argmax_rows(logits.to(DEV), out)
+    assert out.cpu().tolist() == logits.argmax(-1).tolist() and out[5].item() == 20 and out[6].item() == 151935

@@ -29,18 +29,27 @@ int tm_attn_paged_generic(const void* q, int q_stride, void* out, int out_stride
                           int dtype, hipStream_t stream);
 
 int tm_gemm_skinny(const void* A, int lda, const void* W, const void* bias, int bias_dtype, void* C, int ldc, int M,
-                   int N, int K, int out_dtype, int silu, hipStream_t stream);
+                   int N, int K, int out_dtype, int silu, float* accum, int ldacc, hipStream_t stream);
 
 int tm_attn_decode_mfma(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
                         const void* v_pool, const int* block_tables, int table_width, const int* context_lens,
-                        float* part_o, float* part_ml, int max_chunks, int S, int H, int KVH, int D, int page,
-                        float scale, int window, hipStream_t stream);
+                        float* part_o, float* part_ml, int* counters, int max_chunks, int S, int H, int KVH, int D,
+                        int page, float scale, int window, hipStream_t stream);
+
+int tm_fused_norm_qkv_rope(const float* resid, const void* norm_w, int norm_w_dtype, float eps, int M, int K,
+                           const void* W, const void* bias, int bias_dtype, void* q_out, int H, int KVH, int D,
+                           const float* cos_t, const float* sin_t, const int* positions, const int* slots,
+                           void* k_pool, void* v_pool, int page, hipStream_t stream);
+
+int tm_fused_norm_gate_up_silu(const float* resid, const void* norm_w, int norm_w_dtype, float eps, int M, int K,
+                               const void* W, void* act_out, int I, hipStream_t stream);
 
 int tm_attn_prefill_mfma(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
                          const void* v_pool, const int* block_tables, int table_width, const int* tiles, int n_tiles,
                          int H, int KVH, int D, int page, float scale, int window, hipStream_t stream);
 
-int tm_argmax_rows(const float* logits, int R, int V, int* out, hipStream_t stream);
+int tm_argmax_work_chunks(int V);
+int tm_argmax_rows(const float* logits, int R, int V, int* out, float* work_v, int* work_i, hipStream_t stream);
 
 int tm_sample_rows(const float* logits, int R, int V, const float* temperature, const int* top_k,
                    const float* top_p, const float* u, int* out, hipStream_t stream);

@@ -5,9 +5,10 @@
 //   (the reference folds the group into query rows the same way: src/infer/model/layers.py:110-124).
 //   The context is cut into chunks of 256 positions, fixed by position alone; each block of four
 //   wavefronts takes one chunk of one (request, kv head), each wavefront 64 keys of it, and writes
-//   an unnormalised partial (max, sum, weighted values) in 32-bit; attn_decode_merge adds the
-//   partials of a request in ascending chunk order. What a request gets therefore does not depend
-//   on which other requests are in the batch.
+//   an unnormalised partial (max, sum, weighted values) in 32-bit. The block that finishes last for
+//   a (request, kv head) (a counter tells it) adds the partials in ascending chunk order and writes
+//   the result; the order of the sum is fixed, whichever block happens to do it. What a request
+//   gets therefore does not depend on which other requests are in the batch.
 //
 //   Operand layouts need no LDS: keys K[page][slot][kvh][d] give the A operand of S^T = K Q^T
 //   (16 keys x 32 d per instruction), values V[page][kvh][d][slot] give the A operand of
@@ -45,7 +46,8 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_pool,
     const bf16_t* __restrict__ v_pool, const int* __restrict__ block_tables, int table_width,
     const int* __restrict__ context_lens, float* __restrict__ part_o, float* __restrict__ part_ml,
-    int max_chunks, int H, int KVH, int page_shift, float scale_log2, int window) {
+    int* __restrict__ counters, bf16_t* __restrict__ out, int out_stride, int max_chunks, int H, int KVH,
+    int page_shift, float scale_log2, int window) {
     constexpr int NDC = D / 32;          // 32-wide d chunks of the q.k product
     constexpr int NDT = D / 16;          // 16-wide d tiles of the output
     __shared__ float s_m[4][16], s_l[4][16];
@@ -192,59 +194,66 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
             part_ml[slot * 2 + 1] = ll;
         }
     }
-}
-
-// out[s, h, :] = sum over the visible chunks (ascending) of partial values, normalised.
-__global__ void attn_decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                         const int* __restrict__ context_lens, bf16_t* __restrict__ out,
-                                         int out_stride, int max_chunks, int H, int D, int window) {
-    const int s = blockIdx.x, h = blockIdx.y;
-    const int ctx = context_lens[s];
-    const int p = ctx - 1;
-    const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+    // Is this the last block of its (request, kv head)? Its partial is published first (release),
+    // the counter is bumped, and the one that sees the full count reads the others' (acquire).
+    __shared__ int s_last;
     const int c0 = lo / AD_CHUNK, c1 = (ctx - 1) / AD_CHUNK;
-    const size_t base = ((size_t)s * H + h) * max_chunks;
-    float mm = -INFINITY;
-    for (int c = c0; c <= c1; ++c) mm = fmaxf(mm, part_ml[(base + c) * 2]);
-    for (int d = threadIdx.x; d < D; d += blockDim.x) {
+    __threadfence();
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int* cnt = counters + (size_t)s * KVH + kvh;
+        const int old = __hip_atomic_fetch_add(cnt, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        s_last = (old == c1 - c0);
+        if (s_last) __hip_atomic_store(cnt, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next call
+    }
+    __syncthreads();
+    if (!s_last) return;
+    __threadfence();
+    for (int idx = threadIdx.x; idx < G * D; idx += 256) {
+        const int n = idx / D, d = idx % D;
+        const size_t base = ((size_t)s * H + kvh * G + n) * max_chunks;
+        float mm = -INFINITY;
+        for (int c = c0; c <= c1; ++c)
+            mm = fmaxf(mm, __hip_atomic_load(part_ml + (base + c) * 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
         float ll = 0.f, oo = 0.f;
         for (int c = c0; c <= c1; ++c) {
-            const float mc = part_ml[(base + c) * 2];
+            const float mc = __hip_atomic_load(part_ml + (base + c) * 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             const float f = (mc == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mc - mm);
-            ll += part_ml[(base + c) * 2 + 1] * f;
-            oo += part_o[(base + c) * D + d] * f;
+            ll += __hip_atomic_load(part_ml + (base + c) * 2 + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * f;
+            oo += __hip_atomic_load(part_o + (base + c) * D + d, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * f;
         }
-        out[(size_t)s * out_stride + (size_t)h * D + d] = f32_to_bf16(oo / ll);
+        out[(size_t)s * out_stride + (size_t)(kvh * G + n) * D + d] = f32_to_bf16(oo / ll);
     }
 }
 
 template <int D>
 static int launch_decode(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
                          const void* v_pool, const int* block_tables, int table_width, const int* context_lens,
-                         float* part_o, float* part_ml, int max_chunks, int S, int H, int KVH, int page,
-                         float scale, int window, hipStream_t stream) {
+                         float* part_o, float* part_ml, int* counters, int max_chunks, int S, int H, int KVH,
+                         int page, float scale, int window, hipStream_t stream) {
     int page_shift = 0;
     while ((1 << page_shift) < page) ++page_shift;
     const float scale_log2 = scale * 1.4426950408889634f;
     dim3 grid(S, KVH, max_chunks);
     attn_decode_mfma_kernel<D><<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)k_pool,
                                                          (const bf16_t*)v_pool, block_tables, table_width,
-                                                         context_lens, part_o, part_ml, max_chunks, H, KVH,
-                                                         page_shift, scale_log2, window);
-    TM_CHECK_LAUNCH();
-    attn_decode_merge_kernel<<<dim3(S, H), 64, 0, stream>>>(part_o, part_ml, context_lens, (bf16_t*)out, out_stride,
-                                                            max_chunks, H, D, window);
+                                                         context_lens, part_o, part_ml, counters, (bf16_t*)out,
+                                                         out_stride, max_chunks, H, KVH, page_shift, scale_log2,
+                                                         window);
     TM_CHECK_LAUNCH();
     return TM_OK;
 }
 
 // q: first decode row (one row per request, rows q_stride apart); out likewise; block_tables and
-// context_lens: first decode request. part_o: float [S, H, max_chunks, D]; part_ml: [S, H, max_chunks, 2].
+// context_lens: first decode request. part_o: float [S, H, max_chunks, D]; part_ml: [S, H, max_chunks, 2];
+// counters: int [S * KVH], all zero on entry (and again on exit). Calls that share counters must not overlap.
 extern "C" int tm_attn_decode_mfma(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
                                    const void* v_pool, const int* block_tables, int table_width,
-                                   const int* context_lens, float* part_o, float* part_ml, int max_chunks, int S,
-                                   int H, int KVH, int D, int page, float scale, int window, hipStream_t stream) {
+                                   const int* context_lens, float* part_o, float* part_ml, int* counters,
+                                   int max_chunks, int S, int H, int KVH, int D, int page, float scale, int window,
+                                   hipStream_t stream) {
     if (S <= 0) return TM_OK;
+    if (!counters) return TM_ERR_ARG;
     if (H <= 0 || KVH <= 0 || H % KVH || H / KVH > 16 || page < 16 || (page & (page - 1)) || max_chunks <= 0 ||
         !(scale > 0.f) ||
         max_chunks > 65535 || KVH > 65535 || window < 0 || table_width <= 0 || (q_stride % 8) ||
@@ -253,7 +262,7 @@ extern "C" int tm_attn_decode_mfma(const void* q, int q_stride, void* out, int o
 #define TM_DECODE_CASE(DD)                                                                                        \
     case DD:                                                                                                      \
         return launch_decode<DD>(q, q_stride, out, out_stride, k_pool, v_pool, block_tables, table_width,         \
-                                 context_lens, part_o, part_ml, max_chunks, S, H, KVH, page, scale, window, stream)
+                                 context_lens, part_o, part_ml, counters, max_chunks, S, H, KVH, page, scale, window, stream)
     switch (D) {
         TM_DECODE_CASE(32);
         TM_DECODE_CASE(64);

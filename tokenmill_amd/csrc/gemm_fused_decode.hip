@@ -1,0 +1,300 @@
+// Decode-step products with the RMSNorm in front and the layer's own epilogue behind, for at most 16
+// tokens (bfloat16 weights and activations, 32-bit residual stream and sums).
+//
+//   x = weight * round(resid * rsqrt(mean(resid^2) + eps))     (reference src/infer/model/layers.py:41-44)
+//   is computed by every block into LDS (a few KB of L2 reads against a matrix streamed from HBM), then
+//
+//   QKV epilogue  : y = x Wqkv^T + b; q and k rotated by their token's position; q to a dense
+//                   [M, H*D] buffer, k and v straight to their cache slots
+//                   (reference src/infer/model/layers.py:142-147,60-64; src/infer/kv/paged_cache.py:40-43)
+//   SiLU epilogue : act = silu(x Wgate^T) * (x Wup^T)          (reference src/infer/model/layers.py:163-164)
+//
+// A block owns two strips of 16 matrix rows whose results meet in the epilogue (the two halves of a
+// rotary pair; gate and up). Its four wavefronts split K; partial sums are added through LDS in
+// wavefront order. Everything is rounded where the unfused path stores a bfloat16 tensor, so both
+// paths agree up to the order of 32-bit sums.
+#include "common.h"
+#include "api.h"
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+union FFrag {
+    u32x4_t u;
+    bf16x8_t b;
+};
+
+__device__ __forceinline__ uint32_t fd_pack(float a, float b) {
+    const bf16x2_t v = __builtin_convertvector(f32x2_t{a, b}, bf16x2_t);
+    return *(const uint32_t*)&v;
+}
+
+__device__ __forceinline__ float fd_round(float a) { return bf16_to_f32(f32_to_bf16(a)); }
+
+#define FD_EPI_QKV 0
+#define FD_EPI_SILU 1
+#define FD_KCH 8            // k-steps whose matrix loads are in flight at once, per wavefront
+#define FD_XPAD 8           // padding of an LDS row of x, in elements
+
+struct FusedArgs {
+    // norm + product
+    const float* resid;     // [M, K]
+    const void* norm_w;     // [K]
+    int norm_w_f32;
+    float eps;
+    int M, K;
+    const bf16_t* W;        // [rows, K]
+    const void* bias;       // [rows] or null
+    int bias_f32;
+    // QKV epilogue
+    bf16_t* q_out;          // [M, H*D]
+    int H, KVH, D;
+    const float* cos_t;     // [max_pos, D/2]
+    const float* sin_t;
+    const int* positions;   // [M]
+    const int* slots;       // [M]; < 0: not stored
+    bf16_t* k_pool;         // [pages, page, KVH, D]
+    bf16_t* v_pool;         // [pages, KVH, D, page]
+    int page_shift;
+    // SiLU epilogue
+    bf16_t* act_out;        // [M, I]
+    int I;
+};
+
+template <int EPI>
+__global__ __launch_bounds__(256) void fused_norm_gemm_kernel(const FusedArgs a) {
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    bf16_t* xs = (bf16_t*)smem_raw;                                  // [16][K + FD_XPAD]
+    __shared__ float red[4][2][64][4 + 1];
+    const int K = a.K, M = a.M;
+    const int xstride = K + FD_XPAD;
+    const int wave = threadIdx.x / TM_WAVE, lane = threadIdx.x % TM_WAVE;
+    const int r = lane % 16, g = lane / 16;
+    const int u = blockIdx.x;
+
+    // the two strips of this block
+    int nA, nB, head = 0, jt = 0;
+    bool rows_ok = true;
+    if (EPI == FD_EPI_QKV) {
+        const int per_head = a.D / 32;
+        head = u / per_head;
+        jt = u % per_head;
+        if (head < a.H + a.KVH) {
+            nA = head * a.D + 16 * jt;
+            nB = nA + a.D / 2;
+        } else {
+            nA = head * a.D + 32 * jt;
+            nB = nA + 16;
+        }
+    } else {
+        nA = 16 * u;
+        nB = a.I + 16 * u;
+        rows_ok = nA + r < a.I;
+    }
+
+    // matrix loads of the first group go out before the norm is computed
+    const int ksteps = (K + 31) / 32;
+    const int per = (ksteps + 3) / 4;
+    const int ks0 = wave * per;
+    const int ks1 = ks0 + per < ksteps ? ks0 + per : ksteps;
+    const bf16_t* wA = a.W + (size_t)(nA + r) * K + 8 * g;
+    const bf16_t* wB = a.W + (size_t)(nB + r) * K + 8 * g;
+    FFrag fa[FD_KCH], fb[FD_KCH];
+#pragma unroll
+    for (int j = 0; j < FD_KCH; ++j) {
+        const int k = (ks0 + j) * 32;
+        const bool in = rows_ok && ks0 + j < ks1 && k + 8 * g < K;
+        fa[j].u = in ? *(const u32x4_t*)(wA + k) : u32x4_t{0, 0, 0, 0};
+        fb[j].u = in ? *(const u32x4_t*)(wB + k) : u32x4_t{0, 0, 0, 0};
+    }
+
+    // x = norm(resid) into LDS: 16 threads per token
+    {
+        const int row = threadIdx.x / 16, sub = threadIdx.x % 16;
+        bf16_t* xrow = xs + (size_t)row * xstride;
+        if (row < M) {
+            const float* src = a.resid + (size_t)row * K;
+            float ss = 0.f;
+            for (int c = sub * 4; c < K; c += 64) {
+                const f32x4_t v = *(const f32x4_t*)(src + c);
+                ss += v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
+            }
+            ss += __shfl_xor(ss, 1, TM_WAVE);
+            ss += __shfl_xor(ss, 2, TM_WAVE);
+            ss += __shfl_xor(ss, 4, TM_WAVE);
+            ss += __shfl_xor(ss, 8, TM_WAVE);
+            const float rs = rsqrtf(ss / (float)K + a.eps);
+            for (int c = sub * 4; c < K; c += 64) {
+                const f32x4_t v = *(const f32x4_t*)(src + c);
+                float w[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    w[i] = a.norm_w_f32 ? ((const float*)a.norm_w)[c + i] : bf16_to_f32(((const bf16_t*)a.norm_w)[c + i]);
+                uint2 pk;
+                pk.x = fd_pack(w[0] * fd_round(v[0] * rs), w[1] * fd_round(v[1] * rs));
+                pk.y = fd_pack(w[2] * fd_round(v[2] * rs), w[3] * fd_round(v[3] * rs));
+                *(uint2*)(xrow + c) = pk;
+            }
+        } else {
+            for (int c = sub * 4; c < K; c += 64) *(uint2*)(xrow + c) = uint2{0u, 0u};
+        }
+    }
+    __syncthreads();
+
+    f32x4_t accA = {0.f, 0.f, 0.f, 0.f}, accB = {0.f, 0.f, 0.f, 0.f};
+    const bf16_t* xr = xs + (size_t)r * xstride + 8 * g;
+    for (int base = ks0; base < ks1; base += FD_KCH) {
+        if (base != ks0) {
+#pragma unroll
+            for (int j = 0; j < FD_KCH; ++j) {
+                const int k = (base + j) * 32;
+                const bool in = rows_ok && base + j < ks1 && k + 8 * g < K;
+                fa[j].u = in ? *(const u32x4_t*)(wA + k) : u32x4_t{0, 0, 0, 0};
+                fb[j].u = in ? *(const u32x4_t*)(wB + k) : u32x4_t{0, 0, 0, 0};
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < FD_KCH; ++j) {
+            const int k = (base + j) * 32;
+            FFrag xf;
+            xf.u = (base + j < ks1 && k + 8 * g < K) ? *(const u32x4_t*)(xr + k) : u32x4_t{0, 0, 0, 0};
+            accA = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[j].b, xf.b, accA, 0, 0, 0);
+            accB = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb[j].b, xf.b, accB, 0, 0, 0);
+        }
+    }
+    // partial sums of the four wavefronts, added in wavefront order
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        red[wave][0][lane][i] = accA[i];
+        red[wave][1][lane][i] = accB[i];
+    }
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        accA[i] = red[0][0][lane][i] + red[1][0][lane][i] + red[2][0][lane][i] + red[3][0][lane][i];
+        accB[i] = red[0][1][lane][i] + red[1][1][lane][i] + red[2][1][lane][i] + red[3][1][lane][i];
+    }
+
+    // lane: token r, rows nA + 4g + i and nB + 4g + i
+    const int tok = r;
+    if (tok >= M) return;
+    if (EPI == FD_EPI_SILU) {
+        const int col = 16 * u + 4 * g;
+        if (col >= a.I) return;
+        float v[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float gt = fd_round(accA[i]), up = fd_round(accB[i]);
+            v[i] = gt / (1.f + expf(-gt)) * up;
+        }
+        bf16_t* dst = a.act_out + (size_t)tok * a.I + col;
+        if (col + 4 <= a.I) {
+            *(uint2*)dst = uint2{fd_pack(v[0], v[1]), fd_pack(v[2], v[3])};
+        } else {
+            for (int i = 0; i < 4 && col + i < a.I; ++i) dst[i] = f32_to_bf16(v[i]);
+        }
+        return;
+    }
+    float xA[4], xB[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        float bA = 0.f, bB = 0.f;
+        if (a.bias) {
+            bA = a.bias_f32 ? ((const float*)a.bias)[nA + 4 * g + i] : bf16_to_f32(((const bf16_t*)a.bias)[nA + 4 * g + i]);
+            bB = a.bias_f32 ? ((const float*)a.bias)[nB + 4 * g + i] : bf16_to_f32(((const bf16_t*)a.bias)[nB + 4 * g + i]);
+        }
+        xA[i] = fd_round(accA[i] + bA);
+        xB[i] = fd_round(accB[i] + bB);
+    }
+    const int slot = a.slots ? a.slots[tok] : -1;
+    if (head < a.H + a.KVH) {
+        const int half = a.D / 2;
+        const int j0 = 16 * jt + 4 * g;                              // pair index of element 0
+        const float* c = a.cos_t + (size_t)a.positions[tok] * half + j0;
+        const float* s = a.sin_t + (size_t)a.positions[tok] * half + j0;
+        float y1[4], y2[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            y1[i] = xA[i] * c[i] - xB[i] * s[i];
+            y2[i] = xB[i] * c[i] + xA[i] * s[i];
+        }
+        bf16_t* dst = nullptr;
+        if (head < a.H)
+            dst = a.q_out + (size_t)tok * a.H * a.D + (size_t)head * a.D + j0;
+        else if (slot >= 0)
+            dst = a.k_pool + ((size_t)slot * a.KVH + (head - a.H)) * a.D + j0;
+        if (dst) {
+            *(uint2*)dst = uint2{fd_pack(y1[0], y1[1]), fd_pack(y1[2], y1[3])};
+            *(uint2*)(dst + half) = uint2{fd_pack(y2[0], y2[1]), fd_pack(y2[2], y2[3])};
+        }
+    } else if (slot >= 0) {
+        const int vh = head - a.H - a.KVH;
+        const int pg = slot >> a.page_shift, in_page = slot & ((1 << a.page_shift) - 1);
+        const int d0 = 32 * jt + 4 * g;
+        bf16_t* dst = a.v_pool + ((((size_t)pg * a.KVH + vh) * a.D + d0) << a.page_shift) + in_page;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            dst[(size_t)i << a.page_shift] = f32_to_bf16(xA[i]);
+            dst[(size_t)(i + 16) << a.page_shift] = f32_to_bf16(xB[i]);
+        }
+    }
+}
+
+static int fused_lds_bytes(int K) { return 16 * (K + FD_XPAD) * (int)sizeof(bf16_t); }
+
+template <int EPI>
+static int launch_fused(const FusedArgs& a, int blocks, hipStream_t stream) {
+    const int lds = fused_lds_bytes(a.K);
+    if (lds + 6 * 1024 > 160 * 1024) return TM_ERR_ARG;
+    static int raised = 0;          // largest dynamic LDS size this kernel has been allowed so far
+    if (lds > 48 * 1024 && lds > raised) {
+        if (hipFuncSetAttribute((const void*)fused_norm_gemm_kernel<EPI>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                lds) != hipSuccess)
+            return TM_ERR_LAUNCH;
+        raised = lds;
+    }
+    fused_norm_gemm_kernel<EPI><<<blocks, 256, lds, stream>>>(a);
+    TM_CHECK_LAUNCH();
+    return TM_OK;
+}
+
+static bool fused_common_ok(int M, int K, const void* resid, const void* W) {
+    return M > 0 && M <= 16 && K > 0 && K % 8 == 0 && ((uintptr_t)resid % 16) == 0 && ((uintptr_t)W % 16) == 0;
+}
+
+// q_out[M, H*D], K cache, V cache <- rope(norm(resid) Wqkv^T + b).  Needs M <= 16, D % 32 == 0, a
+// rotary table over the whole head, page a power of two.
+extern "C" int tm_fused_norm_qkv_rope(const float* resid, const void* norm_w, int norm_w_dtype, float eps, int M,
+                                      int K, const void* W, const void* bias, int bias_dtype, void* q_out, int H,
+                                      int KVH, int D, const float* cos_t, const float* sin_t, const int* positions,
+                                      const int* slots, void* k_pool, void* v_pool, int page, hipStream_t stream) {
+    if (M == 0) return TM_OK;
+    if (!fused_common_ok(M, K, resid, W) || H <= 0 || KVH <= 0 || D <= 0 || D % 32 || !cos_t || !sin_t || !positions ||
+        !q_out || ((uintptr_t)q_out % 8) || page <= 0 || (page & (page - 1)) || !(eps > 0.f))
+        return TM_ERR_ARG;
+    if (slots && (!k_pool || !v_pool)) return TM_ERR_ARG;
+    FusedArgs a{};
+    a.resid = resid; a.norm_w = norm_w; a.norm_w_f32 = norm_w_dtype == TM_F32; a.eps = eps; a.M = M; a.K = K;
+    a.W = (const bf16_t*)W; a.bias = bias; a.bias_f32 = bias_dtype == TM_F32;
+    a.q_out = (bf16_t*)q_out; a.H = H; a.KVH = KVH; a.D = D; a.cos_t = cos_t; a.sin_t = sin_t;
+    a.positions = positions; a.slots = slots; a.k_pool = (bf16_t*)k_pool; a.v_pool = (bf16_t*)v_pool;
+    a.page_shift = 0;
+    while ((1 << a.page_shift) < page) ++a.page_shift;
+    return launch_fused<FD_EPI_QKV>(a, (H + 2 * KVH) * (D / 32), stream);
+}
+
+// act[M, I] <- silu(norm(resid) Wg^T) * (norm(resid) Wu^T), W = [Wg; Wu] [2I, K].  Needs M <= 16.
+extern "C" int tm_fused_norm_gate_up_silu(const float* resid, const void* norm_w, int norm_w_dtype, float eps, int M,
+                                          int K, const void* W, void* act_out, int I, hipStream_t stream) {
+    if (M == 0) return TM_OK;
+    if (!fused_common_ok(M, K, resid, W) || I <= 0 || !act_out || ((uintptr_t)act_out % 8) || (I % 4) || !(eps > 0.f))
+        return TM_ERR_ARG;
+    FusedArgs a{};
+    a.resid = resid; a.norm_w = norm_w; a.norm_w_f32 = norm_w_dtype == TM_F32; a.eps = eps; a.M = M; a.K = K;
+    a.W = (const bf16_t*)W; a.act_out = (bf16_t*)act_out; a.I = I;
+    return launch_fused<FD_EPI_SILU>(a, (I + 15) / 16, stream);
+}

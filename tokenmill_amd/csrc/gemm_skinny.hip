@@ -70,7 +70,8 @@ template <int NT, int WAVES, bool SPLIT, bool SILU, typename TC>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ A, int lda,
                                                                  const bf16_t* __restrict__ W,
                                                                  const void* __restrict__ bias, int bias_f32,
-                                                                 TC* __restrict__ C, int ldc, int M, int N, int K) {
+                                                                 TC* __restrict__ C, int ldc, int M, int N, int K,
+                                                                 float* __restrict__ accum, int ldacc) {
     constexpr int NACC = SILU ? 2 : 1;
     // k-steps in flight per wavefront (fewer where 16 wavefronts share the register file)
     constexpr int KCH = (WAVES > 4 && SILU && NT > 2) ? 4 : ((WAVES > 4 || NT > 2 || SILU) ? 8 : 16);
@@ -165,23 +166,28 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
             }
             v[i] = x;
         }
-        store4<TC>(C + (size_t)tok * ldc + nf, v, N - nf);
+        if (accum) {            // the rounded result goes into the 32-bit residual stream (each element has one owner)
+            float* dst = accum + (size_t)tok * ldacc + nf;
+            for (int i = 0; i < 4 && nf + i < N; ++i) dst[i] += bf16_to_f32(f32_to_bf16(v[i]));
+        } else {
+            store4<TC>(C + (size_t)tok * ldc + nf, v, N - nf);
+        }
     }
 }
 
 template <int NT, bool SILU, typename TC>
 static int launch_skinny(const void* A, int lda, const void* W, const void* bias, int bias_f32, void* C, int ldc,
-                         int M, int N, int K, hipStream_t stream) {
+                         int M, int N, int K, float* accum, int ldacc, hipStream_t stream) {
     const int strips = (N + 15) / 16;
     if (strips >= 2048) {                      // many rows: a strip per wavefront
         gemm_skinny_kernel<NT, 4, false, SILU, TC><<<(strips + 3) / 4, 256, 0, stream>>>(
-            (const bf16_t*)A, lda, (const bf16_t*)W, bias, bias_f32, (TC*)C, ldc, M, N, K);
+            (const bf16_t*)A, lda, (const bf16_t*)W, bias, bias_f32, (TC*)C, ldc, M, N, K, accum, ldacc);
     } else if (strips >= 256 || K < 2048) {    // a block of 4 wavefronts per strip
         gemm_skinny_kernel<NT, 4, true, SILU, TC><<<strips, 256, 0, stream>>>(
-            (const bf16_t*)A, lda, (const bf16_t*)W, bias, bias_f32, (TC*)C, ldc, M, N, K);
+            (const bf16_t*)A, lda, (const bf16_t*)W, bias, bias_f32, (TC*)C, ldc, M, N, K, accum, ldacc);
     } else {                                   // few rows, long K: 16 wavefronts per strip
         gemm_skinny_kernel<NT, 16, true, SILU, TC><<<strips, 1024, 0, stream>>>(
-            (const bf16_t*)A, lda, (const bf16_t*)W, bias, bias_f32, (TC*)C, ldc, M, N, K);
+            (const bf16_t*)A, lda, (const bf16_t*)W, bias, bias_f32, (TC*)C, ldc, M, N, K, accum, ldacc);
     }
     TM_CHECK_LAUNCH();
     return TM_OK;
@@ -189,30 +195,35 @@ static int launch_skinny(const void* A, int lda, const void* W, const void* bias
 
 template <bool SILU, typename TC>
 static int launch_skinny_nt(const void* A, int lda, const void* W, const void* bias, int bias_f32, void* C, int ldc,
-                            int M, int N, int K, hipStream_t stream) {
+                            int M, int N, int K, float* accum, int ldacc, hipStream_t stream) {
     switch ((M + 15) / 16) {
-        case 1: return launch_skinny<1, SILU, TC>(A, lda, W, bias, bias_f32, C, ldc, M, N, K, stream);
-        case 2: return launch_skinny<2, SILU, TC>(A, lda, W, bias, bias_f32, C, ldc, M, N, K, stream);
-        case 3: return launch_skinny<3, SILU, TC>(A, lda, W, bias, bias_f32, C, ldc, M, N, K, stream);
-        case 4: return launch_skinny<4, SILU, TC>(A, lda, W, bias, bias_f32, C, ldc, M, N, K, stream);
+        case 1: return launch_skinny<1, SILU, TC>(A, lda, W, bias, bias_f32, C, ldc, M, N, K, accum, ldacc, stream);
+        case 2: return launch_skinny<2, SILU, TC>(A, lda, W, bias, bias_f32, C, ldc, M, N, K, accum, ldacc, stream);
+        case 3: return launch_skinny<3, SILU, TC>(A, lda, W, bias, bias_f32, C, ldc, M, N, K, accum, ldacc, stream);
+        case 4: return launch_skinny<4, SILU, TC>(A, lda, W, bias, bias_f32, C, ldc, M, N, K, accum, ldacc, stream);
         default: return TM_ERR_ARG;
     }
 }
 
 // silu == 0: C[M, N] = A W^T + bias, W [N, K].   silu == 1: C[M, N] = silu(A Wg^T) * (A Wu^T), W = [Wg; Wu] [2N, K].
 // A, W bfloat16; C bfloat16 (out_dtype 1) or float32 (0); bias bfloat16 or float32 or null.
+// accum != null: nothing is stored to C; the bfloat16-rounded result is added to accum[M, N] (float32, row
+// stride ldacc) instead: the residual add of the layer, done by the product that feeds it.
 // Needs M <= 64, K % 8 == 0, lda % 8 == 0 and 16-byte aligned A and W.
 extern "C" int tm_gemm_skinny(const void* A, int lda, const void* W, const void* bias, int bias_dtype, void* C,
-                              int ldc, int M, int N, int K, int out_dtype, int silu, hipStream_t stream) {
+                              int ldc, int M, int N, int K, int out_dtype, int silu, float* accum, int ldacc,
+                              hipStream_t stream) {
     if (M <= 0 || N <= 0) return TM_OK;
+    if (accum && (silu || ldacc < N)) return TM_ERR_ARG;
+    if (!accum && !C) return TM_ERR_ARG;
     if (M > 64 || K <= 0 || (K % 8) || (lda % 8) || lda < K || ldc < N || ((uintptr_t)A % 16) || ((uintptr_t)W % 16))
         return TM_ERR_ARG;
     if (silu && bias) return TM_ERR_ARG;
     const int bias_f32 = bias_dtype == TM_F32;
     if (out_dtype == TM_BF16)
-        return silu ? launch_skinny_nt<true, bf16_t>(A, lda, W, bias, bias_f32, C, ldc, M, N, K, stream)
-                    : launch_skinny_nt<false, bf16_t>(A, lda, W, bias, bias_f32, C, ldc, M, N, K, stream);
+        return silu ? launch_skinny_nt<true, bf16_t>(A, lda, W, bias, bias_f32, C, ldc, M, N, K, accum, ldacc, stream)
+                    : launch_skinny_nt<false, bf16_t>(A, lda, W, bias, bias_f32, C, ldc, M, N, K, accum, ldacc, stream);
     if (out_dtype == TM_F32 && !silu)
-        return launch_skinny_nt<false, float>(A, lda, W, bias, bias_f32, C, ldc, M, N, K, stream);
+        return launch_skinny_nt<false, float>(A, lda, W, bias, bias_f32, C, ldc, M, N, K, accum, ldacc, stream);
     return TM_ERR_ARG;
 }

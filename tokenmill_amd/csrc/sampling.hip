@@ -56,10 +56,71 @@ __global__ __launch_bounds__(SM_NT) void argmax_rows_kernel(const float* __restr
     if (threadIdx.x == 0) out[blockIdx.x] = r.i;
 }
 
-extern "C" int tm_argmax_rows(const float* logits, int R, int V, int* out, hipStream_t stream) {
+// Two stages for wide vocabularies: a row is cut into NB chunks, one block each, then the NB
+// candidates are reduced. Ties go to the lower index in both stages (the first maximum).
+#define AM_NT 256
+__global__ __launch_bounds__(AM_NT) void argmax_partial_kernel(const float* __restrict__ logits, int V, int chunk,
+                                                               float* __restrict__ part_v, int* __restrict__ part_i) {
+    __shared__ ArgMax smem[AM_NT / TM_WAVE];
+    const int row = blockIdx.x, c = blockIdx.y, NB = gridDim.y;
+    const int lo = c * chunk, hi = lo + chunk < V ? lo + chunk : V;
+    const float* src = logits + (size_t)row * V;
+    ArgMax best{-INFINITY, -1};
+    for (int i = lo + threadIdx.x; i < hi; i += AM_NT) {
+        const float v = src[i];
+        if (v == v) best = better(best, ArgMax{v, i});
+    }
+#pragma unroll
+    for (int off = TM_WAVE / 2; off > 0; off >>= 1) {
+        ArgMax o{__shfl_xor(best.v, off, TM_WAVE), __shfl_xor(best.i, off, TM_WAVE)};
+        best = better(best, o);
+    }
+    const int wave = threadIdx.x / TM_WAVE, lane = threadIdx.x % TM_WAVE;
+    if (lane == 0) smem[wave] = best;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        ArgMax r = smem[0];
+        for (int w = 1; w < AM_NT / TM_WAVE; ++w) r = better(r, smem[w]);
+        part_v[(size_t)row * NB + c] = r.v;
+        part_i[(size_t)row * NB + c] = r.i;
+    }
+}
+
+__global__ __launch_bounds__(TM_WAVE) void argmax_final_kernel(const float* __restrict__ part_v,
+                                                               const int* __restrict__ part_i, int NB,
+                                                               int* __restrict__ out) {
+    const int row = blockIdx.x;
+    ArgMax best{-INFINITY, -1};
+    for (int c = threadIdx.x; c < NB; c += TM_WAVE)
+        best = better(best, ArgMax{part_v[(size_t)row * NB + c], part_i[(size_t)row * NB + c]});
+#pragma unroll
+    for (int off = TM_WAVE / 2; off > 0; off >>= 1) {
+        ArgMax o{__shfl_xor(best.v, off, TM_WAVE), __shfl_xor(best.i, off, TM_WAVE)};
+        best = better(best, o);
+    }
+    if (threadIdx.x == 0) out[row] = best.i < 0 ? 0 : best.i;
+}
+
+// work: at least R * tm_argmax_work_chunks(V) floats and as many ints (may be null when that is 1 chunk)
+extern "C" int tm_argmax_work_chunks(int V) {
+    int nb = (V + 4095) / 4096;
+    return nb < 1 ? 1 : (nb > 256 ? 256 : nb);
+}
+
+extern "C" int tm_argmax_rows(const float* logits, int R, int V, int* out, float* work_v, int* work_i,
+                              hipStream_t stream) {
     if (R <= 0) return TM_OK;
     if (V <= 0) return TM_ERR_ARG;
-    argmax_rows_kernel<<<R, SM_NT, 0, stream>>>(logits, V, out);
+    const int NB = tm_argmax_work_chunks(V);
+    if (NB == 1 || !work_v || !work_i) {
+        argmax_rows_kernel<<<R, SM_NT, 0, stream>>>(logits, V, out);
+        TM_CHECK_LAUNCH();
+        return TM_OK;
+    }
+    const int chunk = (V + NB - 1) / NB;
+    argmax_partial_kernel<<<dim3(R, NB), AM_NT, 0, stream>>>(logits, V, chunk, work_v, work_i);
+    TM_CHECK_LAUNCH();
+    argmax_final_kernel<<<R, TM_WAVE, 0, stream>>>(work_v, work_i, NB, out);
     TM_CHECK_LAUNCH();
     return TM_OK;
 }

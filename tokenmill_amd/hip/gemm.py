@@ -50,3 +50,19 @@ def gate_up_silu(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor) ->
         ops.gemm_skinny(x, w_gate_up, None, out, silu=True)
         return True
     return False
+
+
+def linear_accumulate(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, accum: torch.Tensor) -> bool:
+    """accum[M, N] (float32) += round_bf16(x @ w^T + bias) in the product's epilogue, if a kernel does that
+    for this shape."""
+    if 0 < x.shape[0] <= SKINNY_ROWS and _skinny_ok(x, w):
+        ops.gemm_skinny(x, w, bias, None, accum=accum)
+        return True
+    return False
+
+
+def fused_decode_ok(resid: torch.Tensor, w: torch.Tensor) -> bool:
+    """Can the norm-fused decode products take this residual and matrix?"""
+    M, K = resid.shape
+    return (0 < M <= ops.FUSED_DECODE_ROWS and w.dtype == torch.bfloat16 and K % 8 == 0 and ops.fused_lds_fits(K)
+            and resid.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)

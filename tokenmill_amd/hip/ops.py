@@ -207,7 +207,13 @@ def argmax_rows(logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     R, V = logits.shape
     _need(logits.dtype == torch.float32 and logits.is_contiguous(), "argmax: logits must be contiguous float32 [R, V]")
     _ints(out, R, "out")
-    _check(library().tm_argmax_rows(_p(logits), c_int(R), c_int(V), _p(out), _stream()), "argmax_rows")
+    nb = library().tm_argmax_work_chunks(c_int(V))
+    work_v = work_i = None
+    if nb > 1:                                   # a wide vocabulary: every row is cut over nb blocks
+        work_v = torch.empty(R * nb, dtype=torch.float32, device=logits.device)
+        work_i = torch.empty(R * nb, dtype=torch.int32, device=logits.device)
+    _check(library().tm_argmax_rows(_p(logits), c_int(R), c_int(V), _p(out), _p(work_v), _p(work_i), _stream()),
+           "argmax_rows")
     return out
 
 
@@ -227,13 +233,31 @@ def sample_rows(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Te
     return out
 
 
-def gemm_skinny(a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, out: torch.Tensor,
-                silu: bool = False) -> torch.Tensor:
+def gemm_skinny(a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, out: torch.Tensor | None,
+                silu: bool = False, accum: torch.Tensor | None = None) -> torch.Tensor:
     """MFMA product for at most 64 rows of bfloat16 activations: out[M, N] = a @ w^T (+ bias), or with
     ``silu`` out[M, N] = silu(a @ w[:N]^T) * (a @ w[N:]^T) for a stacked [gate; up] matrix w [2N, K].
-    out is bfloat16 or float32 (float32 not with silu)."""
-    _gpu(a, w, bias, out)
+    out is bfloat16 or float32 (float32 not with silu). With ``accum`` (float32 [M, N]) nothing is
+    stored to out: the result, rounded to bfloat16, is added into accum (the residual stream)."""
+    _gpu(a, w, bias, out, accum)
     M, K = a.shape
+    if accum is not None:
+        _need(out is None and not silu and accum.dtype == torch.float32 and accum.dim() == 2 and accum.shape[0] == M
+              and accum.stride(1) == 1, "gemm_skinny: accum must be float32 [M, N], and excludes out and silu")
+        N = accum.shape[1]
+        _need(tuple(w.shape) == (N, K) and w.is_contiguous() and a.dtype == w.dtype == torch.bfloat16 and 0 < M <= 64
+              and a.stride(1) == 1, "gemm_skinny: bfloat16 a [M<=64, K], contiguous w [N, K]")
+        lda = a.stride(0) if M > 1 else max(K, a.stride(0))
+        _need(K % 8 == 0 and lda % 8 == 0 and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0,
+              "gemm_skinny: K and the row stride must be multiples of 8 and the operands 16-byte aligned")
+        if bias is not None:
+            _need(tuple(bias.shape) == (N,) and bias.is_contiguous(), "gemm_skinny: bias must be [N]")
+        ldacc = accum.stride(0) if M > 1 else max(N, accum.stride(0))
+        _check(library().tm_gemm_skinny(_p(a), c_int(lda), _p(w), _p(bias),
+                                        c_int(code(bias.dtype) if bias is not None else -1), _p(None), c_int(N),
+                                        c_int(M), c_int(N), c_int(K), c_int(BF16), c_int(0), _p(accum), c_int(ldacc),
+                                        _stream()), "gemm_skinny")
+        return accum
     N = out.shape[1]
     _need(a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_skinny: bfloat16 inputs")
     _need(0 < M <= 64, f"gemm_skinny: at most 64 rows, got {M}")
@@ -250,11 +274,22 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, out
     _check(library().tm_gemm_skinny(_p(a), c_int(lda), _p(w), _p(bias),
                                     c_int(code(bias.dtype) if bias is not None else -1), _p(out), c_int(ldc),
                                     c_int(M), c_int(N), c_int(K), code(out.dtype), c_int(1 if silu else 0),
-                                    _stream()), "gemm_skinny")
+                                    _p(None), c_int(0), _stream()), "gemm_skinny")
     return out
 
 
 DECODE_CHUNK = 256          # keys per block of the split decode attention
+_decode_counters: dict = {}  # per device: int32 zeros the decode kernel counts finished blocks in (and zeroes again)
+
+
+def decode_counters(device, n: int) -> torch.Tensor:
+    """Zeroed counters for n (request, kv head) pairs. The kernel leaves them zero, so one buffer
+    serves every call on the device's stream; it must exist before a HIP graph is captured."""
+    buf = _decode_counters.get(device)
+    if buf is None or buf.numel() < n:
+        buf = torch.zeros(max(n, 1 << 16), dtype=torch.int32, device=device)
+        _decode_counters[device] = buf
+    return buf
 
 
 def attn_decode_mfma_supported(dtype, H: int, KVH: int, D: int, page: int) -> bool:
@@ -290,9 +325,10 @@ def attn_decode_mfma(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v
     part_o, part_ml = workspace
     _need(part_o.numel() >= S * H * chunks * D and part_ml.numel() >= S * H * chunks * 2
           and part_o.dtype == torch.float32 and part_ml.dtype == torch.float32, "attn_decode: workspace too small")
+    counters = decode_counters(q.device, S * KVH)
     _check(library().tm_attn_decode_mfma(_p(q), c_int(q_stride), _p(out), c_int(out_stride), _p(k_pool), _p(v_pool),
                                          _p(block_tables), c_int(W), _p(context_lens), _p(part_o), _p(part_ml),
-                                         c_int(chunks), c_int(S), c_int(H), c_int(KVH), c_int(D), c_int(page),
+                                         _p(counters), c_int(chunks), c_int(S), c_int(H), c_int(KVH), c_int(D), c_int(page),
                                          c_float(scale), c_int(window), _stream()), "attn_decode_mfma")
     return out
 
@@ -330,3 +366,66 @@ def attn_prefill_mfma(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, 
                                           c_int(tiles.shape[0]), c_int(H), c_int(KVH), c_int(D), c_int(page),
                                           c_float(scale), c_int(window), _stream()), "attn_prefill_mfma")
     return out
+
+
+FUSED_DECODE_ROWS = 16      # most tokens the norm-fused decode products take
+
+
+def fused_norm_qkv_rope(resid: torch.Tensor, norm_w: torch.Tensor, eps: float, w: torch.Tensor,
+                        bias: torch.Tensor | None, q_out: torch.Tensor, H: int, KVH: int, D: int, cos: torch.Tensor,
+                        sin: torch.Tensor, positions: torch.Tensor, slots: torch.Tensor | None,
+                        k_pool: torch.Tensor | None, v_pool: torch.Tensor | None) -> torch.Tensor:
+    """q_out[M, H*D] and the cache <- rope(rmsnorm(resid) * norm_w @ w^T + bias) for at most 16 tokens.
+    resid float32 [M, K]; w bfloat16 [(H + 2 KVH) D, K]; cos/sin float32 [max_pos, D/2]."""
+    _gpu(resid, norm_w, w, bias, q_out, cos, sin, positions, slots, k_pool, v_pool)
+    M, K = resid.shape
+    _need(0 < M <= FUSED_DECODE_ROWS, f"fused qkv: at most {FUSED_DECODE_ROWS} tokens, got {M}")
+    _need(resid.dtype == torch.float32 and resid.is_contiguous() and resid.data_ptr() % 16 == 0, "fused qkv: resid float32 [M, K]")
+    _need(w.dtype == torch.bfloat16 and w.is_contiguous() and tuple(w.shape) == ((H + 2 * KVH) * D, K) and K % 8 == 0
+          and w.data_ptr() % 16 == 0, "fused qkv: w must be contiguous bfloat16 [(H+2KVH)D, K], K a multiple of 8")
+    _need(D % 32 == 0, f"fused qkv: head size {D} must be a multiple of 32")
+    _need(tuple(norm_w.shape) == (K,) and norm_w.is_contiguous(), "fused qkv: norm weight [K]")
+    _need(cos.dtype == torch.float32 and sin.dtype == torch.float32 and cos.is_contiguous() and sin.is_contiguous()
+          and cos.shape == sin.shape and cos.dim() == 2 and cos.shape[1] * 2 == D,
+          "fused qkv: cos/sin must be float32 [max_pos, D/2] (rotation over the whole head)")
+    _need(q_out.dtype == torch.bfloat16 and q_out.is_contiguous() and tuple(q_out.shape) == (M, H * D), "fused qkv: q_out [M, H*D]")
+    _ints(positions, M, "positions")
+    page = 16
+    if slots is not None:
+        _need(k_pool is not None and v_pool is not None, "fused qkv: slots need the cache pools")
+        page = _check_pools(k_pool, v_pool, KVH, D, torch.bfloat16, "fused qkv")
+        _need(page & (page - 1) == 0, "fused qkv: the page size must be a power of two")
+        _ints(slots, M, "slots")
+    if bias is not None:
+        _need(tuple(bias.shape) == (w.shape[0],) and bias.is_contiguous(), "fused qkv: bias [rows]")
+    _need(eps > 0, "fused qkv: eps must be positive")
+    _check(library().tm_fused_norm_qkv_rope(_p(resid), _p(norm_w), code(norm_w.dtype), c_float(eps), c_int(M), c_int(K),
+                                            _p(w), _p(bias), c_int(code(bias.dtype) if bias is not None else -1),
+                                            _p(q_out), c_int(H), c_int(KVH), c_int(D), _p(cos), _p(sin), _p(positions),
+                                            _p(slots), _p(k_pool if slots is not None else None),
+                                            _p(v_pool if slots is not None else None), c_int(page), _stream()),
+           "fused_norm_qkv_rope")
+    return q_out
+
+
+def fused_norm_gate_up_silu(resid: torch.Tensor, norm_w: torch.Tensor, eps: float, w: torch.Tensor,
+                            out: torch.Tensor) -> torch.Tensor:
+    """out[M, I] <- silu(x Wg^T) * (x Wu^T), x = rmsnorm(resid) * norm_w, w = [Wg; Wu] bfloat16 [2I, K]."""
+    _gpu(resid, norm_w, w, out)
+    M, K = resid.shape
+    I = out.shape[1]
+    _need(0 < M <= FUSED_DECODE_ROWS, f"fused gate-up: at most {FUSED_DECODE_ROWS} tokens, got {M}")
+    _need(resid.dtype == torch.float32 and resid.is_contiguous() and resid.data_ptr() % 16 == 0, "fused gate-up: resid float32 [M, K]")
+    _need(w.dtype == torch.bfloat16 and w.is_contiguous() and tuple(w.shape) == (2 * I, K) and K % 8 == 0 and I % 4 == 0
+          and w.data_ptr() % 16 == 0, "fused gate-up: w must be contiguous bfloat16 [2I, K]; K % 8 == 0, I % 4 == 0")
+    _need(tuple(norm_w.shape) == (K,) and norm_w.is_contiguous(), "fused gate-up: norm weight [K]")
+    _need(out.dtype == torch.bfloat16 and out.is_contiguous() and out.shape[0] == M, "fused gate-up: out bfloat16 [M, I]")
+    _need(eps > 0, "fused gate-up: eps must be positive")
+    _check(library().tm_fused_norm_gate_up_silu(_p(resid), _p(norm_w), code(norm_w.dtype), c_float(eps), c_int(M),
+                                                c_int(K), _p(w), _p(out), c_int(I), _stream()),
+           "fused_norm_gate_up_silu")
+    return out
+
+
+def fused_lds_fits(K: int) -> bool:
+    return 16 * (K + 8) * 2 + 6 * 1024 <= 160 * 1024

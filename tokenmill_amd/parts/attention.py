@@ -11,7 +11,9 @@ from __future__ import annotations
 import torch
 
 from tokenmill_amd.hip import attention as attn_kernels
-from tokenmill_amd.parts.base import KVCacheSpec, KVCacheView, Mixer, PositionEncoding, StepContext
+from tokenmill_amd.hip import gemm, ops
+from tokenmill_amd.parts.base import (KVCacheSpec, KVCacheView, Mixer, NormedInput, PositionEncoding, StepContext,
+                                      as_tensor)
 from tokenmill_amd.parts.linear import Linear
 
 
@@ -42,10 +44,31 @@ class GQAttention(Mixer):
     def cache_spec(self):
         return KVCacheSpec(self.num_kv_heads, self.head_dim, self.window)
 
-    def forward(self, x: torch.Tensor, step: StepContext, cache: KVCacheView) -> torch.Tensor:
-        qkv = self.qkv.forward(x)                                          # [T, (H + 2 KVH) D]
-        self.position.encode_and_store(qkv, self.num_heads, self.num_kv_heads, self.head_dim, step, cache)
-        out = torch.empty((x.shape[0], self.q_size), dtype=qkv.dtype, device=x.device)
-        attn_kernels.paged_attention(qkv, out, cache, step, self.num_heads, self.num_kv_heads, self.head_dim,
+    def _fused_qkv(self, x, step: StepContext, cache: KVCacheView) -> torch.Tensor | None:
+        """q [T, H*D] with k and v already in the cache, by the kernel that starts at the norm; None if
+        that kernel does not take this step."""
+        if not isinstance(x, NormedInput) or x.dtype != torch.bfloat16 or self.head_dim % 32:
+            return None
+        rms = x.fusable_rms()
+        tables = getattr(self.position, "fusable_tables", lambda: None)()
+        page = cache.k.shape[1]
+        if (rms is None or tables is None or not gemm.fused_decode_ok(x.resid, self.qkv.weight) or page & (page - 1)
+                or step.max_context_len > self.position.max_positions):
+            return None
+        q = torch.empty((x.num_tokens, self.q_size), dtype=torch.bfloat16, device=x.resid.device)
+        write = cache.write
+        ops.fused_norm_qkv_rope(x.resid, rms[0], rms[1], self.qkv.weight, self.qkv.bias, q, self.num_heads,
+                                self.num_kv_heads, self.head_dim, tables[0], tables[1], step.positions,
+                                step.groups[cache.group].slot_mapping if write else None,
+                                cache.k if write else None, cache.v if write else None)
+        return q
+
+    def forward(self, x, step: StepContext, cache: KVCacheView, residual: torch.Tensor | None = None):
+        q = self._fused_qkv(x, step, cache)
+        if q is None:
+            q = self.qkv.forward(as_tensor(x))                             # [T, (H + 2 KVH) D], q first
+            self.position.encode_and_store(q, self.num_heads, self.num_kv_heads, self.head_dim, step, cache)
+        out = torch.empty((q.shape[0], self.q_size), dtype=q.dtype, device=q.device)
+        attn_kernels.paged_attention(q, out, cache, step, self.num_heads, self.num_kv_heads, self.head_dim,
                                      self.scale, self.window or 0)
-        return self.o.forward(out)
+        return self.o.forward(out, accumulate_into=residual)

@@ -107,6 +107,44 @@ class Norm(Part):
         With ``rows``: only those rows, and resid is left as it is."""
         raise NotImplementedError
 
+    def rms_params(self) -> tuple[torch.Tensor, float] | None:
+        """(weight, eps) if this norm is weight * round(x * rsqrt(mean(x^2) + eps)), which kernels that
+        follow it can compute themselves; None for any other norm."""
+        return None
+
+
+class NormedInput:
+    """The input of a mixer or feed-forward that is still to be computed: norm(resid + delta).
+
+    A part either calls ``tensor()`` (the add and the norm run as one kernel; resid is updated in
+    place) or, if it has a kernel that starts with the norm, takes ``fusable_rms()`` and reads
+    ``resid`` itself. One of the two must happen, or a pending delta would be lost."""
+
+    def __init__(self, norm: Norm, resid: torch.Tensor, delta: torch.Tensor | None, dtype: torch.dtype):
+        self.norm, self.resid, self.delta, self.dtype = norm, resid, delta, dtype
+        self._tensor: torch.Tensor | None = None
+
+    @property
+    def num_tokens(self) -> int:
+        return self.resid.shape[0]
+
+    def tensor(self) -> torch.Tensor:
+        if self._tensor is None:
+            self._tensor = self.norm.add_norm(self.resid, self.delta, self.dtype)
+            self.delta = None
+        return self._tensor
+
+    def fusable_rms(self) -> tuple[torch.Tensor, float] | None:
+        """(weight, eps) when nothing is pending on the residual and the norm is an RMS norm."""
+        if self._tensor is not None or self.delta is not None:
+            return None
+        return self.norm.rms_params()
+
+
+def as_tensor(x) -> torch.Tensor:
+    """The input of a part as a tensor, whether it came lazily or not."""
+    return x.tensor() if isinstance(x, NormedInput) else x
+
 
 class PositionEncoding(Part):
     def encode_and_store(self, qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
@@ -119,11 +157,14 @@ class Mixer(Part):
     def cache_spec(self) -> KVCacheSpec | StateSpec | None:
         return None
 
-    def forward(self, x: torch.Tensor, step: StepContext, cache) -> torch.Tensor:
-        """x: normed [T, hidden] in the compute type -> [T, hidden] to be added to the residual."""
+    def forward(self, x, step: StepContext, cache, residual: torch.Tensor | None = None) -> torch.Tensor | None:
+        """x: the normed input [T, hidden], as a tensor or a ``NormedInput`` (``as_tensor(x)`` gives the
+        tensor). Returns [T, hidden] to be added to the residual stream; or, if ``residual`` (float32
+        [T, hidden]) is given, it may add its result there itself and return None."""
         raise NotImplementedError
 
 
 class FeedForward(Part):
-    def forward(self, x: torch.Tensor, step: StepContext) -> torch.Tensor:
+    def forward(self, x, step: StepContext, residual: torch.Tensor | None = None) -> torch.Tensor | None:
+        """Same contract as ``Mixer.forward``, without a cache."""
         raise NotImplementedError

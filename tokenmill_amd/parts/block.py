@@ -9,7 +9,7 @@ from __future__ import annotations
 
 import torch
 
-from tokenmill_amd.parts.base import FeedForward, Mixer, Norm, Part, StepContext
+from tokenmill_amd.parts.base import FeedForward, Mixer, Norm, NormedInput, Part, StepContext
 
 
 class PreNormBlock(Part):
@@ -34,8 +34,7 @@ class PreNormBlock(Part):
 
     def forward(self, resid: torch.Tensor, delta: torch.Tensor | None, step: StepContext, cache,
                 dtype: torch.dtype) -> torch.Tensor:
-        """resid float32 [T, hidden], updated in place; returns the delta still to be added."""
-        h = self.norm_in.add_norm(resid, delta, dtype)
-        a = self.mixer.forward(h, step, cache)
-        h = self.norm_post.add_norm(resid, a, dtype)
-        return self.ffn.forward(h, step)
+        """resid float32 [T, hidden], updated in place; returns the delta still to be added (None if the
+        feed-forward added its result itself)."""
+        a = self.mixer.forward(NormedInput(self.norm_in, resid, delta, dtype), step, cache, residual=resid)
+        return self.ffn.forward(NormedInput(self.norm_post, resid, a, dtype), step, residual=resid)

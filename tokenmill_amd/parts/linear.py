@@ -46,16 +46,21 @@ class Linear(Part):
         """Share another part's matrix (a tied output head)."""
         self.weight = weight
 
-    def forward(self, x: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor:
-        """x [M, in] (row-strided views allowed) -> [M, out] in ``out_dtype`` (default: x's type)."""
+    def forward(self, x: torch.Tensor, out_dtype: torch.dtype | None = None,
+                accumulate_into: torch.Tensor | None = None) -> torch.Tensor | None:
+        """x [M, in] (row-strided views allowed) -> [M, out] in ``out_dtype`` (default: x's type).
+        With ``accumulate_into`` (float32 [M, out]) the result may be added there by the product's own
+        epilogue; then None is returned."""
         w = self.weight
         out_dtype = out_dtype or x.dtype
+        from tokenmill_amd.hip import gemm
+        if accumulate_into is not None and w.dtype == x.dtype and gemm.linear_accumulate(x, w, self.bias, accumulate_into):
+            return None
         if w.dtype != x.dtype:
             # a matrix the checkpoint stores in 32-bit stays 32-bit: widen the activations for it
             x = ops.convert(x.contiguous(), torch.empty(x.shape, dtype=w.dtype, device=x.device))
         inner_dtype = torch.float32 if x.dtype == torch.float32 else out_dtype
         out = torch.empty((x.shape[0], self.out_features), dtype=inner_dtype, device=x.device)
-        from tokenmill_amd.hip import gemm
         gemm.linear(x, w, self.bias, out)
         if out.dtype != out_dtype:
             out = ops.convert(out, torch.empty(out.shape, dtype=out_dtype, device=out.device))

@@ -5,7 +5,7 @@ from __future__ import annotations
 import torch
 
 from tokenmill_amd.hip import gemm, ops
-from tokenmill_amd.parts.base import FeedForward, StepContext
+from tokenmill_amd.parts.base import FeedForward, NormedInput, StepContext, as_tensor
 from tokenmill_amd.parts.linear import Linear
 
 
@@ -23,9 +23,18 @@ class SwiGLU(FeedForward):
         self.gate_up.load(tensors, prefix)
         self.down.load(tensors, prefix)
 
-    def forward(self, x: torch.Tensor, step: StepContext | None = None) -> torch.Tensor:
-        act = torch.empty((x.shape[0], self.intermediate), dtype=x.dtype, device=x.device)
+    def forward(self, x, step: StepContext | None = None, residual: torch.Tensor | None = None):
         w = self.gate_up.weight
-        if not (w.dtype == x.dtype and self.gate_up.bias is None and gemm.gate_up_silu(x, w, act)):
-            ops.silu_mul(self.gate_up.forward(x), act)
-        return self.down.forward(act)
+        act = None
+        if isinstance(x, NormedInput) and x.dtype == torch.bfloat16 and self.gate_up.bias is None and \
+                self.intermediate % 4 == 0:
+            rms = x.fusable_rms()
+            if rms is not None and gemm.fused_decode_ok(x.resid, w):      # the kernel that starts at the norm
+                act = torch.empty((x.num_tokens, self.intermediate), dtype=torch.bfloat16, device=x.resid.device)
+                ops.fused_norm_gate_up_silu(x.resid, rms[0], rms[1], w, act)
+        if act is None:
+            x = as_tensor(x)
+            act = torch.empty((x.shape[0], self.intermediate), dtype=x.dtype, device=x.device)
+            if not (w.dtype == x.dtype and self.gate_up.bias is None and gemm.gate_up_silu(x, w, act)):
+                ops.silu_mul(self.gate_up.forward(x), act)
+        return self.down.forward(act, accumulate_into=residual)

@@ -27,3 +27,6 @@ class RMSNorm(Norm):
         n = resid.shape[0] if rows is None else rows.numel()
         out = torch.empty((n, self.hidden), dtype=out_dtype, device=resid.device)
         return ops.add_rmsnorm(resid, delta, self.weight, self.eps, out, rows)
+
+    def rms_params(self):
+        return self.weight, self.eps

@@ -47,6 +47,11 @@ class RotaryEmbedding(PositionEncoding):
                           cache.k if write else None, cache.v if write else None)
 
 
+    def fusable_tables(self):
+        """(cos, sin) when the rotation covers the whole head (what the fused q|k|v kernel applies)."""
+        return (self.cos, self.sin) if self.rotary_dim == self.head_dim else None
+
+
 class NoPositionEncoding(PositionEncoding):
     """Stores k and v; q and k stay as they are."""
 
