@@ -33,8 +33,8 @@ int tm_gemm_skinny(const void* A, int lda, const void* W, const void* bias, int 
 
 int tm_attn_decode_mfma(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
                         const void* v_pool, const int* block_tables, int table_width, const int* context_lens,
-                        float* part_o, float* part_ml, int* counters, int max_chunks, int S, int H, int KVH, int D,
-                        int page, float scale, int window, hipStream_t stream);
+                        float* part_o, float* part_ml, int max_chunks, int S, int H, int KVH, int D, int page,
+                        float scale, int window, hipStream_t stream);
 
 int tm_fused_norm_qkv_rope(const float* resid, const void* norm_w, int norm_w_dtype, float eps, int M, int K,
                            const void* W, const void* bias, int bias_dtype, void* q_out, int H, int KVH, int D,

@@ -3,12 +3,20 @@
 //   One token per request; its G = H / KVH query heads that share a kv head are the 16 columns of
 //   one MFMA tile, so the keys and values of a kv head are read once for all of them
 //   (the reference folds the group into query rows the same way: src/infer/model/layers.py:110-124).
-//   The context is cut into chunks of 256 positions, fixed by position alone; each block of four
-//   wavefronts takes one chunk of one (request, kv head), each wavefront 64 keys of it, and writes
-//   an unnormalised partial (max, sum, weighted values) in 32-bit. The block that finishes last for
-//   a (request, kv head) (a counter tells it) adds the partials in ascending chunk order and writes
-//   the result; the order of the sum is fixed, whichever block happens to do it. What a request
-//   gets therefore does not depend on which other requests are in the batch.
+//   A wavefront always takes 64 consecutive keys, aligned to a multiple of 64 positions, and gets
+//   their unnormalised partial (max, sum, weighted values) in 32-bit. Two ways to cover a context:
+//
+//   block kernel : one block of 8 (16 for head size 32) wavefronts per (request, kv head); wavefront
+//                  w takes keys [64 (i W + w), +64) for i = 0, 1, ...; the partials are merged
+//                  through LDS in wavefront order. One launch, no scratch memory: the way for large
+//                  batches.
+//   split kernels: with few requests more blocks than (request, kv head) pairs are needed to pull
+//                  the cache at speed: blocks of four wavefronts take chunks of 256 positions and
+//                  write partials to scratch memory; a second kernel adds the partials of a request
+//                  in ascending chunk order.
+//
+//   Which keys meet in which partial and in which order partials are added depends on positions
+//   only, so what a request gets does not depend on which other requests are in the batch.
 //
 //   Operand layouts need no LDS: keys K[page][slot][kvh][d] give the A operand of S^T = K Q^T
 //   (16 keys x 32 d per instruction), values V[page][kvh][d][slot] give the A operand of
@@ -39,49 +47,21 @@ union Bf16x8Bits {
     bf16x8_t b;
 };
 
-// D = head size (multiple of 32, at most 128); page a power of two >= 16; G <= 16.
-// Scores are kept as score * scale * log2(e) so that the exponentials are single exp2 instructions.
+// The partial of 64 keys [wbase, wbase + 64) for the (up to 16) query heads of one kv head.
+// Every load is issued before the first product. m is in units of score * scale * log2(e).
 template <int D>
-__global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
-    const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_pool,
-    const bf16_t* __restrict__ v_pool, const int* __restrict__ block_tables, int table_width,
-    const int* __restrict__ context_lens, float* __restrict__ part_o, float* __restrict__ part_ml,
-    int* __restrict__ counters, bf16_t* __restrict__ out, int out_stride, int max_chunks, int H, int KVH,
-    int page_shift, float scale_log2, int window) {
-    constexpr int NDC = D / 32;          // 32-wide d chunks of the q.k product
-    constexpr int NDT = D / 16;          // 16-wide d tiles of the output
-    __shared__ float s_m[4][16], s_l[4][16];
-    __shared__ float s_o[4][16][D + 1];
-
-    const int s = blockIdx.x, kvh = blockIdx.y, chunk = blockIdx.z;
-    const int G = H / KVH;
-    const int ctx = context_lens[s];
-    const int p = ctx - 1;
-    const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
-    const int chunk_lo = chunk * AD_CHUNK;
-    if (chunk_lo >= ctx || chunk_lo + AD_CHUNK <= lo) return;       // nothing of this chunk is visible
-
-    const int wave = threadIdx.x / TM_WAVE, lane = threadIdx.x % TM_WAVE;
-    const int r = lane % 16, g = lane / 16;
-    const int* table = block_tables + (size_t)s * table_width;
+__device__ __forceinline__ void wave_keys64(const Bf16x8Bits (&qreg)[D / 32], const bf16_t* __restrict__ k_pool,
+                                            const bf16_t* __restrict__ v_pool, const int* __restrict__ table,
+                                            int wbase, int ctx, int lo, int kvh, int KVH, int page_shift,
+                                            float scale_log2, int r, int g, float& m, float& l,
+                                            f32x4_t (&o)[D / 16]) {
+    constexpr int NDC = D / 32, NDT = D / 16;
     const int page_mask = (1 << page_shift) - 1;
-    const int wbase = chunk_lo + wave * AD_WKEYS;                   // first key of this wavefront
-
-    // every load of the wavefront is issued before the first product
     int tile_page[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
         const int tile0 = wbase + 16 * t;
         tile_page[t] = (tile0 < ctx && tile0 + 16 > lo) ? table[tile0 >> page_shift] : -1;      // wave-uniform
-    }
-    // Q^T operand: column r = query head kvh*G + r, rows d = 32c + 8g .. +7
-    Bf16x8Bits qreg[NDC];
-#pragma unroll
-    for (int c = 0; c < NDC; ++c) {
-        if (r < G)
-            qreg[c].u = *(const u32x4_t*)(q + (size_t)s * q_stride + (size_t)(kvh * G + r) * D + 32 * c + 8 * g);
-        else
-            qreg[c].u = u32x4_t{0, 0, 0, 0};
     }
     Bf16x8Bits kreg[4][NDC];
     u32x2_t vreg[NDT][4];
@@ -100,7 +80,6 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
         for (int dt = 0; dt < NDT; ++dt)
             vreg[dt][t] = have ? *(const u32x2_t*)(vr + ((size_t)(16 * dt) << page_shift)) : u32x2_t{0, 0};
     }
-
     float sc[4][4];                                                 // [16-key tile][key 4g+i] for head r
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
@@ -114,8 +93,7 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
             sc[t][i] = (kj < ctx && kj >= lo) ? acc[i] * scale_log2 : -INFINITY;
         }
     }
-    // softmax pieces of this wavefront's 64 keys, per head r: combine the four key groups g
-    float m = -INFINITY;
+    m = -INFINITY;
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
@@ -123,7 +101,7 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
     m = fmaxf(m, __shfl_xor(m, 16, TM_WAVE));
     m = fmaxf(m, __shfl_xor(m, 32, TM_WAVE));
     const float neg_m = (m == -INFINITY) ? 0.f : -m;
-    float l = 0.f;
+    l = 0.f;
     float pr[4][4];
 #pragma unroll
     for (int t = 0; t < 4; ++t)
@@ -134,9 +112,7 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
         }
     l += __shfl_xor(l, 16, TM_WAVE);
     l += __shfl_xor(l, 32, TM_WAVE);
-
-    // O^T[d][head] += V^T[d][keys] P^T[keys][head], 32 keys (tiles 2b, 2b+1) per instruction
-    f32x4_t o[NDT];
+    // O^T[d][head] = V^T[d][keys] P^T[keys][head], 32 keys (tiles 2b, 2b+1) per instruction
 #pragma unroll
     for (int dt = 0; dt < NDT; ++dt) o[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -164,8 +140,138 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
             o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.b, pt.b, o[dt], 0, 0, 0);
         }
     }
+}
 
-    // the four wavefronts of the block -> one partial, added in wavefront order
+template <int D>
+__device__ __forceinline__ void load_q_operand(Bf16x8Bits (&qreg)[D / 32], const bf16_t* __restrict__ q, int G,
+                                               int kvh, int r, int g) {
+    // Q^T operand: column r = query head kvh*G + r, rows d = 32c + 8g .. +7
+#pragma unroll
+    for (int c = 0; c < D / 32; ++c) {
+        if (r < G)
+            qreg[c].u = *(const u32x4_t*)(q + (size_t)(kvh * G + r) * D + 32 * c + 8 * g);
+        else
+            qreg[c].u = u32x4_t{0, 0, 0, 0};
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// block kernel: grid (S, KVH), WAVES wavefronts
+// ------------------------------------------------------------------------------------------------
+template <int D, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void attn_decode_block_kernel(
+    const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
+    const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool, const int* __restrict__ block_tables,
+    int table_width, const int* __restrict__ context_lens, int H, int KVH, int page_shift, float scale_log2,
+    int window) {
+    constexpr int NDT = D / 16;
+    __shared__ float s_m[WAVES][16], s_l[WAVES][16];
+    __shared__ float s_o[WAVES][16][16 + 1];                         // one 16-wide d tile at a time
+    const int s = blockIdx.x, kvh = blockIdx.y;
+    const int G = H / KVH;
+    const int ctx = context_lens[s];
+    const int p = ctx - 1;
+    const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+    const int wave = threadIdx.x / TM_WAVE, lane = threadIdx.x % TM_WAVE;
+    const int r = lane % 16, g = lane / 16;
+    const int* table = block_tables + (size_t)s * table_width;
+
+    Bf16x8Bits qreg[D / 32];
+    load_q_operand<D>(qreg, q + (size_t)s * q_stride, G, kvh, r, g);
+
+    float m = -INFINITY, l = 0.f;
+    f32x4_t o[NDT];
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) o[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    const int first = (lo / AD_WKEYS) * AD_WKEYS;                   // aligned to 64 positions
+    for (int wbase = first + wave * AD_WKEYS; wbase < ctx; wbase += WAVES * AD_WKEYS) {
+        float mi, li;
+        f32x4_t oi[NDT];
+        wave_keys64<D>(qreg, k_pool, v_pool, table, wbase, ctx, lo, kvh, KVH, page_shift, scale_log2, r, g, mi, li, oi);
+        const float mn = fmaxf(m, mi);
+        const float f0 = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m - mn);
+        const float f1 = (mi == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mi - mn);
+        l = l * f0 + li * f1;
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) o[dt][i] = o[dt][i] * f0 + oi[dt][i] * f1;
+        m = mn;
+    }
+    // merge the wavefronts in wavefront order; lane: head r, d = 16 dt + 4 g + i
+    if (g == 0) {
+        s_m[wave][r] = m;
+        s_l[wave][r] = l;
+    }
+    __syncthreads();
+    float mm = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) mm = fmaxf(mm, s_m[w][r]);
+    float ll = 0.f;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w)
+        ll += s_l[w][r] * ((s_m[w][r] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(s_m[w][r] - mm));
+    const float inv = 1.f / ll;
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) s_o[wave][r][4 * g + i] = o[dt][i];
+        __syncthreads();
+        // wavefront dt % WAVES writes this tile: thread -> (head n, 4 consecutive d)
+        if (wave == dt % WAVES) {
+            const int n = lane / 4, d4 = (lane % 4) * 4;
+            if (n < G) {
+                float mx = -INFINITY;
+#pragma unroll
+                for (int w = 0; w < WAVES; ++w) mx = fmaxf(mx, s_m[w][n]);
+                float lsum = 0.f, acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int w = 0; w < WAVES; ++w) {
+                    const float f = (s_m[w][n] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(s_m[w][n] - mx);
+                    lsum += s_l[w][n] * f;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) acc[i] += s_o[w][n][d4 + i] * f;
+                }
+                const float iv = 1.f / lsum;
+                uint2 pk;
+                pk.x = pack_bf16(acc[0] * iv, acc[1] * iv);
+                pk.y = pack_bf16(acc[2] * iv, acc[3] * iv);
+                *(uint2*)(out + (size_t)s * out_stride + (size_t)(kvh * G + n) * D + 16 * dt + d4) = pk;
+            }
+        }
+        __syncthreads();
+    }
+    (void)inv;
+}
+
+// ------------------------------------------------------------------------------------------------
+// split kernels: grid (S, KVH, chunks) with four wavefronts, then the merge
+// ------------------------------------------------------------------------------------------------
+template <int D>
+__global__ __launch_bounds__(256) void attn_decode_split_kernel(
+    const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_pool,
+    const bf16_t* __restrict__ v_pool, const int* __restrict__ block_tables, int table_width,
+    const int* __restrict__ context_lens, float* __restrict__ part_o, float* __restrict__ part_ml,
+    int max_chunks, int H, int KVH, int page_shift, float scale_log2, int window) {
+    constexpr int NDT = D / 16;
+    __shared__ float s_m[4][16], s_l[4][16];
+    __shared__ float s_o[4][16][D + 1];
+    const int s = blockIdx.x, kvh = blockIdx.y, chunk = blockIdx.z;
+    const int G = H / KVH;
+    const int ctx = context_lens[s];
+    const int p = ctx - 1;
+    const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+    const int chunk_lo = chunk * AD_CHUNK;
+    if (chunk_lo >= ctx || chunk_lo + AD_CHUNK <= lo) return;       // nothing of this chunk is visible
+    const int wave = threadIdx.x / TM_WAVE, lane = threadIdx.x % TM_WAVE;
+    const int r = lane % 16, g = lane / 16;
+    const int* table = block_tables + (size_t)s * table_width;
+    Bf16x8Bits qreg[D / 32];
+    load_q_operand<D>(qreg, q + (size_t)s * q_stride, G, kvh, r, g);
+    float m, l;
+    f32x4_t o[NDT];
+    wave_keys64<D>(qreg, k_pool, v_pool, table, chunk_lo + wave * AD_WKEYS, ctx, lo, kvh, KVH, page_shift, scale_log2,
+                   r, g, m, l, o);
     if (g == 0) {
         s_m[wave][r] = m;
         s_l[wave][r] = l;
@@ -194,75 +300,77 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
             part_ml[slot * 2 + 1] = ll;
         }
     }
-    // Is this the last block of its (request, kv head)? Its partial is published first (release),
-    // the counter is bumped, and the one that sees the full count reads the others' (acquire).
-    __shared__ int s_last;
+}
+
+// out[s, h, :] = sum over the visible chunks (ascending) of partial values, normalised.
+__global__ void attn_decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                         const int* __restrict__ context_lens, bf16_t* __restrict__ out,
+                                         int out_stride, int max_chunks, int H, int D, int window) {
+    const int s = blockIdx.x, h = blockIdx.y;
+    const int ctx = context_lens[s];
+    const int p = ctx - 1;
+    const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
     const int c0 = lo / AD_CHUNK, c1 = (ctx - 1) / AD_CHUNK;
-    __threadfence();
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        int* cnt = counters + (size_t)s * KVH + kvh;
-        const int old = __hip_atomic_fetch_add(cnt, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-        s_last = (old == c1 - c0);
-        if (s_last) __hip_atomic_store(cnt, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next call
-    }
-    __syncthreads();
-    if (!s_last) return;
-    __threadfence();
-    for (int idx = threadIdx.x; idx < G * D; idx += 256) {
-        const int n = idx / D, d = idx % D;
-        const size_t base = ((size_t)s * H + kvh * G + n) * max_chunks;
-        float mm = -INFINITY;
-        for (int c = c0; c <= c1; ++c)
-            mm = fmaxf(mm, __hip_atomic_load(part_ml + (base + c) * 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+    const size_t base = ((size_t)s * H + h) * max_chunks;
+    float mm = -INFINITY;
+    for (int c = c0; c <= c1; ++c) mm = fmaxf(mm, part_ml[(base + c) * 2]);
+    for (int d = threadIdx.x; d < D; d += blockDim.x) {
         float ll = 0.f, oo = 0.f;
         for (int c = c0; c <= c1; ++c) {
-            const float mc = __hip_atomic_load(part_ml + (base + c) * 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const float mc = part_ml[(base + c) * 2];
             const float f = (mc == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mc - mm);
-            ll += __hip_atomic_load(part_ml + (base + c) * 2 + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * f;
-            oo += __hip_atomic_load(part_o + (base + c) * D + d, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * f;
+            ll += part_ml[(base + c) * 2 + 1] * f;
+            oo += part_o[(base + c) * D + d] * f;
         }
-        out[(size_t)s * out_stride + (size_t)(kvh * G + n) * D + d] = f32_to_bf16(oo / ll);
+        out[(size_t)s * out_stride + (size_t)h * D + d] = f32_to_bf16(oo / ll);
     }
 }
 
 template <int D>
 static int launch_decode(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
                          const void* v_pool, const int* block_tables, int table_width, const int* context_lens,
-                         float* part_o, float* part_ml, int* counters, int max_chunks, int S, int H, int KVH,
-                         int page, float scale, int window, hipStream_t stream) {
+                         float* part_o, float* part_ml, int max_chunks, int S, int H, int KVH, int page,
+                         float scale, int window, hipStream_t stream) {
     int page_shift = 0;
     while ((1 << page_shift) < page) ++page_shift;
     const float scale_log2 = scale * 1.4426950408889634f;
-    dim3 grid(S, KVH, max_chunks);
-    attn_decode_mfma_kernel<D><<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)k_pool,
-                                                         (const bf16_t*)v_pool, block_tables, table_width,
-                                                         context_lens, part_o, part_ml, counters, (bf16_t*)out,
-                                                         out_stride, max_chunks, H, KVH, page_shift, scale_log2,
-                                                         window);
+    constexpr int WAVES = D <= 32 ? 16 : 8;       // 16 wavefronts leave 128 registers each: enough for D = 32 only
+    // few (request, kv head) pairs: more blocks than pairs are needed to pull the cache at speed
+    const bool split = part_o && part_ml && (long long)S * KVH < 64 && max_chunks > 1;
+    if (!split) {
+        attn_decode_block_kernel<D, WAVES><<<dim3(S, KVH), 64 * WAVES, 0, stream>>>(
+            (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool,
+            block_tables, table_width, context_lens, H, KVH, page_shift, scale_log2, window);
+        TM_CHECK_LAUNCH();
+        return TM_OK;
+    }
+    attn_decode_split_kernel<D><<<dim3(S, KVH, max_chunks), 256, 0, stream>>>(
+        (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, block_tables, table_width,
+        context_lens, part_o, part_ml, max_chunks, H, KVH, page_shift, scale_log2, window);
+    TM_CHECK_LAUNCH();
+    attn_decode_merge_kernel<<<dim3(S, H), 64, 0, stream>>>(part_o, part_ml, context_lens, (bf16_t*)out, out_stride,
+                                                            max_chunks, H, D, window);
     TM_CHECK_LAUNCH();
     return TM_OK;
 }
 
 // q: first decode row (one row per request, rows q_stride apart); out likewise; block_tables and
-// context_lens: first decode request. part_o: float [S, H, max_chunks, D]; part_ml: [S, H, max_chunks, 2];
-// counters: int [S * KVH], all zero on entry (and again on exit). Calls that share counters must not overlap.
+// context_lens: first decode request. part_o: float [S, H, max_chunks, D] and part_ml: [S, H, max_chunks, 2]
+// are scratch for the split kernels (used when there are fewer than 64 (request, kv head) pairs); without
+// them the block kernel runs.
 extern "C" int tm_attn_decode_mfma(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
                                    const void* v_pool, const int* block_tables, int table_width,
-                                   const int* context_lens, float* part_o, float* part_ml, int* counters,
-                                   int max_chunks, int S, int H, int KVH, int D, int page, float scale, int window,
-                                   hipStream_t stream) {
+                                   const int* context_lens, float* part_o, float* part_ml, int max_chunks, int S,
+                                   int H, int KVH, int D, int page, float scale, int window, hipStream_t stream) {
     if (S <= 0) return TM_OK;
-    if (!counters) return TM_ERR_ARG;
     if (H <= 0 || KVH <= 0 || H % KVH || H / KVH > 16 || page < 16 || (page & (page - 1)) || max_chunks <= 0 ||
-        !(scale > 0.f) ||
-        max_chunks > 65535 || KVH > 65535 || window < 0 || table_width <= 0 || (q_stride % 8) ||
-        ((uintptr_t)q % 16) || q_stride < H * D || out_stride < H * D)
+        !(scale > 0.f) || max_chunks > 65535 || KVH > 65535 || window < 0 || table_width <= 0 || (q_stride % 8) ||
+        ((uintptr_t)q % 16) || (out_stride % 4) || ((uintptr_t)out % 8) || q_stride < H * D || out_stride < H * D)
         return TM_ERR_ARG;
 #define TM_DECODE_CASE(DD)                                                                                        \
     case DD:                                                                                                      \
         return launch_decode<DD>(q, q_stride, out, out_stride, k_pool, v_pool, block_tables, table_width,         \
-                                 context_lens, part_o, part_ml, counters, max_chunks, S, H, KVH, page, scale, window, stream)
+                                 context_lens, part_o, part_ml, max_chunks, S, H, KVH, page, scale, window, stream)
     switch (D) {
         TM_DECODE_CASE(32);
         TM_DECODE_CASE(64);

@@ -38,6 +38,7 @@ __device__ __forceinline__ float fd_round(float a) { return bf16_to_f32(f32_to_b
 #define FD_EPI_SILU 1
 #define FD_KCH 8            // k-steps whose matrix loads are in flight at once, per wavefront
 #define FD_XPAD 8           // padding of an LDS row of x, in elements
+#define FD_RC 8             // 4-element vectors of a residual row a thread keeps in registers
 
 struct FusedArgs {
     // norm + product
@@ -111,36 +112,84 @@ __global__ __launch_bounds__(256) void fused_norm_gemm_kernel(const FusedArgs a)
         fb[j].u = in ? *(const u32x4_t*)(wB + k) : u32x4_t{0, 0, 0, 0};
     }
 
-    // x = norm(resid) into LDS: 16 threads per token
+    // what the epilogue will need from memory is asked for now, long before it is used
+    const int etok = r;                                              // the epilogue's token of this lane
+    float e_bias[2][4] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+    float e_cos[4] = {1.f, 1.f, 1.f, 1.f}, e_sin[4] = {0.f, 0.f, 0.f, 0.f};
+    int e_slot = -1;
+    if (EPI == FD_EPI_QKV && wave == 0 && etok < M) {
+        if (a.bias) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int ia = nA + 4 * g + i, ib = nB + 4 * g + i;
+                e_bias[0][i] = a.bias_f32 ? ((const float*)a.bias)[ia] : bf16_to_f32(((const bf16_t*)a.bias)[ia]);
+                e_bias[1][i] = a.bias_f32 ? ((const float*)a.bias)[ib] : bf16_to_f32(((const bf16_t*)a.bias)[ib]);
+            }
+        }
+        e_slot = a.slots ? a.slots[etok] : -1;
+        if (head < a.H + a.KVH) {
+            const size_t at = (size_t)a.positions[etok] * (a.D / 2) + 16 * jt + 4 * g;
+            const f32x4_t cv = *(const f32x4_t*)(a.cos_t + at), sv = *(const f32x4_t*)(a.sin_t + at);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                e_cos[i] = cv[i];
+                e_sin[i] = sv[i];
+            }
+        }
+    }
+
+    // x = norm(resid) into LDS. A row is shared by TPR threads (all 256 are busy: 16 rows x 16 threads,
+    // 8 x 32, or 4 x 64); each keeps its first FD_RC vectors in registers between the two passes.
     {
-        const int row = threadIdx.x / 16, sub = threadIdx.x % 16;
+        const int mpad = M <= 4 ? 4 : (M <= 8 ? 8 : 16);
+        const int tpr = 256 / mpad;
+        const int row = threadIdx.x / tpr, sub = threadIdx.x % tpr;
         bf16_t* xrow = xs + (size_t)row * xstride;
+        const int step = 4 * tpr;
         if (row < M) {
             const float* src = a.resid + (size_t)row * K;
+            f32x4_t cache[FD_RC];
             float ss = 0.f;
-            for (int c = sub * 4; c < K; c += 64) {
+#pragma unroll
+            for (int j = 0; j < FD_RC; ++j) {
+                const int c = sub * 4 + j * step;
+                cache[j] = c < K ? *(const f32x4_t*)(src + c) : f32x4_t{0.f, 0.f, 0.f, 0.f};
+                ss += cache[j][0] * cache[j][0] + cache[j][1] * cache[j][1] + cache[j][2] * cache[j][2] +
+                      cache[j][3] * cache[j][3];
+            }
+            for (int c = sub * 4 + FD_RC * step; c < K; c += step) {
                 const f32x4_t v = *(const f32x4_t*)(src + c);
                 ss += v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
             }
-            ss += __shfl_xor(ss, 1, TM_WAVE);
-            ss += __shfl_xor(ss, 2, TM_WAVE);
-            ss += __shfl_xor(ss, 4, TM_WAVE);
-            ss += __shfl_xor(ss, 8, TM_WAVE);
+            for (int off = 1; off < tpr; off <<= 1) ss += __shfl_xor(ss, off, TM_WAVE);
             const float rs = rsqrtf(ss / (float)K + a.eps);
-            for (int c = sub * 4; c < K; c += 64) {
-                const f32x4_t v = *(const f32x4_t*)(src + c);
+            auto emit = [&](int c, const f32x4_t v) {
                 float w[4];
+                if (a.norm_w_f32) {
+                    const f32x4_t wv = *(const f32x4_t*)((const float*)a.norm_w + c);
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    w[i] = a.norm_w_f32 ? ((const float*)a.norm_w)[c + i] : bf16_to_f32(((const bf16_t*)a.norm_w)[c + i]);
+                    for (int i = 0; i < 4; ++i) w[i] = wv[i];
+                } else {
+                    const uint2 wv = *(const uint2*)((const bf16_t*)a.norm_w + c);
+                    w[0] = __uint_as_float(wv.x << 16);
+                    w[1] = __uint_as_float(wv.x & 0xffff0000u);
+                    w[2] = __uint_as_float(wv.y << 16);
+                    w[3] = __uint_as_float(wv.y & 0xffff0000u);
+                }
                 uint2 pk;
                 pk.x = fd_pack(w[0] * fd_round(v[0] * rs), w[1] * fd_round(v[1] * rs));
                 pk.y = fd_pack(w[2] * fd_round(v[2] * rs), w[3] * fd_round(v[3] * rs));
                 *(uint2*)(xrow + c) = pk;
+            };
+#pragma unroll
+            for (int j = 0; j < FD_RC; ++j) {
+                const int c = sub * 4 + j * step;
+                if (c < K) emit(c, cache[j]);
             }
-        } else {
-            for (int c = sub * 4; c < K; c += 64) *(uint2*)(xrow + c) = uint2{0u, 0u};
+            for (int c = sub * 4 + FD_RC * step; c < K; c += step) emit(c, *(const f32x4_t*)(src + c));
         }
+        // rows M..15 of x stay as they are: they only feed result columns of tokens that do not exist,
+        // which no lane stores
     }
     __syncthreads();
 
@@ -202,25 +251,18 @@ __global__ __launch_bounds__(256) void fused_norm_gemm_kernel(const FusedArgs a)
     float xA[4], xB[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        float bA = 0.f, bB = 0.f;
-        if (a.bias) {
-            bA = a.bias_f32 ? ((const float*)a.bias)[nA + 4 * g + i] : bf16_to_f32(((const bf16_t*)a.bias)[nA + 4 * g + i]);
-            bB = a.bias_f32 ? ((const float*)a.bias)[nB + 4 * g + i] : bf16_to_f32(((const bf16_t*)a.bias)[nB + 4 * g + i]);
-        }
-        xA[i] = fd_round(accA[i] + bA);
-        xB[i] = fd_round(accB[i] + bB);
+        xA[i] = fd_round(accA[i] + e_bias[0][i]);
+        xB[i] = fd_round(accB[i] + e_bias[1][i]);
     }
-    const int slot = a.slots ? a.slots[tok] : -1;
+    const int slot = e_slot;
     if (head < a.H + a.KVH) {
         const int half = a.D / 2;
         const int j0 = 16 * jt + 4 * g;                              // pair index of element 0
-        const float* c = a.cos_t + (size_t)a.positions[tok] * half + j0;
-        const float* s = a.sin_t + (size_t)a.positions[tok] * half + j0;
         float y1[4], y2[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            y1[i] = xA[i] * c[i] - xB[i] * s[i];
-            y2[i] = xB[i] * c[i] + xA[i] * s[i];
+            y1[i] = xA[i] * e_cos[i] - xB[i] * e_sin[i];
+            y2[i] = xB[i] * e_cos[i] + xA[i] * e_sin[i];
         }
         bf16_t* dst = nullptr;
         if (head < a.H)

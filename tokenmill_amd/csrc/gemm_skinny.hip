@@ -74,7 +74,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
                                                                  float* __restrict__ accum, int ldacc) {
     constexpr int NACC = SILU ? 2 : 1;
     // k-steps in flight per wavefront (fewer where 16 wavefronts share the register file)
-    constexpr int KCH = (WAVES > 4 && SILU && NT > 2) ? 4 : ((WAVES > 4 || NT > 2 || SILU) ? 8 : 16);
+    constexpr int KCH = (WAVES > 4 && SILU && NT > 2) ? 4 : ((WAVES > 4 && NT == 1 && !SILU) ? 12 : ((WAVES > 4 || NT > 2 || SILU) ? 8 : 16));
     __shared__ float red[SPLIT ? WAVES : 1][64][4 + 1];        // one accumulator tile at a time
     const int wave = threadIdx.x / TM_WAVE, lane = threadIdx.x % TM_WAVE;
     const int r = lane % 16, g = lane / 16;
@@ -168,7 +168,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
         }
         if (accum) {            // the rounded result goes into the 32-bit residual stream (each element has one owner)
             float* dst = accum + (size_t)tok * ldacc + nf;
-            for (int i = 0; i < 4 && nf + i < N; ++i) dst[i] += bf16_to_f32(f32_to_bf16(v[i]));
+            if (nf + 4 <= N && ((uintptr_t)dst % 16) == 0) {
+                f32x4_t cur = *(f32x4_t*)dst;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) cur[i] += bf16_to_f32(f32_to_bf16(v[i]));
+                *(f32x4_t*)dst = cur;
+            } else {
+                for (int i = 0; i < 4 && nf + i < N; ++i) dst[i] += bf16_to_f32(f32_to_bf16(v[i]));
+            }
         } else {
             store4<TC>(C + (size_t)tok * ldc + nf, v, N - nf);
         }

@@ -279,17 +279,7 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, out
 
 
 DECODE_CHUNK = 256          # keys per block of the split decode attention
-_decode_counters: dict = {}  # per device: int32 zeros the decode kernel counts finished blocks in (and zeroes again)
-
-
-def decode_counters(device, n: int) -> torch.Tensor:
-    """Zeroed counters for n (request, kv head) pairs. The kernel leaves them zero, so one buffer
-    serves every call on the device's stream; it must exist before a HIP graph is captured."""
-    buf = _decode_counters.get(device)
-    if buf is None or buf.numel() < n:
-        buf = torch.zeros(max(n, 1 << 16), dtype=torch.int32, device=device)
-        _decode_counters[device] = buf
-    return buf
+DECODE_SPLIT_PAIRS = 64     # below this many (request, kv head) pairs the split kernels (with scratch memory) run
 
 
 def attn_decode_mfma_supported(dtype, H: int, KVH: int, D: int, page: int) -> bool:
@@ -319,16 +309,18 @@ def attn_decode_mfma(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v
     _ints(context_lens, S, "context_lens")
     _need(0 < max_context <= W * page, "attn_decode: max_context exceeds what the block tables hold")
     chunks = -(-max_context // DECODE_CHUNK)
-    if workspace is None:
-        workspace = (torch.empty((S, H, chunks, D), dtype=torch.float32, device=q.device),
-                     torch.empty((S, H, chunks, 2), dtype=torch.float32, device=q.device))
-    part_o, part_ml = workspace
-    _need(part_o.numel() >= S * H * chunks * D and part_ml.numel() >= S * H * chunks * 2
-          and part_o.dtype == torch.float32 and part_ml.dtype == torch.float32, "attn_decode: workspace too small")
-    counters = decode_counters(q.device, S * KVH)
+    part_o = part_ml = None
+    if S * KVH < DECODE_SPLIT_PAIRS and chunks > 1:
+        if workspace is None:
+            workspace = (torch.empty((S, H, chunks, D), dtype=torch.float32, device=q.device),
+                         torch.empty((S, H, chunks, 2), dtype=torch.float32, device=q.device))
+        part_o, part_ml = workspace
+        _need(part_o.numel() >= S * H * chunks * D and part_ml.numel() >= S * H * chunks * 2
+              and part_o.dtype == torch.float32 and part_ml.dtype == torch.float32, "attn_decode: workspace too small")
+    _need(out_stride % 4 == 0 and out.data_ptr() % 8 == 0, "attn_decode: out rows must be 8-byte aligned")
     _check(library().tm_attn_decode_mfma(_p(q), c_int(q_stride), _p(out), c_int(out_stride), _p(k_pool), _p(v_pool),
                                          _p(block_tables), c_int(W), _p(context_lens), _p(part_o), _p(part_ml),
-                                         _p(counters), c_int(chunks), c_int(S), c_int(H), c_int(KVH), c_int(D), c_int(page),
+                                         c_int(chunks), c_int(S), c_int(H), c_int(KVH), c_int(D), c_int(page),
                                          c_float(scale), c_int(window), _stream()), "attn_decode_mfma")
     return out
 
@@ -384,7 +376,7 @@ def fused_norm_qkv_rope(resid: torch.Tensor, norm_w: torch.Tensor, eps: float, w
     _need(w.dtype == torch.bfloat16 and w.is_contiguous() and tuple(w.shape) == ((H + 2 * KVH) * D, K) and K % 8 == 0
           and w.data_ptr() % 16 == 0, "fused qkv: w must be contiguous bfloat16 [(H+2KVH)D, K], K a multiple of 8")
     _need(D % 32 == 0, f"fused qkv: head size {D} must be a multiple of 32")
-    _need(tuple(norm_w.shape) == (K,) and norm_w.is_contiguous(), "fused qkv: norm weight [K]")
+    _need(tuple(norm_w.shape) == (K,) and norm_w.is_contiguous() and norm_w.data_ptr() % 16 == 0, "fused qkv: norm weight [K]")
     _need(cos.dtype == torch.float32 and sin.dtype == torch.float32 and cos.is_contiguous() and sin.is_contiguous()
           and cos.shape == sin.shape and cos.dim() == 2 and cos.shape[1] * 2 == D,
           "fused qkv: cos/sin must be float32 [max_pos, D/2] (rotation over the whole head)")
@@ -418,7 +410,7 @@ def fused_norm_gate_up_silu(resid: torch.Tensor, norm_w: torch.Tensor, eps: floa
     _need(resid.dtype == torch.float32 and resid.is_contiguous() and resid.data_ptr() % 16 == 0, "fused gate-up: resid float32 [M, K]")
     _need(w.dtype == torch.bfloat16 and w.is_contiguous() and tuple(w.shape) == (2 * I, K) and K % 8 == 0 and I % 4 == 0
           and w.data_ptr() % 16 == 0, "fused gate-up: w must be contiguous bfloat16 [2I, K]; K % 8 == 0, I % 4 == 0")
-    _need(tuple(norm_w.shape) == (K,) and norm_w.is_contiguous(), "fused gate-up: norm weight [K]")
+    _need(tuple(norm_w.shape) == (K,) and norm_w.is_contiguous() and norm_w.data_ptr() % 16 == 0, "fused gate-up: norm weight [K]")
     _need(out.dtype == torch.bfloat16 and out.is_contiguous() and out.shape[0] == M, "fused gate-up: out bfloat16 [M, I]")
     _need(eps > 0, "fused gate-up: eps must be positive")
     _check(library().tm_fused_norm_gate_up_silu(_p(resid), _p(norm_w), code(norm_w.dtype), c_float(eps), c_int(M),
