@@ -64,6 +64,8 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (named in config)")
     ap.add_argument("--no-graphs", action="store_true", help="launch decode steps kernel by kernel")
     ap.add_argument("--skip-points", action="store_true", help="only the headline batch and the prefill")
+    ap.add_argument("--part", default="all", choices=["all", "decode", "prefill"],
+                    help="run only the decode steps or only the prefill (for profiling one of them)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -131,8 +133,16 @@ def main() -> int:
             assert outs and outs[0].finished
         return statistics.median(times[1:])              # the first run warms up
 
+    if args.part == "prefill":
+        prefill_s = time_prefill()
+        print(json.dumps({"prefill": {"value": round(PROMPT_LEN / prefill_s, 1), "tokens": PROMPT_LEN,
+                                      "ms": round(prefill_s * 1e3, 3)}}))
+        return 0
     step_s, context = time_decode(args.batch, args.steps, args.warmup)
     value = args.batch / step_s
+    if args.part == "decode":
+        print(json.dumps({"value": round(value, 1), "ms_per_step": round(step_s * 1e3, 4), "batch": args.batch}))
+        return 0
     prefill_s = time_prefill()
     points = {}
     if not args.skip_points:
