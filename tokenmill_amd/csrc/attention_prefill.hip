@@ -28,7 +28,7 @@ union PFrag {
     bf16x8_t b;
 };
 
-#define AP_HPW 4            // query heads per wavefront
+#define AP_HPW 2            // query heads per wavefront
 #define AP_KSPLIT 4         // wavefronts of a block, each taking every fourth block of 32 keys
 
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
@@ -79,8 +79,9 @@ __device__ __forceinline__ void load_kv_block(KVBlock<D>& blk, int kb, int first
 // with kb % AP_KSPLIT == j and the partial results are merged through LDS in wavefront order.
 // Which blocks a wavefront takes depends on absolute positions only, and a block in which a token
 // sees no key changes nothing for it, so a token's bits do not depend on the tile it falls into.
+// (two blocks per CU where the head size leaves room: a second wavefront per SIMD hides the first one's loads)
 template <int D>
-__global__ __launch_bounds__(64 * AP_KSPLIT) void attn_prefill_mfma_kernel(
+__global__ __launch_bounds__(64 * AP_KSPLIT, D <= 64 ? 3 : 1) void attn_prefill_mfma_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
     const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool, const int* __restrict__ block_tables,
     int table_width, const int* __restrict__ tiles, int H, int KVH, int page_shift, float scale_log2, int window) {

@@ -68,20 +68,95 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const T* __restric
     }
 }
 
+// The same for widths that are a multiple of 4 and at most 4096: every thread keeps its (up to four)
+// 4-element groups of the row in registers, so the row is read once.
+typedef float ew_f32x4 __attribute__((ext_vector_type(4)));
+
+template <typename T> struct Vec4;
+template <> struct Vec4<float> {
+    static __device__ __forceinline__ ew_f32x4 load(const float* p) { return *(const ew_f32x4*)p; }
+    static __device__ __forceinline__ void store(float* p, ew_f32x4 v) { *(ew_f32x4*)p = v; }
+};
+template <> struct Vec4<bf16_t> {
+    static __device__ __forceinline__ ew_f32x4 load(const bf16_t* p) {
+        const uint2 u = *(const uint2*)p;
+        return ew_f32x4{__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u), __uint_as_float(u.y << 16),
+                        __uint_as_float(u.y & 0xffff0000u)};
+    }
+    static __device__ __forceinline__ void store(bf16_t* p, ew_f32x4 v) {
+        uint2 u;
+        u.x = (uint32_t)f32_to_bf16(v[0]) | ((uint32_t)f32_to_bf16(v[1]) << 16);
+        u.y = (uint32_t)f32_to_bf16(v[2]) | ((uint32_t)f32_to_bf16(v[3]) << 16);
+        *(uint2*)p = u;
+    }
+};
+
+template <typename T, typename WT>
+__global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict__ resid, const T* __restrict__ delta,
+                                                              const int* __restrict__ rows,
+                                                              const WT* __restrict__ weight, T* __restrict__ out,
+                                                              int hidden, float eps) {
+    __shared__ float red[4];
+    const int r = blockIdx.x;
+    const size_t src = rows ? (size_t)rows[r] : (size_t)r;
+    float* x = resid + src * hidden;
+    const T* d = delta ? delta + src * hidden : nullptr;
+    T* o = out + (size_t)r * hidden;
+    const int groups = hidden / 4;
+    ew_f32x4 v[4];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int gidx = threadIdx.x + i * 256;
+        v[i] = ew_f32x4{0.f, 0.f, 0.f, 0.f};
+        if (gidx < groups) {
+            v[i] = Vec4<float>::load(x + 4 * gidx);
+            if (d) {
+                v[i] += Vec4<T>::load(d + 4 * gidx);
+                if (!rows) Vec4<float>::store(x + 4 * gidx, v[i]);
+            }
+            ss += v[i][0] * v[i][0] + v[i][1] * v[i][1] + v[i][2] * v[i][2] + v[i][3] * v[i][3];
+        }
+    }
+    ss = block_sum<256>(ss, red);
+    const float rs = rsqrtf(ss / (float)hidden + eps);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int gidx = threadIdx.x + i * 256;
+        if (gidx < groups) {
+            const ew_f32x4 w = Vec4<WT>::load(weight + 4 * gidx);
+            ew_f32x4 y;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) y[k] = w[k] * Elem<T>::round(v[i][k] * rs);   // rounded BEFORE the weight multiplies
+            Vec4<T>::store(o + 4 * gidx, y);
+        }
+    }
+}
+
+template <typename T, typename WT>
+static void launch_add_rmsnorm(float* resid, const void* delta, const int* rows, const void* weight, void* out, int R,
+                               int hidden, float eps, hipStream_t stream) {
+    const bool vec = hidden % 4 == 0 && hidden <= 4096 && ((uintptr_t)resid % 16) == 0 && ((uintptr_t)weight % 16) == 0 &&
+                     ((uintptr_t)out % 16) == 0 && (!delta || ((uintptr_t)delta % 16) == 0);
+    if (vec)
+        add_rmsnorm_vec_kernel<T, WT><<<R, 256, 0, stream>>>(resid, (const T*)delta, rows, (const WT*)weight, (T*)out,
+                                                             hidden, eps);
+    else
+        add_rmsnorm_kernel<T, WT><<<R, 256, 0, stream>>>(resid, (const T*)delta, rows, (const WT*)weight, (T*)out,
+                                                         hidden, eps);
+}
+
 extern "C" int tm_add_rmsnorm(float* resid, const void* delta, const int* rows, const void* weight,
                               int w_dtype, void* out, int dtype, int R, int hidden, float eps,
                               hipStream_t stream) {
     if (R <= 0) return TM_OK;
     if (hidden <= 0 || !(eps > 0.f)) return TM_ERR_ARG;
     if (dtype == TM_F32 && w_dtype == TM_F32)
-        add_rmsnorm_kernel<float, float><<<R, 256, 0, stream>>>(resid, (const float*)delta, rows,
-                                                               (const float*)weight, (float*)out, hidden, eps);
+        launch_add_rmsnorm<float, float>(resid, delta, rows, weight, out, R, hidden, eps, stream);
     else if (dtype == TM_BF16 && w_dtype == TM_BF16)
-        add_rmsnorm_kernel<bf16_t, bf16_t><<<R, 256, 0, stream>>>(resid, (const bf16_t*)delta, rows,
-                                                                 (const bf16_t*)weight, (bf16_t*)out, hidden, eps);
+        launch_add_rmsnorm<bf16_t, bf16_t>(resid, delta, rows, weight, out, R, hidden, eps, stream);
     else if (dtype == TM_BF16 && w_dtype == TM_F32)
-        add_rmsnorm_kernel<bf16_t, float><<<R, 256, 0, stream>>>(resid, (const bf16_t*)delta, rows,
-                                                                (const float*)weight, (bf16_t*)out, hidden, eps);
+        launch_add_rmsnorm<bf16_t, float>(resid, delta, rows, weight, out, R, hidden, eps, stream);
     else
         return TM_ERR_ARG;
     TM_CHECK_LAUNCH();
@@ -104,37 +179,43 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int H, int KVH, int D,
                                      const float* __restrict__ cos_t, const float* __restrict__ sin_t,
                                      const int* __restrict__ positions, const int* __restrict__ slots,
                                      T* __restrict__ k_pool, T* __restrict__ v_pool, int page, int write_kv) {
-    const int t = blockIdx.x, hh = blockIdx.y;
+    // one block per token; its threads walk (head, pair) for q and k and (head, d) for v
+    const int t = blockIdx.x;
     const int width = (H + 2 * KVH) * D;
-    T* x = qkv + (size_t)t * width + (size_t)hh * D;
-    const bool is_q = hh < H, is_k = !is_q && hh < H + KVH;
+    T* row = qkv + (size_t)t * width;
     const int slot = slots ? slots[t] : -1;
-    const bool store = write_kv && slot >= 0 && !is_q;
-    if (is_q || is_k) {
-        T* dst = nullptr;
-        if (store) dst = k_pool + ((size_t)slot * KVH + (hh - H)) * D;
-        const int half = rot / 2;
-        if (cos_t) {
-            const float* c = cos_t + (size_t)positions[t] * half;
-            const float* s = sin_t + (size_t)positions[t] * half;
-            for (int j = threadIdx.x; j < half; j += blockDim.x) {
-                const float x1 = Elem<T>::load(x + j), x2 = Elem<T>::load(x + j + half);
-                const float y1 = x1 * c[j] - x2 * s[j];
-                const float y2 = x2 * c[j] + x1 * s[j];
-                Elem<T>::store(x + j, y1);
-                Elem<T>::store(x + j + half, y2);
-                if (dst) { Elem<T>::store(dst + j, y1); Elem<T>::store(dst + j + half, y2); }
+    const bool store = write_kv && slot >= 0;
+    const int half = rot / 2;
+    const float* c = cos_t ? cos_t + (size_t)positions[t] * half : nullptr;
+    const float* s = cos_t ? sin_t + (size_t)positions[t] * half : nullptr;
+    if (cos_t) {
+        for (int idx = threadIdx.x; idx < (H + KVH) * half; idx += blockDim.x) {
+            const int hh = idx / half, j = idx - hh * half;
+            T* x = row + (size_t)hh * D;
+            const float x1 = Elem<T>::load(x + j), x2 = Elem<T>::load(x + j + half);
+            const float y1 = x1 * c[j] - x2 * s[j];
+            const float y2 = x2 * c[j] + x1 * s[j];
+            Elem<T>::store(x + j, y1);
+            Elem<T>::store(x + j + half, y2);
+            if (store && hh >= H) {
+                T* dst = k_pool + ((size_t)slot * KVH + (hh - H)) * D;
+                Elem<T>::store(dst + j, y1);
+                Elem<T>::store(dst + j + half, y2);
             }
-            if (dst)
-                for (int j = rot + threadIdx.x; j < D; j += blockDim.x) dst[j] = x[j];
-        } else if (dst) {
-            for (int j = threadIdx.x; j < D; j += blockDim.x) dst[j] = x[j];
         }
-    } else if (store) {
-        const int kvh = hh - H - KVH;
-        const int pg = slot / page, in_page = slot % page;
-        T* dst = v_pool + ((size_t)pg * KVH + kvh) * D * page + in_page;
-        for (int j = threadIdx.x; j < D; j += blockDim.x) dst[(size_t)j * page] = x[j];
+    }
+    if (!store) return;
+    // the part of k that is not rotated (all of it without a table) and v
+    const int tail = D - rot * (cos_t ? 1 : 0);
+    const int k_from = cos_t ? rot : 0;
+    for (int idx = threadIdx.x; idx < KVH * tail; idx += blockDim.x) {
+        const int kvh = idx / tail, j = k_from + idx - kvh * tail;
+        k_pool[((size_t)slot * KVH + kvh) * D + j] = row[(size_t)(H + kvh) * D + j];
+    }
+    const int pg = slot / page, in_page = slot % page;
+    for (int idx = threadIdx.x; idx < KVH * D; idx += blockDim.x) {
+        const int kvh = idx / D, j = idx - kvh * D;
+        v_pool[(((size_t)pg * KVH + kvh) * D + j) * page + in_page] = row[(size_t)(H + KVH + kvh) * D + j];
     }
 }
 
@@ -146,12 +227,12 @@ extern "C" int tm_rope_kv_write(void* qkv, int dtype, int T, int H, int KVH, int
     if (H <= 0 || KVH <= 0 || D <= 0 || rot < 0 || rot > D || (rot & 1)) return TM_ERR_ARG;
     if (cos_t && (!sin_t || !positions)) return TM_ERR_ARG;
     if (write_kv && (!slots || !k_pool || !v_pool || page <= 0)) return TM_ERR_ARG;
-    dim3 grid(T, H + 2 * KVH);
+    const int grid = T;
     if (dtype == TM_F32)
-        rope_kv_write_kernel<float><<<grid, 64, 0, stream>>>((float*)qkv, H, KVH, D, rot, cos_t, sin_t, positions,
+        rope_kv_write_kernel<float><<<grid, 256, 0, stream>>>((float*)qkv, H, KVH, D, rot, cos_t, sin_t, positions,
                                                             slots, (float*)k_pool, (float*)v_pool, page, write_kv);
     else if (dtype == TM_BF16)
-        rope_kv_write_kernel<bf16_t><<<grid, 64, 0, stream>>>((bf16_t*)qkv, H, KVH, D, rot, cos_t, sin_t,
+        rope_kv_write_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)qkv, H, KVH, D, rot, cos_t, sin_t,
                                                              positions, slots, (bf16_t*)k_pool, (bf16_t*)v_pool,
                                                              page, write_kv);
     else
@@ -175,10 +256,40 @@ __global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, i
     }
 }
 
+// bfloat16 rows whose width is a multiple of 8: eight elements (16 bytes) per thread and step
+__global__ void silu_mul_bf16x8_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ out, int I, size_t groups) {
+    const int per_row = I / 8;
+    for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < groups;
+         idx += (size_t)gridDim.x * blockDim.x) {
+        const size_t t = idx / per_row;
+        const int i = (int)(idx - t * per_row) * 8;
+        const uint4 gv = *(const uint4*)(gu + t * 2 * I + i);
+        const uint4 uv = *(const uint4*)(gu + t * 2 * I + I + i);
+        const uint32_t gw[4] = {gv.x, gv.y, gv.z, gv.w}, uw[4] = {uv.x, uv.y, uv.z, uv.w};
+        uint32_t ow[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const float g0 = __uint_as_float(gw[k] << 16), g1 = __uint_as_float(gw[k] & 0xffff0000u);
+            const float u0 = __uint_as_float(uw[k] << 16), u1 = __uint_as_float(uw[k] & 0xffff0000u);
+            const float r0 = g0 / (1.f + expf(-g0)) * u0, r1 = g1 / (1.f + expf(-g1)) * u1;
+            ow[k] = (uint32_t)f32_to_bf16(r0) | ((uint32_t)f32_to_bf16(r1) << 16);
+        }
+        *(uint4*)(out + t * I + i) = uint4{ow[0], ow[1], ow[2], ow[3]};
+    }
+}
+
 extern "C" int tm_silu_mul(const void* gu, void* out, int dtype, int T, int I, hipStream_t stream) {
     if (T <= 0) return TM_OK;
     if (I <= 0) return TM_ERR_ARG;
     const size_t total = (size_t)T * I;
+    if (dtype == TM_BF16 && I % 8 == 0 && ((uintptr_t)gu % 16) == 0 && ((uintptr_t)out % 16) == 0) {
+        const size_t groups = total / 8;
+        size_t want = (groups + 255) / 256;
+        silu_mul_bf16x8_kernel<<<(int)(want < 65536 ? want : 65536), 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out,
+                                                                                  I, groups);
+        TM_CHECK_LAUNCH();
+        return TM_OK;
+    }
     size_t want = (total + 255) / 256;
     const int blocks = (int)(want < 16384 ? want : 16384);
     if (dtype == TM_F32)
