@@ -42,6 +42,7 @@ class _Bucket:
         host[self.seq_of[0]:self.seq_of[1]] = np.arange(B)
         host[self.cu[0]:self.cu[1]] = np.arange(B + 1)
         host[self.rows[0]:self.rows[1]] = np.arange(B)
+        self.rows_held: list[list] = [[None] * B for _ in range(n_groups)]   # whose table each row holds
         self.graph: torch.cuda.CUDAGraph | None = None
         self.logits: torch.Tensor | None = None
 
@@ -112,14 +113,23 @@ class DecodeGraphs:
             slots = host[bk.g_slot[g][0]:bk.g_slot[g][1]]
             tabs = host[bk.g_tab[g][0]:bk.g_tab[g][1]].reshape(B, W)
             slots[:] = -1
+            windowed = runner.pools.groups[g].window is not None
+            rows = bk.rows_held[g]
             for i, e in enumerate(entries):
                 table = e.cache.tables[g]
                 need = e.start // page + 1
                 if len(table) < need or table[need - 1] == RELEASED:
                     raise ValueError(f"{e.cache.request_id}: no page for position {e.start}")
-                row = np.asarray(table[:need], dtype=np.int64)
-                tabs[i, :need] = np.where(row == RELEASED, 0, row)
+                # a row that held this request's table last time only needs its new pages
+                held = rows[i]
+                have = held[1] if (held is not None and held[0] is e.cache and not windowed and held[1] <= need) else 0
+                if have < need:
+                    row = np.asarray(table[have:need], dtype=np.int64)
+                    tabs[i, have:need] = np.where(row == RELEASED, 0, row)
+                rows[i] = (e.cache, need)
                 slots[i] = table[need - 1] * page + e.start % page
+            for i in range(n, B):
+                rows[i] = None
         bk.dev.copy_(bk.pinned, non_blocking=True)
         self._copied.record()
         if bk.graph is None:
