@@ -174,6 +174,22 @@ def test_command_line(model_dirs, plains):
     verify(plains["A"], [4, 5], lines[1]["output_ids"], torch.float32)
 
 
+def test_command_line_random_weights(model_dirs):
+    """--random CONFIG: weights drawn on the device from --weights-seed; the same seed gives the same tokens,
+    another seed another model."""
+    def run(seed):
+        r = subprocess.run([sys.executable, "-m", "tokenmill_amd.generate", "--random", str(model_dirs["B"]),
+                            "--weights-seed", str(seed), "--prompt-lens", "9,4", "--max-tokens", "8", "--ignore-eos",
+                            "--num-blocks", "16", "--max-model-len", "64", "--block-size", "8"],
+                           capture_output=True, text=True, cwd=ROOT, timeout=300)
+        assert r.returncode == 0, r.stderr[-2000:]
+        return [json.loads(ln)["output_ids"] for ln in r.stdout.splitlines() if ln.startswith("{")]
+    first, again, other = run(3), run(3), run(4)
+    assert [len(o) for o in first] == [8, 8]
+    assert first == again
+    assert first != other
+
+
 @pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
 def test_decode_steps_replayed_from_hip_graphs(model_dirs, plains, dtype_name):
     """Graph replays between eager prefill steps, batch sizes that change as requests come and go:

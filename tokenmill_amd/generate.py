@@ -4,6 +4,10 @@ engine flags, plus where the prompts come from and how to sample.
 
     python -m tokenmill_amd.generate --model DIR --prompt-ids "1,2,3;4,5" --max-tokens 16
     python -m tokenmill_amd.generate --model DIR --prompt-lens 5,17,33 --prompt-seed 0 --temperature 0.8
+    python -m tokenmill_amd.generate --random CONFIG.json --weights-seed 1 --prompt-lens 64 --max-tokens 32
+
+``--random`` takes a config.json (or a folder holding one) and draws the weights on the device
+from ``--weights-seed`` instead of reading a checkpoint.
 
 Token ids in, token ids out (one JSON line per prompt).
 """
@@ -20,6 +24,9 @@ from tokenmill_amd.config.engine_config import add_engine_args, engine_config_fr
 def main(argv=None) -> int:
     parser = argparse.ArgumentParser(description="tokenmill_amd: continuous-batching generation on one MI355X")
     add_engine_args(parser)
+    parser.add_argument("--random", default=None, metavar="CONFIG",
+                        help="a config.json (or its folder): run it with random weights instead of --model")
+    parser.add_argument("--weights-seed", type=int, default=0, help="seed of the random weights")
     parser.add_argument("--prompt-ids", default=None, help='prompts as token ids: "1,2,3;4,5"')
     parser.add_argument("--prompt-lens", default=None, help="lengths of uniform-random prompts: 5,17,33")
     parser.add_argument("--prompt-seed", type=int, default=0)
@@ -34,8 +41,8 @@ def main(argv=None) -> int:
     logging.basicConfig(level=args.log_level.upper(), format="%(asctime)s %(levelname)s %(name)s: %(message)s")
     if args.debug_steps:
         logging.getLogger("tokenmill_amd.engine").setLevel(logging.INFO)
-    if not args.model:
-        parser.error("--model DIR is required")
+    if bool(args.model) == bool(args.random):
+        parser.error("give exactly one of --model DIR and --random CONFIG")
     if (args.prompt_ids is None) == (args.prompt_lens is None):
         parser.error("give exactly one of --prompt-ids and --prompt-lens")
 
@@ -44,7 +51,18 @@ def main(argv=None) -> int:
     from tokenmill_amd.engine.engine import LLMEngine
     from tokenmill_amd.sampling.sampler import SamplingParams
 
-    engine = LLMEngine(engine_config_from_args(args))
+    cfg = engine_config_from_args(args)
+    model = None
+    if args.random:
+        from pathlib import Path
+
+        from tokenmill_amd.engine.loading import load_random_model, resolve_device, resolve_dtype
+
+        path = Path(args.random)
+        config = json.loads((path / "config.json" if path.is_dir() else path).read_text())
+        model = load_random_model(config, args.weights_seed, resolve_dtype(cfg.dtype), resolve_device(cfg.device),
+                                  max_positions=cfg.max_model_len)
+    engine = LLMEngine(cfg, model=model)
     if args.prompt_ids is not None:
         prompts = [[int(t) for t in part.split(",") if t.strip()] for part in args.prompt_ids.split(";") if part.strip()]
     else:
