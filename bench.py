@@ -63,6 +63,7 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (named in config)")
     ap.add_argument("--no-graphs", action="store_true", help="launch decode steps kernel by kernel")
+    ap.add_argument("--no-tune", action="store_true", help="keep the library's first choice of matrix-product algorithm")
     ap.add_argument("--skip-points", action="store_true", help="only the headline batch and the prefill")
     ap.add_argument("--part", default="all", choices=["all", "decode", "prefill"],
                     help="run only the decode steps or only the prefill (for profiling one of them)")
@@ -94,7 +95,7 @@ def main() -> int:
         pages = batch * (-(-(PROMPT_LEN + args.steps + args.warmup + 64) // BLOCK_SIZE)) + 8
         cfg = EngineConfig(dtype=args.dtype, block_size=BLOCK_SIZE, num_blocks=pages, max_model_len=MAX_MODEL_LEN,
                            max_num_seqs=max(batch, 1), max_num_batched_tokens=max(PROMPT_LEN, batch),
-                           watermark=0.0, hip_graphs=not args.no_graphs)
+                           watermark=0.0, hip_graphs=not args.no_graphs, tune_gemm=not args.no_tune)
         return LLMEngine(cfg, model=model)
 
     def time_decode(batch, steps, warmup):
@@ -164,7 +165,7 @@ def main() -> int:
                    "intermediate": shape["intermediate_size"], "vocab": shape["vocab_size"], "tied": True,
                    "global_batch": args.batch, "seq_len": PROMPT_LEN, "context": context,
                    "max_model_len": MAX_MODEL_LEN, "block_size": BLOCK_SIZE, "parallelism": "single GPU",
-                   "hip_graphs": not args.no_graphs},
+                   "hip_graphs": not args.no_graphs, "tune_gemm": not args.no_tune},
         "prefill": {"value": round(PROMPT_LEN / prefill_s, 1), "tokens": PROMPT_LEN, "ms": round(prefill_s * 1e3, 3),
                     "frac": round(flops / prefill_s / PEAK_FLOPS[args.dtype], 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",

@@ -28,9 +28,6 @@ union PFrag {
     bf16x8_t b;
 };
 
-#define AP_HPW 2            // query heads per wavefront
-#define AP_KSPLIT 4         // wavefronts of a block, each taking every fourth block of 32 keys
-
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef float f32x2_t __attribute__((ext_vector_type(2)));
 
@@ -46,206 +43,298 @@ struct KVBlock {
     u32x2_t v[D / 16][2];   // [d tile][16-key tile]: 4 keys each
 };
 
+// What a lane adds to a tile's (wave-uniform) base address: constant for the whole kernel.
+struct LaneOffsets {
+    uint32_t k;             // bytes: key r of the tile, d = 8 g
+    uint32_t v;             // bytes: d = r, keys 4 g .. 4 g + 3 of the tile
+};
+
+// A raw buffer descriptor over memory that starts at a wave-uniform address: loads through it take
+// the base from scalar registers and a 32-bit offset per lane, so no lane computes a 64-bit address.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t uniform_buffer(const void* base) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, 0x7fffffff, 0x00020000);
+}
+
+// The pages of the next 32 key blocks of a wavefront (blocks kb, kb + KS, ...), one 16-key tile per
+// lane: lane 2 i + t holds the page of tile t of block kb + i * KS. A tile that holds no key any
+// query of this wavefront may see (beyond the newest key, or wholly behind the window) is replaced
+// by the nearest tile that does: its table entry may name no page. The caller masks every score of
+// such a tile by the key's real position, so what is loaded in its place only has to be finite.
+template <int KS>
+__device__ __forceinline__ int2 lane_pages(int kb, int lane, int first_tile, int last_tile,
+                                           const int* __restrict__ table, int page_shift) {
+    int tile = 2 * (kb + (lane >> 1) * KS) + (lane & 1);
+    tile = tile < first_tile ? first_tile : (tile > last_tile ? last_tile : tile);
+    const int tile0 = 16 * tile;
+    return int2{table[tile0 >> page_shift], tile0 & ((1 << page_shift) - 1)};
+}
+
+// Loads one block of 32 keys (two tiles of 16); slot = which of the 32 blocks held in `pages`.
 template <int D>
-__device__ __forceinline__ void load_kv_block(KVBlock<D>& blk, int kb, int first_key, int last_key,
-                                              const int* __restrict__ table,
+__device__ __forceinline__ void load_kv_block(KVBlock<D>& blk, int2 pages, int slot,
                                               const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
-                                              int kvh, int KVH, int page_shift, int r, int g) {
-    const int page = 1 << page_shift;
+                                              int kvh, int KVH, int page_shift, LaneOffsets off) {
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
-        const int tile0 = kb * 32 + 16 * t;
-        if (tile0 <= last_key && tile0 + 15 >= first_key) {         // wave-uniform: the tile holds a visible key
-            const int pg = table[tile0 >> page_shift];
-            const int in_page = tile0 & (page - 1);
-            const bf16_t* kr = k_pool + ((((size_t)pg << page_shift) + in_page + r) * KVH + kvh) * D + 8 * g;
+        const int pg = __builtin_amdgcn_readlane(pages.x, 2 * slot + t);                    // wave-uniform
+        const int in_page = __builtin_amdgcn_readlane(pages.y, 2 * slot + t);
+        const __amdgpu_buffer_rsrc_t kbuf =
+            uniform_buffer(k_pool + ((((size_t)pg << page_shift) + in_page) * KVH + kvh) * D);
+        const __amdgpu_buffer_rsrc_t vbuf =
+            uniform_buffer(v_pool + ((((size_t)pg * KVH + kvh) * D) << page_shift) + in_page);
 #pragma unroll
-            for (int c = 0; c < D / 32; ++c) blk.k[t][c].u = *(const u32x4_t*)(kr + 32 * c);
-            const bf16_t* vr = v_pool + ((((size_t)pg * KVH + kvh) * D + r) << page_shift) + in_page + 4 * g;
+        for (int c = 0; c < D / 32; ++c)
+            blk.k[t][c].u = __builtin_amdgcn_raw_buffer_load_b128(kbuf, off.k, 64 * c, 0);
 #pragma unroll
-            for (int dt = 0; dt < D / 16; ++dt) blk.v[dt][t] = *(const u32x2_t*)(vr + ((size_t)(16 * dt) << page_shift));
-        } else {
+        for (int dt = 0; dt < D / 16; ++dt)
+            blk.v[dt][t] = __builtin_amdgcn_raw_buffer_load_b64(vbuf, off.v, (32 * dt) << page_shift, 0);
+    }
+}
+
+// maximum over the four lanes (r, 0..3) that hold one query column
+__device__ __forceinline__ float column_max(float v) {
+    const uint32_t u = __float_as_uint(v);
+    const auto a = __builtin_amdgcn_permlane32_swap(u, u, false, false);     // lanes l and l ^ 32
+    const float m32 = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+    const uint32_t w = __float_as_uint(m32);
+    const auto b = __builtin_amdgcn_permlane16_swap(w, w, false, false);     // lanes l and l ^ 16
+    return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+
+// Running softmax state of the query heads a wavefront works on.
+//   m: running maximum of (score * scale * log2 e) of this lane's column; l: this lane's share of
+//   the running sum (its 8 keys of every block), reduced over the lanes of a column at the end
+template <int D, int HPW>
+struct HeadState {
+    float m[HPW], l[HPW];
+    f32x4_t o[HPW][D / 16];
+};
+
+// What a wavefront knows about the tile it works on (all wave-uniform but my_pos and my_lo).
+struct TileView {
+    int pos0;               // position of the tile's first query
+    int last_key;           // newest key any query of the tile sees
+    int last_lo;            // oldest key the tile's last query sees (0 without a window)
+    int my_pos, my_lo;      // this lane's query column: its position and the oldest key it sees
+};
+
+// One block of 32 keys against the wavefront's heads.
+template <int D, int HPW>
+__device__ __forceinline__ void attend_block(KVBlock<D>& blk, HeadState<D, HPW>& st, const PFrag (&qf)[HPW][D / 32],
+                                             int key0, int nh, const TileView& tv, int g, float scale_log2) {
+    constexpr int NDC = D / 32, NDT = D / 16;
+    // values of keys nobody may see (beyond the newest key) can hold anything: clear them
+    if (key0 + 31 > tv.last_key) {
 #pragma unroll
-            for (int c = 0; c < D / 32; ++c) blk.k[t][c].u = u32x4_t{0, 0, 0, 0};
+        for (int t = 0; t < 2; ++t) {
+            const int k0 = key0 + 16 * t + 4 * g;
+            const uint32_t keep0 = ((k0 <= tv.last_key) ? 0x0000ffffu : 0u) | ((k0 + 1 <= tv.last_key) ? 0xffff0000u : 0u);
+            const uint32_t keep1 = ((k0 + 2 <= tv.last_key) ? 0x0000ffffu : 0u) | ((k0 + 3 <= tv.last_key) ? 0xffff0000u : 0u);
 #pragma unroll
-            for (int dt = 0; dt < D / 16; ++dt) blk.v[dt][t] = u32x2_t{0, 0};
+            for (int dt = 0; dt < NDT; ++dt) {
+                blk.v[dt][t][0] &= keep0;
+                blk.v[dt][t][1] &= keep1;
+            }
+        }
+    }
+    // does any (query, key) pair of this block fall outside the causal / window limits?
+    const bool edge = (key0 + 31 > tv.pos0) || (key0 < tv.last_lo);
+    // all score products first: the matrix unit works on the next head's while the vector unit
+    // does the softmax of this one
+    f32x4_t sc[HPW][2];
+#pragma unroll
+    for (int hh = 0; hh < HPW; ++hh) {
+        if (hh >= nh) continue;                                  // wave-uniform
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int c = 0; c < NDC; ++c)
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(blk.k[t][c].b, qf[hh][c].b, acc, 0, 0, 0);
+            sc[hh][t] = acc;
+        }
+    }
+#pragma unroll
+    for (int hh = 0; hh < HPW; ++hh) {
+        if (hh >= nh) continue;                                  // wave-uniform
+        if (edge) {
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int kj = key0 + 16 * t + 4 * g + i;
+                    if (kj > tv.my_pos || kj < tv.my_lo) sc[hh][t][i] = -INFINITY;
+                }
+        }
+        float bm = fmaxf(fmaxf(fmaxf(sc[hh][0][0], sc[hh][0][1]), fmaxf(sc[hh][0][2], sc[hh][0][3])),
+                         fmaxf(fmaxf(sc[hh][1][0], sc[hh][1][1]), fmaxf(sc[hh][1][2], sc[hh][1][3])));
+        bm = column_max(bm) * scale_log2;                        // scale > 0: the maximum commutes with it
+        if (__any(bm > st.m[hh])) {                              // some column's maximum grew: rescale
+            const float m_new = fmaxf(st.m[hh], bm);
+            const float corr = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(st.m[hh] - m_new);
+            st.m[hh] = m_new;
+            st.l[hh] *= corr;
+#pragma unroll
+            for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) st.o[hh][dt][i] *= corr;
+        }
+        // a column that has seen no key yet (m = -inf) gets zeros: exp2(-inf - 0)
+        const float neg_m = (st.m[hh] == -INFINITY) ? 0.f : -st.m[hh];
+        float pr[2][4];
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                pr[t][i] = __builtin_amdgcn_exp2f(fmaf(sc[hh][t][i], scale_log2, neg_m));
+                st.l[hh] += pr[t][i];
+            }
+        PFrag pt;
+        pt.u = u32x4_t{pk_bf16(pr[0][0], pr[0][1]), pk_bf16(pr[0][2], pr[0][3]), pk_bf16(pr[1][0], pr[1][1]),
+                       pk_bf16(pr[1][2], pr[1][3])};
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt) {
+            PFrag vf;
+            vf.u = u32x4_t{blk.v[dt][0][0], blk.v[dt][0][1], blk.v[dt][1][0], blk.v[dt][1][1]};
+            st.o[hh][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.b, pt.b, st.o[hh][dt], 0, 0, 0);
         }
     }
 }
 
 // tiles: int32 [n_tiles][4] = (request index in the step, first row of the tile in the flat batch,
 //                              tokens in the tile (1..16), position of its first token)
-// A block is AP_KSPLIT wavefronts on the same tile and heads; wavefront j takes the key blocks kb
-// with kb % AP_KSPLIT == j and the partial results are merged through LDS in wavefront order.
-// Which blocks a wavefront takes depends on absolute positions only, and a block in which a token
-// sees no key changes nothing for it, so a token's bits do not depend on the tile it falls into.
-// (two blocks per CU where the head size leaves room: a second wavefront per SIMD hides the first one's loads)
-template <int D>
-__global__ __launch_bounds__(64 * AP_KSPLIT, D <= 64 ? 3 : 1) void attn_prefill_mfma_kernel(
+// A block is KS wavefronts on the same tile and heads; wavefront j takes the key blocks kb with
+// kb % KS == j and the partial results are merged through LDS in wavefront order. Which blocks a
+// wavefront takes depends on absolute positions only, and a block in which a token sees no key
+// changes nothing for it, so a token's bits do not depend on the tile it falls into.
+// With pair != 0 a block takes tile b and then tile n_tiles - 1 - b: in a table sorted by the
+// number of keys a tile sees, the longest goes with the shortest and every block has the same work
+// (the lower triangle of a prompt, folded).
+template <int D, int HPW, int KS>
+__global__ __launch_bounds__(64 * KS) void attn_prefill_mfma_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
     const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool, const int* __restrict__ block_tables,
-    int table_width, const int* __restrict__ tiles, int H, int KVH, int page_shift, float scale_log2, int window) {
+    int table_width, const int* __restrict__ tiles, int n_tiles, int pair, int H, int KVH, int page_shift,
+    float scale_log2, int window) {
     constexpr int NDC = D / 32, NDT = D / 16;
-    __shared__ float s_m[AP_KSPLIT][16], s_l[AP_KSPLIT][16];
-    __shared__ float s_o[AP_KSPLIT][16][D + 1];
-    const int wave = threadIdx.x / TM_WAVE, lane = threadIdx.x % TM_WAVE, r = lane % 16, g = lane / 16;
+    __shared__ float s_m[KS][16], s_l[KS][16];
+    __shared__ float s_o[KS][16][D + 1];
+    // the wavefront index in a scalar register: everything derived from it (its key blocks, their
+    // pages, the branches on them) stays wave-uniform
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / TM_WAVE);
+    const int lane = threadIdx.x % TM_WAVE, r = lane % 16, g = lane / 16;
     const int G = H / KVH;
-    const int splits = (G + AP_HPW - 1) / AP_HPW;
+    const int splits = (G + HPW - 1) / HPW;
     const int kvh = blockIdx.y / splits, split = blockIdx.y % splits;
-    const int h0 = kvh * G + split * AP_HPW;
-    const int nh = (G - split * AP_HPW) < AP_HPW ? (G - split * AP_HPW) : AP_HPW;
-    const int* tl = tiles + (size_t)blockIdx.x * 4;
-    const int s = tl[0], row0 = tl[1], valid = tl[2], pos0 = tl[3];
-    const int* table = block_tables + (size_t)s * table_width;
-    const int last_key = pos0 + valid - 1;                           // newest key any query of the tile sees
-    const int my_pos = pos0 + r < last_key ? pos0 + r : last_key;    // position of this lane's query column
-    const int my_lo = (window > 0 && my_pos - window + 1 > 0) ? my_pos - window + 1 : 0;
-    const int first_key = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
-    const int last_lo = (window > 0 && last_key - window + 1 > 0) ? last_key - window + 1 : 0;
-    const int kb0 = first_key / 32, kb1 = last_key / 32;
+    const int h0 = kvh * G + split * HPW;
+    const int nh = (G - split * HPW) < HPW ? (G - split * HPW) : HPW;
+    LaneOffsets off;
+    off.k = (uint32_t)(((size_t)r * KVH * D + 8 * g) * sizeof(bf16_t));
+    off.v = (uint32_t)((((size_t)r << page_shift) + 4 * g) * sizeof(bf16_t));
+    const int other = n_tiles - 1 - (int)blockIdx.x;
+    const int n_mine = (pair && other > (int)blockIdx.x) ? 2 : 1;
 
-    PFrag qf[AP_HPW][NDC];
+#pragma unroll 1
+    for (int which = 0; which < n_mine; ++which) {
+        const int* tl = tiles + (size_t)(which ? other : (int)blockIdx.x) * 4;
+        const int s = tl[0], row0 = tl[1], valid = tl[2], pos0 = tl[3];
+        const int* table = block_tables + (size_t)s * table_width;
+        TileView tv;
+        tv.pos0 = pos0;
+        tv.last_key = pos0 + valid - 1;
+        tv.my_pos = pos0 + r < tv.last_key ? pos0 + r : tv.last_key;
+        tv.my_lo = (window > 0 && tv.my_pos - window + 1 > 0) ? tv.my_pos - window + 1 : 0;
+        tv.last_lo = (window > 0 && tv.last_key - window + 1 > 0) ? tv.last_key - window + 1 : 0;
+        const int first_key = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
+        const int kb0 = first_key / 32, kb1 = tv.last_key / 32;
+        const int first_tile = first_key / 16, last_tile = tv.last_key / 16;
+
+        PFrag qf[HPW][NDC];
 #pragma unroll
-    for (int hh = 0; hh < AP_HPW; ++hh)
+        for (int hh = 0; hh < HPW; ++hh)
 #pragma unroll
-        for (int c = 0; c < NDC; ++c) {
-            if (hh < nh && r < valid)
-                qf[hh][c].u = *(const u32x4_t*)(q + (size_t)(row0 + r) * q_stride + (size_t)(h0 + hh) * D + 32 * c + 8 * g);
-            else
-                qf[hh][c].u = u32x4_t{0, 0, 0, 0};
+            for (int c = 0; c < NDC; ++c) {
+                if (hh < nh && r < valid)
+                    qf[hh][c].u = *(const u32x4_t*)(q + (size_t)(row0 + r) * q_stride + (size_t)(h0 + hh) * D + 32 * c + 8 * g);
+                else
+                    qf[hh][c].u = u32x4_t{0, 0, 0, 0};
+            }
+        HeadState<D, HPW> st;
+#pragma unroll
+        for (int hh = 0; hh < HPW; ++hh) {
+            st.m[hh] = -INFINITY;
+            st.l[hh] = 0.f;
+#pragma unroll
+            for (int dt = 0; dt < NDT; ++dt) st.o[hh][dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
         }
-    // m: running maximum of (score * scale * log2 e) of this lane's column; l: this lane's share of
-    // the running sum (its 8 keys of every block), reduced over the lanes of a column at the end
-    float m[AP_HPW], l[AP_HPW];
-    f32x4_t o[AP_HPW][NDT];
-#pragma unroll
-    for (int hh = 0; hh < AP_HPW; ++hh) {
-        m[hh] = -INFINITY;
-        l[hh] = 0.f;
-#pragma unroll
-        for (int dt = 0; dt < NDT; ++dt) o[hh][dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-    }
 
-    int kb = kb0 + ((wave - kb0) & (AP_KSPLIT - 1));                 // first block >= kb0 of this wavefront
-    KVBlock<D> cur, nxt;
-    if (kb <= kb1) load_kv_block<D>(cur, kb, first_key, last_key, table, k_pool, v_pool, kvh, KVH, page_shift, r, g);
-    for (; kb <= kb1; kb += AP_KSPLIT) {
-        const bool more = kb + AP_KSPLIT <= kb1;
-        if (more)
-            load_kv_block<D>(nxt, kb + AP_KSPLIT, first_key, last_key, table, k_pool, v_pool, kvh, KVH, page_shift, r, g);
-        const int key0 = kb * 32;
-        // values of keys nobody may see (beyond the newest key) can hold anything: clear them
-        if (key0 + 31 > last_key) {
+        // Two register sets take turns: one is worked on while the other's loads are in flight. The
+        // load after the last block repeats it, unused, so that no load hides behind a branch.
+        int kb = kb0 + ((wave - kb0) & (KS - 1));                    // first block >= kb0 of this wavefront
+        KVBlock<D> ba, bb;
+        int2 pages = lane_pages<KS>(kb, lane, first_tile, last_tile, table, page_shift);
+        int slot = 0;                                                // block kb is slot `slot` of `pages`
+        if (kb <= kb1) load_kv_block<D>(ba, pages, 0, k_pool, v_pool, kvh, KVH, page_shift, off);
+        while (kb <= kb1) {
+            if (slot == 31) {                                        // the next block starts a new set of pages
+                pages = lane_pages<KS>(kb + KS, lane, first_tile, last_tile, table, page_shift);
+                slot = -1;
+            }
+            load_kv_block<D>(bb, pages, slot + 1, k_pool, v_pool, kvh, KVH, page_shift, off);
+            attend_block<D, HPW>(ba, st, qf, kb * 32, nh, tv, g, scale_log2);
+            kb += KS;
+            ++slot;
+            if (kb > kb1) break;
+            if (slot == 31) {
+                pages = lane_pages<KS>(kb + KS, lane, first_tile, last_tile, table, page_shift);
+                slot = -1;
+            }
+            load_kv_block<D>(ba, pages, slot + 1, k_pool, v_pool, kvh, KVH, page_shift, off);
+            attend_block<D, HPW>(bb, st, qf, kb * 32, nh, tv, g, scale_log2);
+            kb += KS;
+            ++slot;
+        }
+
+        // merge the wavefronts' partials head by head, in wavefront order; lane: d = 16 dt + 4 g + i of token r
 #pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                const int k0 = key0 + 16 * t + 4 * g;
-                const uint32_t keep0 = ((k0 <= last_key) ? 0x0000ffffu : 0u) | ((k0 + 1 <= last_key) ? 0xffff0000u : 0u);
-                const uint32_t keep1 = ((k0 + 2 <= last_key) ? 0x0000ffffu : 0u) | ((k0 + 3 <= last_key) ? 0xffff0000u : 0u);
+        for (int hh = 0; hh < HPW; ++hh) {
+            if (hh >= nh) continue;                                  // block-uniform
+            float lsum = st.l[hh];
+            lsum += __shfl_xor(lsum, 16, TM_WAVE);
+            lsum += __shfl_xor(lsum, 32, TM_WAVE);
+            if (g == 0) {
+                s_m[wave][r] = st.m[hh];
+                s_l[wave][r] = lsum;
+            }
 #pragma unroll
-                for (int dt = 0; dt < NDT; ++dt) {
-                    cur.v[dt][t][0] &= keep0;
-                    cur.v[dt][t][1] &= keep1;
+            for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) s_o[wave][r][16 * dt + 4 * g + i] = st.o[hh][dt][i];
+            __syncthreads();
+            for (int idx = threadIdx.x; idx < 16 * (D / 2); idx += 64 * KS) {
+                const int col = idx / (D / 2), d = 2 * (idx % (D / 2));
+                if (col >= valid) continue;
+                float mm = s_m[0][col];
+#pragma unroll
+                for (int w = 1; w < KS; ++w) mm = fmaxf(mm, s_m[w][col]);
+                float ll = 0.f, o0 = 0.f, o1 = 0.f;
+#pragma unroll
+                for (int w = 0; w < KS; ++w) {
+                    const float f = (s_m[w][col] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(s_m[w][col] - mm);
+                    ll = fmaf(s_l[w][col], f, ll);
+                    o0 = fmaf(s_o[w][col][d], f, o0);
+                    o1 = fmaf(s_o[w][col][d + 1], f, o1);
                 }
+                const float inv = 1.f / ll;
+                *(uint32_t*)(out + (size_t)(row0 + col) * out_stride + (size_t)(h0 + hh) * D + d) = pk_bf16(o0 * inv, o1 * inv);
             }
+            __syncthreads();
         }
-        // does any (query, key) pair of this block fall outside the causal / window limits?
-        const bool edge = (key0 + 31 > pos0) || (key0 < last_lo);
-#pragma unroll
-        for (int hh = 0; hh < AP_HPW; ++hh) {
-            if (hh >= nh) continue;                                  // wave-uniform
-            float sc[2][4];
-#pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int c = 0; c < NDC; ++c)
-                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.k[t][c].b, qf[hh][c].b, acc, 0, 0, 0);
-#pragma unroll
-                for (int i = 0; i < 4; ++i) sc[t][i] = acc[i];
-            }
-            if (edge) {
-#pragma unroll
-                for (int t = 0; t < 2; ++t)
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const int kj = key0 + 16 * t + 4 * g + i;
-                        if (kj > my_pos || kj < my_lo) sc[t][i] = -INFINITY;
-                    }
-            }
-            float bm = fmaxf(fmaxf(fmaxf(sc[0][0], sc[0][1]), fmaxf(sc[0][2], sc[0][3])),
-                             fmaxf(fmaxf(sc[1][0], sc[1][1]), fmaxf(sc[1][2], sc[1][3])));
-            bm = fmaxf(bm, __shfl_xor(bm, 16, TM_WAVE));
-            bm = fmaxf(bm, __shfl_xor(bm, 32, TM_WAVE));
-            bm *= scale_log2;                                        // scale > 0: the maximum commutes with it
-            if (__any(bm > m[hh])) {                                 // some column's maximum grew: rescale
-                const float m_new = fmaxf(m[hh], bm);
-                const float corr = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m[hh] - m_new);
-                m[hh] = m_new;
-                l[hh] *= corr;
-#pragma unroll
-                for (int dt = 0; dt < NDT; ++dt)
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) o[hh][dt][i] *= corr;
-            }
-            // a column that has seen no key yet (m = -inf) gets zeros: exp2(-inf - 0)
-            const float neg_m = (m[hh] == -INFINITY) ? 0.f : -m[hh];
-            float pr[2][4];
-#pragma unroll
-            for (int t = 0; t < 2; ++t)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    pr[t][i] = __builtin_amdgcn_exp2f(fmaf(sc[t][i], scale_log2, neg_m));
-                    l[hh] += pr[t][i];
-                }
-            PFrag pt;
-            pt.u = u32x4_t{pk_bf16(pr[0][0], pr[0][1]), pk_bf16(pr[0][2], pr[0][3]), pk_bf16(pr[1][0], pr[1][1]),
-                           pk_bf16(pr[1][2], pr[1][3])};
-#pragma unroll
-            for (int dt = 0; dt < NDT; ++dt) {
-                PFrag vf;
-                vf.u = u32x4_t{cur.v[dt][0][0], cur.v[dt][0][1], cur.v[dt][1][0], cur.v[dt][1][1]};
-                o[hh][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.b, pt.b, o[hh][dt], 0, 0, 0);
-            }
-        }
-        if (more) cur = nxt;
-    }
-
-    // merge the wavefronts' partials head by head, in wavefront order; lane: d = 16 dt + 4 g + i of token r
-#pragma unroll
-    for (int hh = 0; hh < AP_HPW; ++hh) {
-        if (hh >= nh) continue;                                      // block-uniform
-        float lsum = l[hh];
-        lsum += __shfl_xor(lsum, 16, TM_WAVE);
-        lsum += __shfl_xor(lsum, 32, TM_WAVE);
-        if (g == 0) {
-            s_m[wave][r] = m[hh];
-            s_l[wave][r] = lsum;
-        }
-#pragma unroll
-        for (int dt = 0; dt < NDT; ++dt)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) s_o[wave][r][16 * dt + 4 * g + i] = o[hh][dt][i];
-        __syncthreads();
-        for (int idx = threadIdx.x; idx < 16 * (D / 2); idx += 64 * AP_KSPLIT) {
-            const int col = idx / (D / 2), d = 2 * (idx % (D / 2));
-            if (col >= valid) continue;
-            float mm = s_m[0][col];
-#pragma unroll
-            for (int w = 1; w < AP_KSPLIT; ++w) mm = fmaxf(mm, s_m[w][col]);
-            float ll = 0.f, o0 = 0.f, o1 = 0.f;
-#pragma unroll
-            for (int w = 0; w < AP_KSPLIT; ++w) {
-                const float f = (s_m[w][col] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(s_m[w][col] - mm);
-                ll = fmaf(s_l[w][col], f, ll);
-                o0 = fmaf(s_o[w][col][d], f, o0);
-                o1 = fmaf(s_o[w][col][d + 1], f, o1);
-            }
-            const float inv = 1.f / ll;
-            *(uint32_t*)(out + (size_t)(row0 + col) * out_stride + (size_t)(h0 + hh) * D + d) = pk_bf16(o0 * inv, o1 * inv);
-        }
-        __syncthreads();
     }
 }
+
+// heads a wavefront takes and wavefronts a block has, by head size (registers decide)
+template <int D> struct PrefillShape { static constexpr int HPW = D <= 64 ? 4 : 2, KS = D <= 64 ? 8 : 4; };
 
 extern "C" int tm_attn_prefill_mfma(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
                                     const void* v_pool, const int* block_tables, int table_width, const int* tiles,
@@ -257,23 +346,27 @@ extern "C" int tm_attn_prefill_mfma(const void* q, int q_stride, void* out, int 
         out_stride < H * D || !(scale > 0.f))
         return TM_ERR_ARG;
     const int G = H / KVH;
-    const int splits = (G + AP_HPW - 1) / AP_HPW;
-    if ((long long)KVH * splits > 65535) return TM_ERR_ARG;
     int page_shift = 0;
     while ((1 << page_shift) < page) ++page_shift;
     const float scale_log2 = scale * 1.4426950408889634f;
-    dim3 grid(n_tiles, KVH * splits);
 #define TM_PREFILL_CASE(DD)                                                                                       \
-    case DD:                                                                                                      \
-        attn_prefill_mfma_kernel<DD><<<grid, 64 * AP_KSPLIT, 0, stream>>>(                                        \
+    case DD: {                                                                                                    \
+        constexpr int HPW = PrefillShape<DD>::HPW, KS = PrefillShape<DD>::KS;                                     \
+        const int splits = (G + HPW - 1) / HPW;                                                                   \
+        if ((long long)KVH * splits > 65535) return TM_ERR_ARG;                                                   \
+        /* fold the table in two once the folded launch still gives every CU a block */                          \
+        const int pair = (long long)(n_tiles / 2) * KVH * splits >= 256 ? 1 : 0;                                  \
+        dim3 grid(pair ? (n_tiles + 1) / 2 : n_tiles, KVH * splits);                                              \
+        attn_prefill_mfma_kernel<DD, HPW, KS><<<grid, 64 * KS, 0, stream>>>(                                      \
             (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool,   \
-            block_tables, table_width, tiles, H, KVH, page_shift, scale_log2, window);                            \
-        break
+            block_tables, table_width, tiles, n_tiles, pair, H, KVH, page_shift, scale_log2, window);             \
+        break;                                                                                                    \
+    }
     switch (D) {
-        TM_PREFILL_CASE(32);
-        TM_PREFILL_CASE(64);
-        TM_PREFILL_CASE(96);
-        TM_PREFILL_CASE(128);
+        TM_PREFILL_CASE(32)
+        TM_PREFILL_CASE(64)
+        TM_PREFILL_CASE(96)
+        TM_PREFILL_CASE(128)
         default:
             return TM_ERR_ARG;
     }

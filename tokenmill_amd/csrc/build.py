@@ -24,6 +24,10 @@ HIPCC_FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-Xclang"
                "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
 
 
+# the library matrix products (gemm_library.hip) call hipBLASLt
+LINK_LIBS = ["-lhipblaslt"]
+
+
 def sources() -> list[Path]:
     return sorted(CSRC.glob("*.hip"))
 
@@ -33,7 +37,7 @@ def source_digest() -> str:
     for p in sorted(list(CSRC.glob("*.hip")) + list(CSRC.glob("*.h"))):
         h.update(p.name.encode())
         h.update(p.read_bytes())
-    h.update(" ".join(HIPCC_FLAGS).encode())
+    h.update(" ".join(HIPCC_FLAGS + LINK_LIBS).encode())
     return h.hexdigest()[:16]
 
 
@@ -96,7 +100,7 @@ def build(verbose: bool = True) -> Path:
         objs = list(pool.map(compile_one, sources()))
     lib = out_dir / LIB_NAME
     tmp = out_dir / (LIB_NAME + f".tmp{os.getpid()}")
-    r = subprocess.run([cc, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", str(tmp), *map(str, objs)],
+    r = subprocess.run([cc, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", str(tmp), *map(str, objs), *LINK_LIBS],
                        capture_output=True, text=True, env=env)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc link failed:\n{r.stdout}\n{r.stderr}")

@@ -15,6 +15,7 @@
 #define TM_OK 0
 #define TM_ERR_ARG 1        // an argument the kernel cannot run with
 #define TM_ERR_LAUNCH 2     // the runtime refused the launch
+#define TM_ERR_UNSUPPORTED 3 // a library has no routine for the request: use another path
 
 typedef uint16_t bf16_t;    // bfloat16 bits
 

@@ -1,0 +1,204 @@
+// C[M, N] = A[M, K] * W[N, K]^T (+ bias) through hipBLASLt, for the large products of a prompt
+// step, where the reference also calls a library (F.linear, reference src/infer/model/layers.py:144-164).
+//
+// What this file adds to the library call is a cache: the descriptors and the algorithm the
+// library's heuristic picks for a (shape, strides, types, epilogue) are made once and kept, so that
+// a call after the first costs one hipblasLtMatmul launch. A prompt step makes about a hundred of
+// these calls; setting each of them up again costs more host time than the step's kernels take.
+//
+// hipBLASLt is column-major. Row-major C = A W^T is the column-major product C^T = W A^T:
+// first operand W as [K, N] with leading dimension ldw, transposed; second A as [K, M] with
+// leading dimension lda; result [N, M] with leading dimension ldc. The bias has one entry per row
+// of that result, i.e. per output feature, and is added to the 32-bit sum before rounding.
+#include <hipblaslt/hipblaslt.h>
+
+#include <mutex>
+#include <unordered_map>
+
+#include "common.h"
+#include "api.h"
+
+namespace {
+
+struct PlanKey {
+    int M, N, K, lda, ldw, ldc, bias_dtype, out_f32, device;
+    bool operator==(const PlanKey& o) const {
+        return M == o.M && N == o.N && K == o.K && lda == o.lda && ldw == o.ldw && ldc == o.ldc &&
+               bias_dtype == o.bias_dtype && out_f32 == o.out_f32 && device == o.device;
+    }
+};
+
+struct PlanKeyHash {
+    size_t operator()(const PlanKey& k) const {
+        size_t h = 1469598103934665603ull;
+        for (int v : {k.M, k.N, k.K, k.lda, k.ldw, k.ldc, k.bias_dtype, k.out_f32, k.device})
+            h = (h ^ (size_t)(uint32_t)v) * 1099511628211ull;
+        return h;
+    }
+};
+
+struct Plan {
+    hipblasLtMatmulDesc_t desc = nullptr;
+    hipblasLtMatrixLayout_t w = nullptr, a = nullptr, c = nullptr;
+    hipblasLtMatmulAlgo_t algo;
+    size_t workspace = 0;
+    bool ok = false;
+};
+
+struct Library {
+    std::mutex lock;
+    std::unordered_map<int, hipblasLtHandle_t> handles;          // one per device
+    std::unordered_map<PlanKey, Plan, PlanKeyHash> plans;
+};
+
+Library& lib() {
+    static Library* l = new Library();      // never destroyed: the runtime may be gone at exit
+    return *l;
+}
+
+// How many of the heuristic's candidates the first call of a shape times before it keeps the
+// fastest (0 or 1: keep the heuristic's first choice untimed).
+int g_tune_candidates = 0;
+
+struct Operands {
+    const void *A, *W, *bias;
+    void *C, *workspace;
+    size_t workspace_bytes;
+    hipStream_t stream;
+};
+
+// Mean time of a few runs of one algorithm on the caller's own operands (the result is the same
+// whichever algorithm wrote it last, up to rounding); negative if it fails.
+float time_algo(hipblasLtHandle_t handle, const Plan& p, const hipblasLtMatmulAlgo_t& algo, const Operands& op) {
+    const float one = 1.f, zero = 0.f;
+    hipEvent_t t0, t1;
+    if (hipEventCreate(&t0) != hipSuccess) return -1.f;
+    if (hipEventCreate(&t1) != hipSuccess) {
+        hipEventDestroy(t0);
+        return -1.f;
+    }
+    float ms = -1.f;
+    bool ok = true;
+    for (int i = 0; i < 2 + 5 && ok; ++i) {
+        if (i == 2) hipEventRecord(t0, op.stream);
+        ok = hipblasLtMatmul(handle, p.desc, &one, op.W, p.w, op.A, p.a, &zero, op.C, p.c, op.C, p.c, &algo, op.workspace,
+                             op.workspace_bytes, op.stream) == HIPBLAS_STATUS_SUCCESS;
+    }
+    hipEventRecord(t1, op.stream);
+    if (hipEventSynchronize(t1) == hipSuccess && ok && hipEventElapsedTime(&ms, t0, t1) == hipSuccess) ms /= 5.f;
+    else ms = -1.f;
+    hipEventDestroy(t0);
+    hipEventDestroy(t1);
+    return ms;
+}
+
+bool make_plan(hipblasLtHandle_t handle, const PlanKey& k, const Operands& op, Plan& p) {
+    const size_t workspace_bytes = op.workspace_bytes;
+    const hipDataType in_t = HIP_R_16BF, out_t = k.out_f32 ? HIP_R_32F : HIP_R_16BF;
+    if (hipblasLtMatmulDescCreate(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F) != HIPBLAS_STATUS_SUCCESS) return false;
+    const hipblasOperation_t tr = HIPBLAS_OP_T, no = HIPBLAS_OP_N;
+    hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &tr, sizeof(tr));
+    hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &no, sizeof(no));
+    if (k.bias_dtype != TM_NONE) {
+        const hipblasLtEpilogue_t epi = HIPBLASLT_EPILOGUE_BIAS;
+        const hipDataType bias_t = k.bias_dtype == TM_F32 ? HIP_R_32F : HIP_R_16BF;
+        hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_EPILOGUE, &epi, sizeof(epi));
+        hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_DATA_TYPE, &bias_t, sizeof(bias_t));
+    }
+    if (hipblasLtMatrixLayoutCreate(&p.w, in_t, k.K, k.N, k.ldw) != HIPBLAS_STATUS_SUCCESS ||
+        hipblasLtMatrixLayoutCreate(&p.a, in_t, k.K, k.M, k.lda) != HIPBLAS_STATUS_SUCCESS ||
+        hipblasLtMatrixLayoutCreate(&p.c, out_t, k.N, k.M, k.ldc) != HIPBLAS_STATUS_SUCCESS)
+        return false;
+    hipblasLtMatmulPreference_t pref = nullptr;
+    if (hipblasLtMatmulPreferenceCreate(&pref) != HIPBLAS_STATUS_SUCCESS) return false;
+    const uint64_t max_ws = workspace_bytes;
+    hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &max_ws, sizeof(max_ws));
+    constexpr int MAX_CANDIDATES = 32;
+    hipblasLtMatmulHeuristicResult_t found[MAX_CANDIDATES];
+    int n_found = 0;
+    // timing needs the stream to run now: never while it is being captured into a graph
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    hipStreamIsCapturing(op.stream, &capturing);
+    int want = g_tune_candidates < 1 || capturing != hipStreamCaptureStatusNone ? 1 : g_tune_candidates;
+    if (want > MAX_CANDIDATES) want = MAX_CANDIDATES;
+    const hipblasStatus_t st =
+        hipblasLtMatmulAlgoGetHeuristic(handle, p.desc, p.w, p.a, p.c, p.c, pref, want, found, &n_found);
+    hipblasLtMatmulPreferenceDestroy(pref);
+    if (st != HIPBLAS_STATUS_SUCCESS || n_found < 1) return false;
+    int best = -1;
+    if (want > 1) {
+        if (k.bias_dtype != TM_NONE)
+            hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &op.bias, sizeof(op.bias));
+        float best_ms = 0.f;
+        for (int i = 0; i < n_found; ++i) {
+            if (found[i].state != HIPBLAS_STATUS_SUCCESS || found[i].workspaceSize > workspace_bytes) continue;
+            const float ms = time_algo(handle, p, found[i].algo, op);
+            if (ms >= 0.f && (best < 0 || ms < best_ms)) {
+                best = i;
+                best_ms = ms;
+            }
+        }
+    }
+    if (best < 0) {                         // untimed, or nothing could be timed: the heuristic's first valid choice
+        for (int i = 0; i < n_found && best < 0; ++i)
+            if (found[i].state == HIPBLAS_STATUS_SUCCESS) best = i;
+        if (best < 0) return false;
+    }
+    p.algo = found[best].algo;
+    p.workspace = found[best].workspaceSize;
+    p.ok = true;
+    return true;
+}
+
+}  // namespace
+
+// The first call of every shape from now on times up to n of the library's candidates on that
+// call's operands and keeps the fastest; 0 keeps the library's first choice (the default).
+extern "C" int tm_gemm_library_tune(int n) {
+    std::lock_guard<std::mutex> guard(lib().lock);
+    g_tune_candidates = n < 0 ? 0 : n;
+    return TM_OK;
+}
+
+// bias_dtype: TM_NONE (no bias), TM_BF16 or TM_F32. out_f32: C is float32 (else bfloat16).
+// workspace: device memory the library may use, the same for every call on a stream.
+// Returns TM_ERR_ARG for arguments it does not take, TM_ERR_UNSUPPORTED when the library has no
+// algorithm for the product (the caller then uses another path), TM_ERR_LAUNCH when the call fails.
+extern "C" int tm_gemm_library(const void* A, int lda, const void* W, int ldw, const void* bias, int bias_dtype,
+                               void* C, int ldc, int out_f32, int M, int N, int K, void* workspace,
+                               size_t workspace_bytes, hipStream_t stream) {
+    if (M <= 0 || N <= 0 || K <= 0 || lda < K || ldw < K || ldc < N || !A || !W || !C ||
+        (bias_dtype != TM_NONE && bias_dtype != TM_BF16 && bias_dtype != TM_F32) || ((bias_dtype != TM_NONE) != (bias != nullptr)))
+        return TM_ERR_ARG;
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess) return TM_ERR_LAUNCH;
+    const PlanKey key{M, N, K, lda, ldw, ldc, bias_dtype, out_f32 ? 1 : 0, device};
+    Library& l = lib();
+    hipblasLtHandle_t handle;
+    Plan plan;
+    {
+        std::lock_guard<std::mutex> guard(l.lock);
+        auto h = l.handles.find(device);
+        if (h == l.handles.end()) {
+            hipblasLtHandle_t made;
+            if (hipblasLtCreate(&made) != HIPBLAS_STATUS_SUCCESS) return TM_ERR_LAUNCH;
+            h = l.handles.emplace(device, made).first;
+        }
+        handle = h->second;
+        auto it = l.plans.find(key);
+        if (it == l.plans.end()) {
+            Plan made;
+            const Operands op{A, W, bias, C, workspace, workspace_bytes, stream};
+            make_plan(handle, key, op, made);                        // a failed plan is kept too: asked once
+            it = l.plans.emplace(key, made).first;
+        }
+        plan = it->second;
+    }
+    if (!plan.ok || plan.workspace > workspace_bytes) return TM_ERR_UNSUPPORTED;
+    if (bias_dtype != TM_NONE)          // the descriptor is shared by every call of this shape: calls on one device are serial
+        hipblasLtMatmulDescSetAttribute(plan.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias, sizeof(bias));
+    const float one = 1.f, zero = 0.f;
+    const hipblasStatus_t st = hipblasLtMatmul(handle, plan.desc, &one, W, plan.w, A, plan.a, &zero, C, plan.c, C, plan.c,
+                                               &plan.algo, workspace, workspace_bytes, stream);
+    return st == HIPBLAS_STATUS_SUCCESS ? TM_OK : TM_ERR_LAUNCH;
+}

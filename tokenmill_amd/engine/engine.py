@@ -49,6 +49,9 @@ def num_cache_pages(cfg: EngineConfig, model, dtype, device, peak_bytes: int) ->
     return int(pages)
 
 
+TUNE_CANDIDATES = 16        # library algorithms timed per shape with tune_gemm
+
+
 class LLMEngine:
     def __init__(self, cfg: EngineConfig, model=None):
         self.cfg = cfg
@@ -59,6 +62,9 @@ class LLMEngine:
         else:
             self.device, self.dtype = model.device, model.dtype
         self.model = model
+        if cfg.tune_gemm:
+            from tokenmill_amd.hip import ops
+            ops.gemm_library_tune(TUNE_CANDIDATES)
         self.eos_ids = set(getattr(model.config, "eos_token_ids", ()) or ())
         peak = self._profile_peak_memory() if (cfg.num_blocks is None and cfg.kv_cache_mb is None) else 0
         pages = num_cache_pages(cfg, model, self.dtype, self.device, peak)

@@ -16,6 +16,7 @@ import numpy as np
 import torch
 
 from tokenmill_amd.cache.manager import RELEASED
+from tokenmill_amd.hip import ops
 from tokenmill_amd.parts.base import GroupStep, StepContext
 
 
@@ -64,6 +65,7 @@ class _Bucket:
 class DecodeGraphs:
     def __init__(self, runner, cfg, max_batch: int = 256):
         self.runner = runner
+        ops.library_workspace(runner.device)      # made now: a capture must not allocate it
         self.page = runner.page_size
         self.max_positions = runner.max_positions
         self.W = -(-runner.max_positions // self.page)

@@ -147,6 +147,11 @@ class ModelRunner:
             q_lens.append(n)
             starts.append(e.start)
             row0 += n
+        if n_tiles > 1:
+            # the tiles that see the most keys first: the long ones start early and the short ones fill
+            # the end of the launch (a tile's result does not depend on where in the table it stands)
+            t = tiles.reshape(n_tiles, 4)
+            t[:] = t[np.argsort(-(t[:, 3] + t[:, 2]), kind="stable")]
         r = 0
         for i, e in enumerate(entries):
             for w in e.want:

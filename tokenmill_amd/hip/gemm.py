@@ -3,7 +3,8 @@
 float32: the LDS-tiled kernel with 32-bit multiply-adds (a true 32-bit product, fixed summation
 order). bfloat16: up to 16 rows (decode steps) the MFMA kernels of this library that stream the
 matrix once and carry the layer's epilogue (bias, rotary + cache write, SiLU·up, residual add) or
-start at the norm; above that the library's matrix product, as the reference's engine uses a library
+start at the norm; above that the library's matrix product (hipBLASLt, called from this package's
+own library with the plan of every shape kept), as the reference's engine uses a library
 for all of its products (reference src/infer/model/layers.py:144,150,163-164, src/infer/model/qwen2.py:51-52);
 measured on an MI355X the library is the faster one from about 32 rows on, and for the wide output
 head at any row count. Shapes neither takes run the tiled kernel.
@@ -16,7 +17,6 @@ from tokenmill_amd.hip import ops
 
 SKINNY_ROWS = 16            # most rows the skinny kernels are preferred for
 SKINNY_MAX_ROWS = 64        # most rows they can take
-_library_f32_out: bool | None = None     # does the library product write float32 from bfloat16 inputs?
 
 
 def _skinny_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
@@ -24,22 +24,6 @@ def _skinny_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
     stride = x.stride(0) if x.shape[0] > 1 else K
     return (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and K % 8 == 0 and stride % 8 == 0
             and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
-
-
-def _library_logits(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> bool:
-    """out (float32) = x @ w^T by the library with 32-bit output, where this torch build has it."""
-    global _library_f32_out
-    if _library_f32_out is False or not out.is_contiguous():
-        return False
-    try:
-        torch.mm(x, w.t(), out_dtype=torch.float32, out=out)
-        _library_f32_out = True
-        return True
-    except (TypeError, RuntimeError):
-        if _library_f32_out:            # it worked before: this is a real error
-            raise
-        _library_f32_out = False
-        return False
 
 
 def linear(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, out: torch.Tensor) -> torch.Tensor:
@@ -50,17 +34,13 @@ def linear(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, out: tor
     if x.dtype != torch.bfloat16:
         return ops.gemm_nt_tiled(x, w, bias, out)
     skinny = _skinny_ok(x, w)
-    if out.dtype == torch.float32 and w.dtype == torch.bfloat16 and bias is None:        # logits
-        if w.shape[0] >= 16384 and _library_logits(x if x.is_contiguous() else x.contiguous(), w, out):
+    library = w.dtype == torch.bfloat16 and x.stride(1) == 1 and out.stride(1) == 1
+    if library and out.dtype == torch.float32 and bias is None and w.shape[0] >= 16384:      # logits
+        if ops.gemm_library(x, w, None, out):
             return out
     if skinny and M <= SKINNY_ROWS:
         return ops.gemm_skinny(x, w, bias, out)
-    if out.dtype == torch.bfloat16 and (bias is None or bias.dtype == torch.bfloat16) and out.is_contiguous() \
-            and w.dtype == torch.bfloat16:
-        if bias is None:
-            torch.mm(x, w.t(), out=out)
-        else:
-            torch.addmm(bias, x, w.t(), out=out)
+    if library and ops.gemm_library(x, w, bias, out):
         return out
     if skinny:                                   # 32-bit results for many rows, 64 rows a call
         for r0 in range(0, M, SKINNY_MAX_ROWS):

@@ -43,7 +43,9 @@ def _p(t: torch.Tensor | None) -> c_void_p:
 
 
 def _stream() -> c_void_p:
-    return c_void_p(torch.cuda.current_stream().cuda_stream)
+    # the current stream of the current device, straight from the C layer: the Python-level
+    # torch.cuda.current_stream() costs more than a launch
+    return c_void_p(torch._C._cuda_getCurrentRawStream(torch._C._cuda_getDevice()))
 
 
 def _check(rc: int, name: str) -> None:
@@ -172,6 +174,54 @@ def gemm_nt_tiled(a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, o
                                       c_int(M), c_int(N), c_int(K), code(a.dtype), code(out.dtype), _stream()),
            "gemm_nt_tiled")
     return out
+
+
+LIBRARY_WORKSPACE_BYTES = 32 << 20
+_library_workspace: dict[int, torch.Tensor] = {}
+
+
+def library_workspace(device: torch.device) -> torch.Tensor:
+    """The device memory the library products may use; made once per device (call it before any
+    graph capture, so that the capture allocates nothing for it)."""
+    ws = _library_workspace.get(device.index)
+    if ws is None:
+        ws = _library_workspace[device.index] = torch.empty(LIBRARY_WORKSPACE_BYTES, dtype=torch.uint8, device=device)
+    return ws
+
+
+def gemm_library_tune(candidates: int) -> None:
+    """From now on the first call of every new shape times up to ``candidates`` of the library's
+    algorithms on its own operands and keeps the fastest (0: the library's first choice, untimed)."""
+    _need(0 <= candidates <= 32, "gemm_library_tune: 0 to 32 candidates")
+    _check(library().tm_gemm_library_tune(c_int(candidates)), "gemm_library_tune")
+
+
+def gemm_library(a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, out: torch.Tensor) -> bool:
+    """out[M, N] = a[M, K] @ w[N, K]^T (+ bias[N]) by hipBLASLt: bfloat16 inputs, 32-bit sums, out
+    bfloat16 or float32. The plan for a shape is made on its first call and kept. Returns False
+    (nothing written) if the library has no algorithm for this product."""
+    _gpu(a, w, bias, out)
+    M, K = a.shape
+    N = w.shape[0]
+    _need(a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out.dtype in (torch.bfloat16, torch.float32),
+          "gemm_library: bfloat16 inputs, bfloat16 or float32 output")
+    _need(w.shape[1] == K and w.is_contiguous(), "gemm_library: w must be contiguous [N, K]")
+    _need(a.stride(1) == 1 and out.stride(1) == 1 and tuple(out.shape) == (M, N),
+          "gemm_library: a [M, K], out [M, N], unit inner stride")
+    if bias is not None:
+        _need(tuple(bias.shape) == (N,) and bias.is_contiguous() and bias.dtype in (torch.bfloat16, torch.float32),
+              "gemm_library: bias must be contiguous [N], bfloat16 or float32")
+    lda = a.stride(0) if M > 1 else max(K, a.stride(0))
+    ldc = out.stride(0) if M > 1 else max(N, out.stride(0))
+    ws = library_workspace(a.device)
+    rc = library().tm_gemm_library(_p(a), c_int(lda), _p(w), c_int(K), _p(bias),
+                                   c_int(code(bias.dtype) if bias is not None else -1), _p(out), c_int(ldc),
+                                   c_int(1 if out.dtype == torch.float32 else 0), c_int(M), c_int(N), c_int(K),
+                                   _p(ws), ctypes.c_size_t(LIBRARY_WORKSPACE_BYTES), _stream())
+    if rc == 3:
+        return False
+    _check(rc, "gemm_library")
+    return True
 
 
 def attn_paged_generic(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
