@@ -350,6 +350,41 @@ def test_gemm_skinny(ops, M, N, K):
     assert torch.equal(out_s, out32)
 
 
+@pytest.mark.parametrize("tune", [0, 6])
+@pytest.mark.parametrize("M,N,K", [(300, 1152, 896), (17, 896, 4864), (2048, 200, 120), (1, 5000, 64), (70, 307, 72)])
+def test_gemm_library(ops, M, N, K, tune):
+    """The library product behind the cached plan: with and without bias, bfloat16 and float32 out,
+    a strided input, the same bits on the second call (the kept plan), with and without timing the
+    candidates first. A shape the library refuses comes back as False and `linear` takes another kernel."""
+    from tokenmill_amd.hip import gemm
+    torch.manual_seed(12)
+    dt = torch.bfloat16
+    a, w, b = q(torch.randn(M, K), dt), q(torch.randn(N, K) * 0.1, dt), q(torch.randn(N), dt)
+    want = a @ w.t()
+    da, dw, db = a.to(dt).to(DEV), w.to(dt).to(DEV), b.to(dt).to(DEV)
+    ops.gemm_library_tune(tune)
+    try:
+        out = torch.full((M, N), 7.0, dtype=dt, device=DEV)
+        if ops.gemm_library(da, dw, db, out):
+            torch.testing.assert_close(out.float().cpu(), q(want + b, dt), **tol(dt))
+            again = torch.empty_like(out)
+            assert ops.gemm_library(da, dw, db, again) and torch.equal(again, out)
+        out32 = torch.full((M, N), 7.0, dtype=torch.float32, device=DEV)
+        if ops.gemm_library(da, dw, None, out32):
+            torch.testing.assert_close(out32.cpu(), want, rtol=1e-4, atol=1e-4 * K ** 0.5)
+        wide = torch.zeros(M, K + 24, dtype=dt, device=DEV)
+        wide[:, :K] = da
+        out_s = torch.full((M, N), 7.0, dtype=dt, device=DEV)
+        if ops.gemm_library(wide[:, :K], dw, None, out_s):
+            torch.testing.assert_close(out_s.float().cpu(), q(want, dt), **tol(dt))
+        # whatever the library takes, the policy above it gives the product
+        out_l = torch.full((M, N), 7.0, dtype=dt, device=DEV)
+        gemm.linear(da, dw, db, out_l)
+        torch.testing.assert_close(out_l.float().cpu(), q(want + b, dt), **tol(dt))
+    finally:
+        ops.gemm_library_tune(0)
+
+
 @pytest.mark.parametrize("M,I,K", [(1, 128, 64), (8, 4864, 896), (40, 200, 120), (64, 320, 192)])
 def test_gemm_skinny_with_silu_epilogue(ops, M, I, K):
     torch.manual_seed(10)

@@ -66,7 +66,10 @@ __device__ __forceinline__ float bias_at(const void* bias, int bias_f32, int n) 
 
 // NT: tiles of 16 tokens. WAVES: wavefronts per block. SPLIT: they share a strip and split K.
 // SILU: W is [2 * N, K] = [gate; up] and the output is silu(gate) * up, N wide.
-template <int NT, int WAVES, bool SPLIT, bool SILU, typename TC>
+// ROWS: rows of W in a strip (16, 8 or 4). A short strip leaves rows of the MFMA tile empty (their
+// lanes load nothing), which costs nothing here, and gives a matrix with few rows enough strips,
+// and so enough blocks, to have loads in flight on every CU of the chip.
+template <int NT, int WAVES, bool SPLIT, bool SILU, typename TC, int ROWS = 16>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ A, int lda,
                                                                  const bf16_t* __restrict__ W,
                                                                  const void* __restrict__ bias, int bias_f32,
@@ -79,7 +82,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
     const int wave = threadIdx.x / TM_WAVE, lane = threadIdx.x % TM_WAVE;
     const int r = lane % 16, g = lane / 16;
     const int strip = SPLIT ? blockIdx.x : blockIdx.x * WAVES + wave;
-    const int n0 = strip * 16;
+    const int n0 = strip * ROWS;
     // K range of this wavefront, in steps of 32
     const int ksteps = (K + 31) / 32;
     int ks0 = 0, ks1 = ksteps;
@@ -88,7 +91,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
         ks0 = wave * per;
         ks1 = ks0 + per < ksteps ? ks0 + per : ksteps;
     }
-    const bool w_ok = n0 + r < N;
+    const bool w_ok = r < ROWS && n0 + r < N;
     const bf16_t* wrow = W + (size_t)(n0 + r) * K + 8 * g;
     const bf16_t* urow = SILU ? W + (size_t)(N + n0 + r) * K + 8 * g : nullptr;
     const bf16_t* arow[NT];
@@ -103,6 +106,15 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
     for (int a = 0; a < NACC; ++a)
 #pragma unroll
         for (int t = 0; t < NT; ++t) acc[a][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    // What the accumulate epilogue will read is asked for now: it arrives while the matrix streams.
+    const int nf = n0 + 4 * g;                  // this lane's output features nf + i (i = 0..3) of token 16t + r
+    const bool acc_fast = accum && nf + 4 <= N && (ldacc % 4) == 0 && ((uintptr_t)accum % 16) == 0;
+    f32x4_t resid_cur[NT];
+    if (acc_fast && (!SPLIT || wave == 0) && 4 * g < ROWS) {
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+            resid_cur[t] = 16 * t + r < M ? *(const f32x4_t*)(accum + (size_t)(16 * t + r) * ldacc + nf) : f32x4_t{0.f, 0.f, 0.f, 0.f};
+    }
 
     if (n0 < N) {
         // KCH k-steps at a time with every load issued before the first product: a wavefront's whole
@@ -148,8 +160,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
         if (wave != 0) return;
     }
     if (n0 >= N) return;
-    // lane: output features n0 + 4g + i (i = 0..3) of token 16t + r
-    const int nf = n0 + 4 * g;
+    if (4 * g >= ROWS) return;
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
         const int tok = 16 * t + r;
@@ -168,8 +179,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
         }
         if (accum) {            // the rounded result goes into the 32-bit residual stream (each element has one owner)
             float* dst = accum + (size_t)tok * ldacc + nf;
-            if (nf + 4 <= N && ((uintptr_t)dst % 16) == 0) {
-                f32x4_t cur = *(f32x4_t*)dst;
+            if (acc_fast) {
+                f32x4_t cur = resid_cur[t];
 #pragma unroll
                 for (int i = 0; i < 4; ++i) cur[i] += bf16_to_f32(f32_to_bf16(v[i]));
                 *(f32x4_t*)dst = cur;
@@ -186,6 +197,21 @@ template <int NT, bool SILU, typename TC>
 static int launch_skinny(const void* A, int lda, const void* W, const void* bias, int bias_f32, void* C, int ldc,
                          int M, int N, int K, float* accum, int ldacc, hipStream_t stream) {
     const int strips = (N + 15) / 16;
+    if (NT == 1 && !SILU && strips < 192) {    // few rows and few tokens: short strips, so that every CU gets a block
+        const bool r8 = (N + 7) / 8 >= 192;
+        const int n_strips = r8 ? (N + 7) / 8 : (N + 3) / 4;
+#define TM_SHORT(WV, RW)                                                                                         \
+    gemm_skinny_kernel<1, WV, true, false, TC, RW><<<n_strips, 64 * WV, 0, stream>>>(                            \
+        (const bf16_t*)A, lda, (const bf16_t*)W, bias, bias_f32, (TC*)C, ldc, M, N, K, accum, ldacc)
+        if (K < 2048) {
+            if (r8) TM_SHORT(4, 8); else TM_SHORT(4, 4);
+        } else {
+            if (r8) TM_SHORT(16, 8); else TM_SHORT(16, 4);
+        }
+#undef TM_SHORT
+        TM_CHECK_LAUNCH();
+        return TM_OK;
+    }
     if (strips >= 2048) {                      // many rows: a strip per wavefront
         gemm_skinny_kernel<NT, 4, false, SILU, TC><<<(strips + 3) / 4, 256, 0, stream>>>(
             (const bf16_t*)A, lda, (const bf16_t*)W, bias, bias_f32, (TC*)C, ldc, M, N, K, accum, ldacc);
