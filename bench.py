@@ -2,6 +2,7 @@
 weights, synthetic token ids, on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype bfloat16|float32] [--layers L]
+                    [--config CONFIG.json]     (another shape of the architecture; the default is the 0.5B shape)
 
 A "step" is one decode step of the engine (scheduling, metadata upload, the forward pass and greedy
 sampling) with a batch of 8 requests, each holding a 2,048-token prompt. One JSON line is printed.
@@ -62,6 +63,7 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (named in config)")
+    ap.add_argument("--config", default=None, help="a config.json: run its shape instead of the 0.5B shape")
     ap.add_argument("--no-graphs", action="store_true", help="launch decode steps kernel by kernel")
     ap.add_argument("--no-tune", action="store_true", help="keep the library's first choice of matrix-product algorithm")
     ap.add_argument("--skip-points", action="store_true", help="only the headline batch and the prefill")
@@ -80,7 +82,9 @@ def main() -> int:
     torch.cuda.set_device(0)
     device = torch.device("cuda:0")
     dtype = {"bfloat16": torch.bfloat16, "float32": torch.float32}[args.dtype]
-    shape = dict(SHAPE)
+    shape, shape_name = dict(SHAPE), "Qwen2.5-0.5B shape"
+    if args.config:
+        shape, shape_name = json.loads(Path(args.config).read_text()), Path(args.config).stem
     layers_full = shape["num_hidden_layers"]
     if args.layers:
         shape["num_hidden_layers"] = args.layers
@@ -154,15 +158,16 @@ def main() -> int:
     achieved = nbytes / step_s / 1e9
     flops = prefill_flops(shape, PROMPT_LEN)
     line = {
-        "metric": "decode tok/s at batch 8, context 2048 (Qwen2.5-0.5B shape); prefill and batch 1/64 alongside",
+        "metric": f"decode tok/s at batch {args.batch}, context 2048 ({shape_name}); prefill and batch 1/64 alongside",
         "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if dtype == torch.bfloat16 else "fp32", "data": "synthetic token ids, random weights",
-        "config": {"model": "Qwen2.5-0.5B shape", "layers": shape["num_hidden_layers"], "layers_full": layers_full,
+        "config": {"model": shape_name, "layers": shape["num_hidden_layers"], "layers_full": layers_full,
                    "hidden": shape["hidden_size"], "q_heads": shape["num_attention_heads"],
                    "kv_heads": shape["num_key_value_heads"],
                    "head_dim": shape["hidden_size"] // shape["num_attention_heads"],
-                   "intermediate": shape["intermediate_size"], "vocab": shape["vocab_size"], "tied": True,
+                   "intermediate": shape["intermediate_size"], "vocab": shape["vocab_size"],
+                   "tied": bool(shape.get("tie_word_embeddings", False)),
                    "global_batch": args.batch, "seq_len": PROMPT_LEN, "context": context,
                    "max_model_len": MAX_MODEL_LEN, "block_size": BLOCK_SIZE, "parallelism": "single GPU",
                    "hip_graphs": not args.no_graphs, "tune_gemm": not args.no_tune},

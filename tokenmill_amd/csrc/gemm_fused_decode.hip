@@ -40,6 +40,9 @@ __device__ __forceinline__ float fd_round(float a) { return bf16_to_f32(f32_to_b
 #define FD_XPAD 8           // padding of an LDS row of x, in elements
 #define FD_RC 8             // 4-element vectors of a residual row a thread keeps in registers
 
+// rows of x a block keeps in LDS for M tokens
+__host__ __device__ __forceinline__ int fused_rows(int M) { return M <= 4 ? 4 : (M <= 8 ? 8 : 16); }
+
 struct FusedArgs {
     // norm + product
     const float* resid;     // [M, K]
@@ -65,83 +68,78 @@ struct FusedArgs {
     int I;
 };
 
-template <int EPI>
-__global__ __launch_bounds__(256) void fused_norm_gemm_kernel(const FusedArgs a) {
+// The two strips of ROWS matrix rows a block multiplies together ("unit" u).
+struct FusedUnit {
+    int nA, nB;             // first rows of the strips
+    int head, jt;           // QKV: the head and which slice of it
+    bool rows_ok;           // this lane's rows exist
+};
+
+// ROWS: rows of a strip (16 or 8). Short strips leave rows of the MFMA tile empty (their lanes load
+// nothing) and double the number of units, for matrices that would otherwise give fewer blocks
+// than the chip has CUs. A block takes the units u = blockIdx.x, + gridDim.x, ...: the norm is
+// computed once and serves all of them.
+// PIPE: a wavefront's K range is longer than one group of FD_KCH steps, and two register groups take
+// turns so that loads are always in flight (more registers; not worth them when one group holds it all).
+template <int EPI, int ROWS, bool PIPE>
+__global__ __launch_bounds__(256, 2) void fused_norm_gemm_kernel(const FusedArgs a, const int n_units) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    bf16_t* xs = (bf16_t*)smem_raw;                                  // [16][K + FD_XPAD]
+    bf16_t* xs = (bf16_t*)smem_raw;                                  // [4, 8 or 16 rows][K + FD_XPAD]
     __shared__ float red[4][2][64][4 + 1];
     const int K = a.K, M = a.M;
     const int xstride = K + FD_XPAD;
     const int wave = threadIdx.x / TM_WAVE, lane = threadIdx.x % TM_WAVE;
     const int r = lane % 16, g = lane / 16;
-    const int u = blockIdx.x;
 
-    // the two strips of this block
-    int nA, nB, head = 0, jt = 0;
-    bool rows_ok = true;
-    if (EPI == FD_EPI_QKV) {
-        const int per_head = a.D / 32;
-        head = u / per_head;
-        jt = u % per_head;
-        if (head < a.H + a.KVH) {
-            nA = head * a.D + 16 * jt;
-            nB = nA + a.D / 2;
-        } else {
-            nA = head * a.D + 32 * jt;
-            nB = nA + 16;
+    auto unit_of = [&](int u) {
+        FusedUnit t;
+        t.head = 0;
+        t.jt = 0;
+        t.rows_ok = r < ROWS;
+        if (EPI == FD_EPI_QKV) {
+            const int per_head = a.D / (2 * ROWS);
+            t.head = u / per_head;
+            t.jt = u % per_head;
+            if (t.head < a.H + a.KVH) {                              // the two halves of ROWS rotary pairs
+                t.nA = t.head * a.D + ROWS * t.jt;
+                t.nB = t.nA + a.D / 2;
+            } else {
+                t.nA = t.head * a.D + 2 * ROWS * t.jt;
+                t.nB = t.nA + ROWS;
+            }
+        } else {                                                     // gate rows and the up rows that meet them
+            t.nA = ROWS * u;
+            t.nB = a.I + ROWS * u;
+            t.rows_ok = r < ROWS && t.nA + r < a.I;
         }
-    } else {
-        nA = 16 * u;
-        nB = a.I + 16 * u;
-        rows_ok = nA + r < a.I;
-    }
+        return t;
+    };
 
-    // matrix loads of the first group go out before the norm is computed
     const int ksteps = (K + 31) / 32;
     const int per = (ksteps + 3) / 4;
     const int ks0 = wave * per;
     const int ks1 = ks0 + per < ksteps ? ks0 + per : ksteps;
-    const bf16_t* wA = a.W + (size_t)(nA + r) * K + 8 * g;
-    const bf16_t* wB = a.W + (size_t)(nB + r) * K + 8 * g;
-    FFrag fa[FD_KCH], fb[FD_KCH];
+    int u = blockIdx.x;
+    FusedUnit cu = unit_of(u);
+    const bf16_t* wA = a.W + (size_t)(cu.nA + r) * K + 8 * g;
+    const bf16_t* wB = a.W + (size_t)(cu.nB + r) * K + 8 * g;
+    auto load_group = [&](auto& ga, auto& gb, int base, bool rows_ok) {
 #pragma unroll
-    for (int j = 0; j < FD_KCH; ++j) {
-        const int k = (ks0 + j) * 32;
-        const bool in = rows_ok && ks0 + j < ks1 && k + 8 * g < K;
-        fa[j].u = in ? *(const u32x4_t*)(wA + k) : u32x4_t{0, 0, 0, 0};
-        fb[j].u = in ? *(const u32x4_t*)(wB + k) : u32x4_t{0, 0, 0, 0};
-    }
-
-    // what the epilogue will need from memory is asked for now, long before it is used
-    const int etok = r;                                              // the epilogue's token of this lane
-    float e_bias[2][4] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
-    float e_cos[4] = {1.f, 1.f, 1.f, 1.f}, e_sin[4] = {0.f, 0.f, 0.f, 0.f};
-    int e_slot = -1;
-    if (EPI == FD_EPI_QKV && wave == 0 && etok < M) {
-        if (a.bias) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int ia = nA + 4 * g + i, ib = nB + 4 * g + i;
-                e_bias[0][i] = a.bias_f32 ? ((const float*)a.bias)[ia] : bf16_to_f32(((const bf16_t*)a.bias)[ia]);
-                e_bias[1][i] = a.bias_f32 ? ((const float*)a.bias)[ib] : bf16_to_f32(((const bf16_t*)a.bias)[ib]);
-            }
+        for (int j = 0; j < FD_KCH; ++j) {
+            const int k = (base + j) * 32;
+            const bool in = rows_ok && base + j < ks1 && k + 8 * g < K;
+            ga[j].u = in ? *(const u32x4_t*)(wA + k) : u32x4_t{0, 0, 0, 0};
+            gb[j].u = in ? *(const u32x4_t*)(wB + k) : u32x4_t{0, 0, 0, 0};
         }
-        e_slot = a.slots ? a.slots[etok] : -1;
-        if (head < a.H + a.KVH) {
-            const size_t at = (size_t)a.positions[etok] * (a.D / 2) + 16 * jt + 4 * g;
-            const f32x4_t cv = *(const f32x4_t*)(a.cos_t + at), sv = *(const f32x4_t*)(a.sin_t + at);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                e_cos[i] = cv[i];
-                e_sin[i] = sv[i];
-            }
-        }
-    }
+    };
+    // matrix loads of the first group go out before the norm is computed
+    FFrag fa[FD_KCH], fb[FD_KCH], fa2[PIPE ? FD_KCH : 1], fb2[PIPE ? FD_KCH : 1];
+    load_group(fa, fb, ks0, cu.rows_ok);
 
     // x = norm(resid) into LDS. A row is shared by TPR threads (all 256 are busy: 16 rows x 16 threads,
     // 8 x 32, or 4 x 64); each keeps its first FD_RC vectors in registers between the two passes.
+    const int mpad = fused_rows(M);
     {
-        const int mpad = M <= 4 ? 4 : (M <= 8 ? 8 : 16);
         const int tpr = 256 / mpad;
         const int row = threadIdx.x / tpr, sub = threadIdx.x % tpr;
         bf16_t* xrow = xs + (size_t)row * xstride;
@@ -188,120 +186,179 @@ __global__ __launch_bounds__(256) void fused_norm_gemm_kernel(const FusedArgs a)
             }
             for (int c = sub * 4 + FD_RC * step; c < K; c += step) emit(c, *(const f32x4_t*)(src + c));
         }
-        // rows M..15 of x stay as they are: they only feed result columns of tokens that do not exist,
-        // which no lane stores
+        // rows M..mpad-1 of x stay as they are, and the lanes of tokens beyond mpad read rows below it
+        // again: they only feed result columns of tokens that do not exist, which no lane stores
     }
     __syncthreads();
 
-    f32x4_t accA = {0.f, 0.f, 0.f, 0.f}, accB = {0.f, 0.f, 0.f, 0.f};
-    const bf16_t* xr = xs + (size_t)r * xstride + 8 * g;
-    for (int base = ks0; base < ks1; base += FD_KCH) {
-        if (base != ks0) {
-#pragma unroll
-            for (int j = 0; j < FD_KCH; ++j) {
-                const int k = (base + j) * 32;
-                const bool in = rows_ok && base + j < ks1 && k + 8 * g < K;
-                fa[j].u = in ? *(const u32x4_t*)(wA + k) : u32x4_t{0, 0, 0, 0};
-                fb[j].u = in ? *(const u32x4_t*)(wB + k) : u32x4_t{0, 0, 0, 0};
-            }
-        }
+    const bf16_t* xr = xs + (size_t)(r & (mpad - 1)) * xstride + 8 * g;
+    f32x4_t accA, accB;
+    auto multiply_group = [&](const auto& ga, const auto& gb, int base) {
 #pragma unroll
         for (int j = 0; j < FD_KCH; ++j) {
             const int k = (base + j) * 32;
             FFrag xf;
             xf.u = (base + j < ks1 && k + 8 * g < K) ? *(const u32x4_t*)(xr + k) : u32x4_t{0, 0, 0, 0};
-            accA = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[j].b, xf.b, accA, 0, 0, 0);
-            accB = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb[j].b, xf.b, accB, 0, 0, 0);
+            accA = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ga[j].b, xf.b, accA, 0, 0, 0);
+            accB = __builtin_amdgcn_mfma_f32_16x16x32_bf16(gb[j].b, xf.b, accB, 0, 0, 0);
         }
-    }
-    // partial sums of the four wavefronts, added in wavefront order
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        red[wave][0][lane][i] = accA[i];
-        red[wave][1][lane][i] = accB[i];
-    }
-    __syncthreads();
-    if (wave != 0) return;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        accA[i] = red[0][0][lane][i] + red[1][0][lane][i] + red[2][0][lane][i] + red[3][0][lane][i];
-        accB[i] = red[0][1][lane][i] + red[1][1][lane][i] + red[2][1][lane][i] + red[3][1][lane][i];
-    }
+    };
+    const int tok = r;                                               // the epilogue's token of this lane
+    const bool epi_lane = wave == 0 && tok < M && 4 * g < ROWS;
 
-    // lane: token r, rows nA + 4g + i and nB + 4g + i
-    const int tok = r;
-    if (tok >= M) return;
-    if (EPI == FD_EPI_SILU) {
-        const int col = 16 * u + 4 * g;
-        if (col >= a.I) return;
-        float v[4];
+    for (;;) {
+        // what the epilogue will need from memory is asked for now, long before it is used
+        float e_bias[2][4] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+        float e_cos[4] = {1.f, 1.f, 1.f, 1.f}, e_sin[4] = {0.f, 0.f, 0.f, 0.f};
+        int e_slot = -1;
+        if (EPI == FD_EPI_QKV && epi_lane) {
+            if (a.bias) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const float gt = fd_round(accA[i]), up = fd_round(accB[i]);
-            v[i] = gt / (1.f + expf(-gt)) * up;
+                for (int i = 0; i < 4; ++i) {
+                    const int ia = cu.nA + 4 * g + i, ib = cu.nB + 4 * g + i;
+                    e_bias[0][i] = a.bias_f32 ? ((const float*)a.bias)[ia] : bf16_to_f32(((const bf16_t*)a.bias)[ia]);
+                    e_bias[1][i] = a.bias_f32 ? ((const float*)a.bias)[ib] : bf16_to_f32(((const bf16_t*)a.bias)[ib]);
+                }
+            }
+            e_slot = a.slots ? a.slots[tok] : -1;
+            if (cu.head < a.H + a.KVH) {
+                const size_t at = (size_t)a.positions[tok] * (a.D / 2) + ROWS * cu.jt + 4 * g;
+                const f32x4_t cv = *(const f32x4_t*)(a.cos_t + at), sv = *(const f32x4_t*)(a.sin_t + at);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    e_cos[i] = cv[i];
+                    e_sin[i] = sv[i];
+                }
+            }
         }
-        bf16_t* dst = a.act_out + (size_t)tok * a.I + col;
-        if (col + 4 <= a.I) {
-            *(uint2*)dst = uint2{fd_pack(v[0], v[1]), fd_pack(v[2], v[3])};
+
+        accA = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        accB = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        if constexpr (PIPE) {
+            // the next group's loads are in flight while this one is multiplied
+            for (int base = ks0; base < ks1; base += 2 * FD_KCH) {
+                if (base + FD_KCH < ks1) load_group(fa2, fb2, base + FD_KCH, cu.rows_ok);
+                multiply_group(fa, fb, base);
+                if (base + FD_KCH >= ks1) break;
+                if (base + 2 * FD_KCH < ks1) load_group(fa, fb, base + 2 * FD_KCH, cu.rows_ok);
+                multiply_group(fa2, fb2, base + FD_KCH);
+            }
         } else {
-            for (int i = 0; i < 4 && col + i < a.I; ++i) dst[i] = f32_to_bf16(v[i]);
+            for (int base = ks0; base < ks1; base += FD_KCH) {
+                if (base != ks0) load_group(fa, fb, base, cu.rows_ok);
+                multiply_group(fa, fb, base);
+            }
         }
-        return;
-    }
-    float xA[4], xB[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        xA[i] = fd_round(accA[i] + e_bias[0][i]);
-        xB[i] = fd_round(accB[i] + e_bias[1][i]);
-    }
-    const int slot = e_slot;
-    if (head < a.H + a.KVH) {
-        const int half = a.D / 2;
-        const int j0 = 16 * jt + 4 * g;                              // pair index of element 0
-        float y1[4], y2[4];
+        // partial sums of the four wavefronts, added in wavefront order
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            y1[i] = xA[i] * e_cos[i] - xB[i] * e_sin[i];
-            y2[i] = xB[i] * e_cos[i] + xA[i] * e_sin[i];
+            red[wave][0][lane][i] = accA[i];
+            red[wave][1][lane][i] = accB[i];
         }
-        bf16_t* dst = nullptr;
-        if (head < a.H)
-            dst = a.q_out + (size_t)tok * a.H * a.D + (size_t)head * a.D + j0;
-        else if (slot >= 0)
-            dst = a.k_pool + ((size_t)slot * a.KVH + (head - a.H)) * a.D + j0;
-        if (dst) {
-            *(uint2*)dst = uint2{fd_pack(y1[0], y1[1]), fd_pack(y1[2], y1[3])};
-            *(uint2*)(dst + half) = uint2{fd_pack(y2[0], y2[1]), fd_pack(y2[2], y2[3])};
+        __syncthreads();
+
+        // the next unit's first loads go out before this unit's epilogue
+        const int un = u + gridDim.x;
+        const bool more = un < n_units;
+        const FusedUnit done = cu;
+        if (more) {
+            cu = unit_of(un);
+            wA = a.W + (size_t)(cu.nA + r) * K + 8 * g;
+            wB = a.W + (size_t)(cu.nB + r) * K + 8 * g;
+            load_group(fa, fb, ks0, cu.rows_ok);
         }
-    } else if (slot >= 0) {
-        const int vh = head - a.H - a.KVH;
-        const int pg = slot >> a.page_shift, in_page = slot & ((1 << a.page_shift) - 1);
-        const int d0 = 32 * jt + 4 * g;
-        bf16_t* dst = a.v_pool + ((((size_t)pg * a.KVH + vh) * a.D + d0) << a.page_shift) + in_page;
+
+        if (epi_lane) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            dst[(size_t)i << a.page_shift] = f32_to_bf16(xA[i]);
-            dst[(size_t)(i + 16) << a.page_shift] = f32_to_bf16(xB[i]);
+            for (int i = 0; i < 4; ++i) {
+                accA[i] = red[0][0][lane][i] + red[1][0][lane][i] + red[2][0][lane][i] + red[3][0][lane][i];
+                accB[i] = red[0][1][lane][i] + red[1][1][lane][i] + red[2][1][lane][i] + red[3][1][lane][i];
+            }
+            // lane: token r, rows nA + 4g + i and nB + 4g + i
+            if (EPI == FD_EPI_SILU) {
+                const int col = done.nA + 4 * g;
+                if (col < a.I) {
+                    float v[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const float gt = fd_round(accA[i]), up = fd_round(accB[i]);
+                        v[i] = gt / (1.f + expf(-gt)) * up;
+                    }
+                    bf16_t* dst = a.act_out + (size_t)tok * a.I + col;
+                    if (col + 4 <= a.I) {
+                        *(uint2*)dst = uint2{fd_pack(v[0], v[1]), fd_pack(v[2], v[3])};
+                    } else {
+                        for (int i = 0; i < 4 && col + i < a.I; ++i) dst[i] = f32_to_bf16(v[i]);
+                    }
+                }
+            } else {
+                float xA[4], xB[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    xA[i] = fd_round(accA[i] + e_bias[0][i]);
+                    xB[i] = fd_round(accB[i] + e_bias[1][i]);
+                }
+                const int slot = e_slot;
+                if (done.head < a.H + a.KVH) {
+                    const int half = a.D / 2;
+                    const int j0 = ROWS * done.jt + 4 * g;                       // pair index of element 0
+                    float y1[4], y2[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        y1[i] = xA[i] * e_cos[i] - xB[i] * e_sin[i];
+                        y2[i] = xB[i] * e_cos[i] + xA[i] * e_sin[i];
+                    }
+                    bf16_t* dst = nullptr;
+                    if (done.head < a.H)
+                        dst = a.q_out + (size_t)tok * a.H * a.D + (size_t)done.head * a.D + j0;
+                    else if (slot >= 0)
+                        dst = a.k_pool + ((size_t)slot * a.KVH + (done.head - a.H)) * a.D + j0;
+                    if (dst) {
+                        *(uint2*)dst = uint2{fd_pack(y1[0], y1[1]), fd_pack(y1[2], y1[3])};
+                        *(uint2*)(dst + half) = uint2{fd_pack(y2[0], y2[1]), fd_pack(y2[2], y2[3])};
+                    }
+                } else if (slot >= 0) {
+                    const int vh = done.head - a.H - a.KVH;
+                    const int pg = slot >> a.page_shift, in_page = slot & ((1 << a.page_shift) - 1);
+                    const int d0 = 2 * ROWS * done.jt + 4 * g;
+                    bf16_t* dst = a.v_pool + ((((size_t)pg * a.KVH + vh) * a.D + d0) << a.page_shift) + in_page;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        dst[(size_t)i << a.page_shift] = f32_to_bf16(xA[i]);
+                        dst[(size_t)(i + ROWS) << a.page_shift] = f32_to_bf16(xB[i]);
+                    }
+                }
+            }
         }
+        if (!more) break;
+        __syncthreads();                                                 // the sums have been read: red is free again
+        u = un;
     }
 }
 
-static int fused_lds_bytes(int K) { return 16 * (K + FD_XPAD) * (int)sizeof(bf16_t); }
+static int fused_lds_bytes(int M, int K) { return fused_rows(M) * (K + FD_XPAD) * (int)sizeof(bf16_t); }
 
-template <int EPI>
-static int launch_fused(const FusedArgs& a, int blocks, hipStream_t stream) {
-    const int lds = fused_lds_bytes(a.K);
+template <int EPI, int ROWS, bool PIPE>
+static int launch_fused_pipe(const FusedArgs& a, int n_units, int blocks, hipStream_t stream) {
+    const int lds = fused_lds_bytes(a.M, a.K);
     if (lds + 6 * 1024 > 160 * 1024) return TM_ERR_ARG;
     static int raised = 0;          // largest dynamic LDS size this kernel has been allowed so far
     if (lds > 48 * 1024 && lds > raised) {
-        if (hipFuncSetAttribute((const void*)fused_norm_gemm_kernel<EPI>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                lds) != hipSuccess)
+        if (hipFuncSetAttribute((const void*)fused_norm_gemm_kernel<EPI, ROWS, PIPE>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
             return TM_ERR_LAUNCH;
         raised = lds;
     }
-    fused_norm_gemm_kernel<EPI><<<blocks, 256, lds, stream>>>(a);
+    fused_norm_gemm_kernel<EPI, ROWS, PIPE><<<blocks, 256, lds, stream>>>(a, n_units);
     TM_CHECK_LAUNCH();
     return TM_OK;
+}
+
+template <int EPI, int ROWS>
+static int launch_fused(const FusedArgs& a, int n_units, int blocks, hipStream_t stream) {
+    const int per = ((a.K + 31) / 32 + 3) / 4;          // k-steps of one wavefront
+    return per > FD_KCH ? launch_fused_pipe<EPI, ROWS, true>(a, n_units, blocks, stream)
+                        : launch_fused_pipe<EPI, ROWS, false>(a, n_units, blocks, stream);
 }
 
 static bool fused_common_ok(int M, int K, const void* resid, const void* W) {
@@ -326,7 +383,10 @@ extern "C" int tm_fused_norm_qkv_rope(const float* resid, const void* norm_w, in
     a.positions = positions; a.slots = slots; a.k_pool = (bf16_t*)k_pool; a.v_pool = (bf16_t*)v_pool;
     a.page_shift = 0;
     while ((1 << a.page_shift) < page) ++a.page_shift;
-    return launch_fused<FD_EPI_QKV>(a, (H + 2 * KVH) * (D / 32), stream);
+    // strips of 16 rows where they give the chip enough blocks, else of 8
+    const int units16 = (H + 2 * KVH) * (D / 32);
+    if (units16 >= 256) return launch_fused<FD_EPI_QKV, 16>(a, units16, units16, stream);
+    return launch_fused<FD_EPI_QKV, 8>(a, 2 * units16, 2 * units16, stream);
 }
 
 // act[M, I] <- silu(norm(resid) Wg^T) * (norm(resid) Wu^T), W = [Wg; Wu] [2I, K].  Needs M <= 16.
@@ -338,5 +398,7 @@ extern "C" int tm_fused_norm_gate_up_silu(const float* resid, const void* norm_w
     FusedArgs a{};
     a.resid = resid; a.norm_w = norm_w; a.norm_w_f32 = norm_w_dtype == TM_F32; a.eps = eps; a.M = M; a.K = K;
     a.W = (const bf16_t*)W; a.act_out = (bf16_t*)act_out; a.I = I;
-    return launch_fused<FD_EPI_SILU>(a, (I + 15) / 16, stream);
+    // at most two blocks a CU: beyond that a block takes several units and the norm is computed once for them
+    const int units = (I + 15) / 16;
+    return launch_fused<FD_EPI_SILU, 16>(a, units, units < 512 ? units : 512, stream);
 }
