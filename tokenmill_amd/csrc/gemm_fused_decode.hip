@@ -36,7 +36,8 @@ __device__ __forceinline__ float fd_round(float a) { return bf16_to_f32(f32_to_b
 
 #define FD_EPI_QKV 0
 #define FD_EPI_SILU 1
-#define FD_KCH 8            // k-steps whose matrix loads are in flight at once, per wavefront
+#define FD_KCH 8            // k-steps of one register group of matrix loads, per wavefront (one group in all)
+#define FD_KCH_PIPE 6       // the same where two groups take turns
 #define FD_XPAD 8           // padding of an LDS row of x, in elements
 #define FD_RC 8             // 4-element vectors of a residual row a thread keeps in registers
 
@@ -81,11 +82,15 @@ struct FusedUnit {
 // computed once and serves all of them.
 // PIPE: a wavefront's K range is longer than one group of FD_KCH steps, and two register groups take
 // turns so that loads are always in flight (more registers; not worth them when one group holds it all).
-template <int EPI, int ROWS, bool PIPE>
-__global__ __launch_bounds__(256, 2) void fused_norm_gemm_kernel(const FusedArgs a, const int n_units) {
+// WAVES: wavefronts of a block (4, or 8 for a long K: they split K, and the norm's rows, between them).
+template <int EPI, int ROWS, bool PIPE, int WAVES>
+__global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void fused_norm_gemm_kernel(const FusedArgs a,
+                                                                                        const int n_units) {
+    constexpr int KCH = PIPE ? FD_KCH_PIPE : FD_KCH;
+    constexpr int THREADS = 64 * WAVES;
     extern __shared__ __align__(16) unsigned char smem_raw[];
     bf16_t* xs = (bf16_t*)smem_raw;                                  // [4, 8 or 16 rows][K + FD_XPAD]
-    __shared__ float red[4][2][64][4 + 1];
+    __shared__ float red[WAVES][2][64][4 + 1];
     const int K = a.K, M = a.M;
     const int xstride = K + FD_XPAD;
     const int wave = threadIdx.x / TM_WAVE, lane = threadIdx.x % TM_WAVE;
@@ -116,7 +121,7 @@ __global__ __launch_bounds__(256, 2) void fused_norm_gemm_kernel(const FusedArgs
     };
 
     const int ksteps = (K + 31) / 32;
-    const int per = (ksteps + 3) / 4;
+    const int per = (ksteps + WAVES - 1) / WAVES;
     const int ks0 = wave * per;
     const int ks1 = ks0 + per < ksteps ? ks0 + per : ksteps;
     int u = blockIdx.x;
@@ -125,7 +130,7 @@ __global__ __launch_bounds__(256, 2) void fused_norm_gemm_kernel(const FusedArgs
     const bf16_t* wB = a.W + (size_t)(cu.nB + r) * K + 8 * g;
     auto load_group = [&](auto& ga, auto& gb, int base, bool rows_ok) {
 #pragma unroll
-        for (int j = 0; j < FD_KCH; ++j) {
+        for (int j = 0; j < KCH; ++j) {
             const int k = (base + j) * 32;
             const bool in = rows_ok && base + j < ks1 && k + 8 * g < K;
             ga[j].u = in ? *(const u32x4_t*)(wA + k) : u32x4_t{0, 0, 0, 0};
@@ -133,14 +138,15 @@ __global__ __launch_bounds__(256, 2) void fused_norm_gemm_kernel(const FusedArgs
         }
     };
     // matrix loads of the first group go out before the norm is computed
-    FFrag fa[FD_KCH], fb[FD_KCH], fa2[PIPE ? FD_KCH : 1], fb2[PIPE ? FD_KCH : 1];
+    FFrag fa[KCH], fb[KCH], fa2[PIPE ? KCH : 1], fb2[PIPE ? KCH : 1];
     load_group(fa, fb, ks0, cu.rows_ok);
+    if constexpr (PIPE) load_group(fa2, fb2, ks0 + KCH, cu.rows_ok);
 
-    // x = norm(resid) into LDS. A row is shared by TPR threads (all 256 are busy: 16 rows x 16 threads,
-    // 8 x 32, or 4 x 64); each keeps its first FD_RC vectors in registers between the two passes.
+    // x = norm(resid) into LDS. A row is shared by TPR threads of one wavefront (256 threads: 16 rows x 16
+    // threads, 8 x 32, or 4 x 64); each keeps its first FD_RC vectors in registers between the two passes.
     const int mpad = fused_rows(M);
     {
-        const int tpr = 256 / mpad;
+        const int tpr = THREADS / mpad < TM_WAVE ? THREADS / mpad : TM_WAVE;
         const int row = threadIdx.x / tpr, sub = threadIdx.x % tpr;
         bf16_t* xrow = xs + (size_t)row * xstride;
         const int step = 4 * tpr;
@@ -155,36 +161,62 @@ __global__ __launch_bounds__(256, 2) void fused_norm_gemm_kernel(const FusedArgs
                 ss += cache[j][0] * cache[j][0] + cache[j][1] * cache[j][1] + cache[j][2] * cache[j][2] +
                       cache[j][3] * cache[j][3];
             }
-            for (int c = sub * 4 + FD_RC * step; c < K; c += step) {
-                const f32x4_t v = *(const f32x4_t*)(src + c);
-                ss += v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
+            // the rest of a long row in groups of FD_RC loads that are in flight together
+            for (int c0 = sub * 4 + FD_RC * step; c0 < K; c0 += FD_RC * step) {
+                f32x4_t v[FD_RC];
+#pragma unroll
+                for (int j = 0; j < FD_RC; ++j)
+                    v[j] = c0 + j * step < K ? *(const f32x4_t*)(src + c0 + j * step) : f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int j = 0; j < FD_RC; ++j)
+                    ss += v[j][0] * v[j][0] + v[j][1] * v[j][1] + v[j][2] * v[j][2] + v[j][3] * v[j][3];
             }
             for (int off = 1; off < tpr; off <<= 1) ss += __shfl_xor(ss, off, TM_WAVE);
             const float rs = rsqrtf(ss / (float)K + a.eps);
-            auto emit = [&](int c, const f32x4_t v) {
-                float w[4];
+            auto weight_at = [&](int c) {
+                f32x4_t w;
                 if (a.norm_w_f32) {
-                    const f32x4_t wv = *(const f32x4_t*)((const float*)a.norm_w + c);
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) w[i] = wv[i];
+                    w = *(const f32x4_t*)((const float*)a.norm_w + c);
                 } else {
                     const uint2 wv = *(const uint2*)((const bf16_t*)a.norm_w + c);
-                    w[0] = __uint_as_float(wv.x << 16);
-                    w[1] = __uint_as_float(wv.x & 0xffff0000u);
-                    w[2] = __uint_as_float(wv.y << 16);
-                    w[3] = __uint_as_float(wv.y & 0xffff0000u);
+                    w = f32x4_t{__uint_as_float(wv.x << 16), __uint_as_float(wv.x & 0xffff0000u),
+                                __uint_as_float(wv.y << 16), __uint_as_float(wv.y & 0xffff0000u)};
                 }
+                return w;
+            };
+            auto emit = [&](int c, const f32x4_t v, const f32x4_t w) {
                 uint2 pk;
                 pk.x = fd_pack(w[0] * fd_round(v[0] * rs), w[1] * fd_round(v[1] * rs));
                 pk.y = fd_pack(w[2] * fd_round(v[2] * rs), w[3] * fd_round(v[3] * rs));
                 *(uint2*)(xrow + c) = pk;
             };
+            // the weights of a group are asked for together (and with the row's values where those
+            // are read again), so that a group costs one trip to memory
+            {
+                f32x4_t w[FD_RC];
 #pragma unroll
-            for (int j = 0; j < FD_RC; ++j) {
-                const int c = sub * 4 + j * step;
-                if (c < K) emit(c, cache[j]);
+                for (int j = 0; j < FD_RC; ++j) {
+                    const int c = sub * 4 + j * step;
+                    w[j] = c < K ? weight_at(c) : f32x4_t{0.f, 0.f, 0.f, 0.f};
+                }
+#pragma unroll
+                for (int j = 0; j < FD_RC; ++j) {
+                    const int c = sub * 4 + j * step;
+                    if (c < K) emit(c, cache[j], w[j]);
+                }
             }
-            for (int c = sub * 4 + FD_RC * step; c < K; c += step) emit(c, *(const f32x4_t*)(src + c));
+            for (int c0 = sub * 4 + FD_RC * step; c0 < K; c0 += FD_RC * step) {
+                f32x4_t v[FD_RC], w[FD_RC];
+#pragma unroll
+                for (int j = 0; j < FD_RC; ++j) {
+                    const bool in = c0 + j * step < K;
+                    v[j] = in ? *(const f32x4_t*)(src + c0 + j * step) : f32x4_t{0.f, 0.f, 0.f, 0.f};
+                    w[j] = in ? weight_at(c0 + j * step) : f32x4_t{0.f, 0.f, 0.f, 0.f};
+                }
+#pragma unroll
+                for (int j = 0; j < FD_RC; ++j)
+                    if (c0 + j * step < K) emit(c0 + j * step, v[j], w[j]);
+            }
         }
         // rows M..mpad-1 of x stay as they are, and the lanes of tokens beyond mpad read rows below it
         // again: they only feed result columns of tokens that do not exist, which no lane stores
@@ -195,7 +227,7 @@ __global__ __launch_bounds__(256, 2) void fused_norm_gemm_kernel(const FusedArgs
     f32x4_t accA, accB;
     auto multiply_group = [&](const auto& ga, const auto& gb, int base) {
 #pragma unroll
-        for (int j = 0; j < FD_KCH; ++j) {
+        for (int j = 0; j < KCH; ++j) {
             const int k = (base + j) * 32;
             FFrag xf;
             xf.u = (base + j < ks1 && k + 8 * g < K) ? *(const u32x4_t*)(xr + k) : u32x4_t{0, 0, 0, 0};
@@ -235,21 +267,22 @@ __global__ __launch_bounds__(256, 2) void fused_norm_gemm_kernel(const FusedArgs
         accA = f32x4_t{0.f, 0.f, 0.f, 0.f};
         accB = f32x4_t{0.f, 0.f, 0.f, 0.f};
         if constexpr (PIPE) {
-            // the next group's loads are in flight while this one is multiplied
-            for (int base = ks0; base < ks1; base += 2 * FD_KCH) {
-                if (base + FD_KCH < ks1) load_group(fa2, fb2, base + FD_KCH, cu.rows_ok);
+            // fa holds group `base` and fa2 the one after it, loaded or on their way: two groups are
+            // always in flight while one is multiplied
+            for (int base = ks0; base < ks1; base += 2 * KCH) {
                 multiply_group(fa, fb, base);
-                if (base + FD_KCH >= ks1) break;
-                if (base + 2 * FD_KCH < ks1) load_group(fa, fb, base + 2 * FD_KCH, cu.rows_ok);
-                multiply_group(fa2, fb2, base + FD_KCH);
+                if (base + 2 * KCH < ks1) load_group(fa, fb, base + 2 * KCH, cu.rows_ok);
+                if (base + KCH >= ks1) break;
+                multiply_group(fa2, fb2, base + KCH);
+                if (base + 3 * KCH < ks1) load_group(fa2, fb2, base + 3 * KCH, cu.rows_ok);
             }
         } else {
-            for (int base = ks0; base < ks1; base += FD_KCH) {
+            for (int base = ks0; base < ks1; base += KCH) {
                 if (base != ks0) load_group(fa, fb, base, cu.rows_ok);
                 multiply_group(fa, fb, base);
             }
         }
-        // partial sums of the four wavefronts, added in wavefront order
+        // partial sums of the wavefronts, added in wavefront order
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             red[wave][0][lane][i] = accA[i];
@@ -266,13 +299,20 @@ __global__ __launch_bounds__(256, 2) void fused_norm_gemm_kernel(const FusedArgs
             wA = a.W + (size_t)(cu.nA + r) * K + 8 * g;
             wB = a.W + (size_t)(cu.nB + r) * K + 8 * g;
             load_group(fa, fb, ks0, cu.rows_ok);
+            if constexpr (PIPE) load_group(fa2, fb2, ks0 + KCH, cu.rows_ok);
         }
 
         if (epi_lane) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                accA[i] = red[0][0][lane][i] + red[1][0][lane][i] + red[2][0][lane][i] + red[3][0][lane][i];
-                accB[i] = red[0][1][lane][i] + red[1][1][lane][i] + red[2][1][lane][i] + red[3][1][lane][i];
+                float sa = red[0][0][lane][i], sb = red[0][1][lane][i];
+#pragma unroll
+                for (int w = 1; w < WAVES; ++w) {
+                    sa += red[w][0][lane][i];
+                    sb += red[w][1][lane][i];
+                }
+                accA[i] = sa;
+                accB[i] = sb;
             }
             // lane: token r, rows nA + 4g + i and nB + 4g + i
             if (EPI == FD_EPI_SILU) {
@@ -338,27 +378,33 @@ __global__ __launch_bounds__(256, 2) void fused_norm_gemm_kernel(const FusedArgs
 
 static int fused_lds_bytes(int M, int K) { return fused_rows(M) * (K + FD_XPAD) * (int)sizeof(bf16_t); }
 
-template <int EPI, int ROWS, bool PIPE>
-static int launch_fused_pipe(const FusedArgs& a, int n_units, int blocks, hipStream_t stream) {
+template <int EPI, int ROWS, bool PIPE, int WAVES>
+static int launch_fused_shape(const FusedArgs& a, int n_units, int blocks, hipStream_t stream) {
     const int lds = fused_lds_bytes(a.M, a.K);
-    if (lds + 6 * 1024 > 160 * 1024) return TM_ERR_ARG;
+    if (lds + (int)sizeof(float) * WAVES * 2 * 64 * 5 + 1024 > 160 * 1024) return TM_ERR_ARG;
     static int raised = 0;          // largest dynamic LDS size this kernel has been allowed so far
     if (lds > 48 * 1024 && lds > raised) {
-        if (hipFuncSetAttribute((const void*)fused_norm_gemm_kernel<EPI, ROWS, PIPE>,
+        if (hipFuncSetAttribute((const void*)fused_norm_gemm_kernel<EPI, ROWS, PIPE, WAVES>,
                                 hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
             return TM_ERR_LAUNCH;
         raised = lds;
     }
-    fused_norm_gemm_kernel<EPI, ROWS, PIPE><<<blocks, 256, lds, stream>>>(a, n_units);
+    fused_norm_gemm_kernel<EPI, ROWS, PIPE, WAVES><<<blocks, 64 * WAVES, lds, stream>>>(a, n_units);
     TM_CHECK_LAUNCH();
     return TM_OK;
 }
 
+// A long K gets 8 wavefronts a block (shorter K ranges, a faster norm); whether a wavefront's range
+// needs more than one register group of loads decides the pipelined variant.
 template <int EPI, int ROWS>
 static int launch_fused(const FusedArgs& a, int n_units, int blocks, hipStream_t stream) {
-    const int per = ((a.K + 31) / 32 + 3) / 4;          // k-steps of one wavefront
-    return per > FD_KCH ? launch_fused_pipe<EPI, ROWS, true>(a, n_units, blocks, stream)
-                        : launch_fused_pipe<EPI, ROWS, false>(a, n_units, blocks, stream);
+    const int ksteps = (a.K + 31) / 32;
+    if (a.K >= 2048) {
+        return (ksteps + 7) / 8 > FD_KCH ? launch_fused_shape<EPI, ROWS, true, 8>(a, n_units, blocks, stream)
+                                         : launch_fused_shape<EPI, ROWS, false, 8>(a, n_units, blocks, stream);
+    }
+    return (ksteps + 3) / 4 > FD_KCH ? launch_fused_shape<EPI, ROWS, true, 4>(a, n_units, blocks, stream)
+                                     : launch_fused_shape<EPI, ROWS, false, 4>(a, n_units, blocks, stream);
 }
 
 static bool fused_common_ok(int M, int K, const void* resid, const void* W) {
@@ -383,9 +429,11 @@ extern "C" int tm_fused_norm_qkv_rope(const float* resid, const void* norm_w, in
     a.positions = positions; a.slots = slots; a.k_pool = (bf16_t*)k_pool; a.v_pool = (bf16_t*)v_pool;
     a.page_shift = 0;
     while ((1 << a.page_shift) < page) ++a.page_shift;
-    // strips of 16 rows where they give the chip enough blocks, else of 8
+    // strips of 16 rows where they give the chip enough blocks, else of 8; a long K runs one block of 8
+    // wavefronts a CU, and more blocks than CUs would mean a second round for a few of them
     const int units16 = (H + 2 * KVH) * (D / 32);
-    if (units16 >= 256) return launch_fused<FD_EPI_QKV, 16>(a, units16, units16, stream);
+    const bool one_block_a_cu = K >= 2048;
+    if (units16 >= 256 || (one_block_a_cu && units16 >= 128)) return launch_fused<FD_EPI_QKV, 16>(a, units16, units16, stream);
     return launch_fused<FD_EPI_QKV, 8>(a, 2 * units16, 2 * units16, stream);
 }
 
@@ -398,7 +446,9 @@ extern "C" int tm_fused_norm_gate_up_silu(const float* resid, const void* norm_w
     FusedArgs a{};
     a.resid = resid; a.norm_w = norm_w; a.norm_w_f32 = norm_w_dtype == TM_F32; a.eps = eps; a.M = M; a.K = K;
     a.W = (const bf16_t*)W; a.act_out = (bf16_t*)act_out; a.I = I;
-    // at most two blocks a CU: beyond that a block takes several units and the norm is computed once for them
+    // no more blocks than the chip holds at once (two a CU, one for a long K): beyond that a block takes
+    // several units and the norm is computed once for all of them
     const int units = (I + 15) / 16;
-    return launch_fused<FD_EPI_SILU, 16>(a, units, units < 512 ? units : 512, stream);
+    const int most = K >= 2048 ? 256 : 512;
+    return launch_fused<FD_EPI_SILU, 16>(a, units, units < most ? units : most, stream);
 }

@@ -69,5 +69,5 @@ def linear_accumulate(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | Non
 def fused_decode_ok(resid: torch.Tensor, w: torch.Tensor) -> bool:
     """Can the norm-fused decode products take this residual and matrix?"""
     M, K = resid.shape
-    return (0 < M <= ops.FUSED_DECODE_ROWS and w.dtype == torch.bfloat16 and K % 8 == 0 and ops.fused_lds_fits(K)
+    return (0 < M <= ops.FUSED_DECODE_ROWS and w.dtype == torch.bfloat16 and K % 8 == 0 and ops.fused_lds_fits(M, K)
             and resid.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)

@@ -469,5 +469,9 @@ def fused_norm_gate_up_silu(resid: torch.Tensor, norm_w: torch.Tensor, eps: floa
     return out
 
 
-def fused_lds_fits(K: int) -> bool:
-    return 16 * (K + 8) * 2 + 6 * 1024 <= 160 * 1024
+def fused_lds_fits(M: int, K: int) -> bool:
+    """Does the normed input of M tokens (4, 8 or 16 rows of K + 8 bfloat16), beside the partial sums of
+    the block's 4 (K < 2048) or 8 wavefronts, fit the 160 KB of LDS a block of the norm-fused products may use?"""
+    rows = 4 if M <= 4 else (8 if M <= 8 else 16)
+    waves = 8 if K >= 2048 else 4
+    return rows * (K + 8) * 2 + 4 * waves * 2 * 64 * 5 + 1024 <= 160 * 1024
