@@ -335,8 +335,9 @@ static int launch_decode(const void* q, int q_stride, void* out, int out_stride,
     while ((1 << page_shift) < page) ++page_shift;
     const float scale_log2 = scale * 1.4426950408889634f;
     constexpr int WAVES = D <= 32 ? 16 : 8;       // 16 wavefronts leave 128 registers each: enough for D = 32 only
-    // few (request, kv head) pairs: more blocks than pairs are needed to pull the cache at speed
-    const bool split = part_o && part_ml && (long long)S * KVH < 64 && max_chunks > 1;
+    // few (request, kv head) pairs: more blocks than pairs are needed to pull the cache at speed; the caller
+    // asks for that by bringing the scratch memory
+    const bool split = part_o && part_ml && max_chunks > 1;
     if (!split) {
         attn_decode_block_kernel<D, WAVES><<<dim3(S, KVH), 64 * WAVES, 0, stream>>>(
             (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool,
@@ -356,8 +357,8 @@ static int launch_decode(const void* q, int q_stride, void* out, int out_stride,
 
 // q: first decode row (one row per request, rows q_stride apart); out likewise; block_tables and
 // context_lens: first decode request. part_o: float [S, H, max_chunks, D] and part_ml: [S, H, max_chunks, 2]
-// are scratch for the split kernels (used when there are fewer than 64 (request, kv head) pairs); without
-// them the block kernel runs.
+// are scratch for the split kernels, which run when both are given (the caller gives them when the
+// (request, kv head) pairs alone are too few blocks for the chip); without them the block kernel runs.
 extern "C" int tm_attn_decode_mfma(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
                                    const void* v_pool, const int* block_tables, int table_width,
                                    const int* context_lens, float* part_o, float* part_ml, int max_chunks, int S,
