@@ -434,3 +434,193 @@ def test_window_groups_a_layer_twice_and_a_shared_cache(tmp_path, dtype_name):
             assert_logits_close(row, want, dt, f"toy window model, {name}, {rid} position {p}")
         session.manager.check_invariants()
         assert not session.manager.live and all(a.num_free == session.num_pages for a in session.manager.allocators)
+
+
+# ----------------------------------------------------------------------------------------------- routed experts, another position encoding
+
+@dataclass(frozen=True)
+class ToyRoutedConfig:
+    vocab_size: int
+    hidden_size: int
+    num_hidden_layers: int
+    num_experts: int
+    max_positions: int
+    eos_token_ids: tuple = ()
+
+    @classmethod
+    def from_dict(cls, raw, generation=None):
+        return cls(raw["vocab_size"], raw["hidden_size"], raw["num_hidden_layers"], raw["num_experts"],
+                   raw["max_positions"])
+
+
+ROUTED_HEADS, ROUTED_KV_HEADS, ROUTED_D, ROUTED_I = 3, 1, 32, 96
+
+
+def plant_routing_signal(model_dir, num_experts, amplitude=1.5, gain=2.0):
+    """Random router weights decide hundreds of tokens by margins that a rounding difference can flip,
+    and a flipped token gets another expert's output: no tolerance would be the right one. So the
+    decision is planted: channels 0 and 1 of every token's embedding hold one of `num_experts`
+    directions (by token id), and the routers read those two channels. The attention in between
+    moves them by far less than the angle between two directions, so engine and plain implementation
+    route alike, while every expert is used and the other 78 channels carry the random signal."""
+    import math
+
+    from safetensors.torch import load_file, save_file
+    path = str(model_dir / "model.safetensors")
+    tensors = load_file(path)
+    angle = [2 * math.pi * e / num_experts for e in range(num_experts)]
+    emb = tensors["model.embed_tokens.weight"]
+    ids = torch.arange(emb.shape[0])
+    emb[:, 0] = (amplitude * torch.tensor([math.cos(a) for a in angle]))[ids % num_experts].to(emb.dtype)
+    emb[:, 1] = (amplitude * torch.tensor([math.sin(a) for a in angle]))[ids % num_experts].to(emb.dtype)
+    for name, t in tensors.items():
+        if name.endswith("mlp.router.weight"):
+            t.zero_()
+            t[:, 0] = gain * torch.tensor([math.cos(a) for a in angle]).to(t.dtype)
+            t[:, 1] = gain * torch.tensor([math.sin(a) for a in angle]).to(t.dtype)
+    save_file(tensors, path)
+
+
+def build_toy_routed_model(cfg: ToyRoutedConfig, max_positions=None):
+    """Attention whose position encoding is a learned table added to q and k, and a feed-forward that
+    sends every token to one of several experts: both defined here, outside the framework."""
+    from tokenmill_amd.hip import ops
+    from tokenmill_amd.models.decoder import DecoderModel
+    from tokenmill_amd.parts import (FeedForward, GQAttention, Linear, OutputHead, PositionEncoding, PreNormBlock,
+                                     RMSNorm, SwiGLU, TokenEmbedding, as_tensor)
+    from tokenmill_amd.weights.loader import TensorSpec
+
+    class AddedPositions(PositionEncoding):
+        """q and k of every head get the row of their position from a learned [positions, D] table."""
+
+        def __init__(self, head_dim, positions):
+            self.head_dim, self.positions = head_dim, positions
+            self.table = None
+
+        def tensor_specs(self, prefix):
+            return {prefix + "pos_table.weight": TensorSpec((self.positions, self.head_dim))}
+
+        def load(self, tensors, prefix):
+            self.table = tensors[prefix + "pos_table.weight"]
+
+        def encode_and_store(self, qkv, num_heads, num_kv_heads, head_dim, step, cache):
+            rows = self.table[step.positions.long()].float()                       # [T, D]
+            n = (num_heads + num_kv_heads) * head_dim
+            qk = qkv[:, :n].view(-1, num_heads + num_kv_heads, head_dim)
+            qk.copy_((qk.float() + rows[:, None, :]).to(qkv.dtype))
+            if cache is not None and cache.write:                                  # store k and v as they now are
+                ops.rope_kv_write(qkv, num_heads, num_kv_heads, head_dim, None, None, None,
+                                  step.groups[cache.group].slot_mapping, cache.k, cache.v)
+
+    class TopOneExperts(FeedForward):
+        """Router logits in 32-bit; a token goes to the expert with the largest logit and its output is
+        weighted by that expert's softmax probability."""
+
+        def __init__(self, hidden, intermediate, num_experts):
+            self.router = Linear(hidden, num_experts, "router")
+            self.experts = [SwiGLU(hidden, intermediate) for _ in range(num_experts)]
+
+        def _parts(self, prefix):
+            return [(self.router, prefix)] + [(e, prefix + f"experts.{i}.") for i, e in enumerate(self.experts)]
+
+        def tensor_specs(self, prefix):
+            specs = {}
+            for part, p in self._parts(prefix):
+                specs.update(part.tensor_specs(p))
+            return specs
+
+        def load(self, tensors, prefix):
+            for part, p in self._parts(prefix):
+                part.load(tensors, p)
+
+        def forward(self, x, step, residual=None):
+            x = as_tensor(x)
+            probs = torch.softmax(self.router.forward(x, out_dtype=torch.float32), dim=-1)
+            weight, choice = probs.max(dim=-1)
+            out = torch.zeros_like(x)
+            for e, expert in enumerate(self.experts):
+                rows = (choice == e).nonzero().flatten()
+                if rows.numel():
+                    y = expert.forward(x[rows].contiguous(), step)
+                    out[rows] = (weight[rows, None] * y.float()).to(x.dtype)
+            return out
+
+    hidden = cfg.hidden_size
+    emb = TokenEmbedding(cfg.vocab_size, hidden)
+    layers = []
+    for i in range(cfg.num_hidden_layers):
+        attention = GQAttention(hidden, ROUTED_HEADS, ROUTED_KV_HEADS, ROUTED_D, ROUTED_D ** -0.5,
+                                AddedPositions(ROUTED_D, cfg.max_positions), qkv_bias=False)
+        ffn = TopOneExperts(hidden, ROUTED_I, cfg.num_experts) if i % 2 == 0 else SwiGLU(hidden, ROUTED_I)
+        layers.append(PreNormBlock(RMSNorm(hidden, 1e-6), attention, RMSNorm(hidden, 1e-6), ffn))
+    return DecoderModel(cfg, emb, layers, RMSNorm(hidden, 1e-6), OutputHead(hidden, cfg.vocab_size, tied_to=None))
+
+
+def plain_toy_routed_logits(w, cfg, ids, dt):
+    """The same model with plain functions, whole sequence. Also returns the smallest gap between the
+    two largest router probabilities of any token (the test wants it wide: see plant_routing_signal)
+    and which experts were used."""
+    T, hidden = len(ids), cfg["hidden_size"]
+    H, KVH, D = ROUTED_HEADS, ROUTED_KV_HEADS, ROUTED_D
+    x = P.rnd(w["model.embed_tokens.weight"], dt)[torch.tensor(ids)]
+    margin = 1.0
+    for i in range(cfg["num_hidden_layers"]):
+        p = f"model.layers.{i}."
+        a = p + "self_attn."
+        h = P.rms_norm(x, w[p + "input_layernorm.weight"], 1e-6, dt)
+        rows = P.rnd(w[a + "pos_table.weight"], dt)[:T]
+        qq = P.rnd(P.linear(h, w[a + "q_proj.weight"], None, dt).view(T, H, D) + rows[:, None, :], dt)
+        kk = P.rnd(P.linear(h, w[a + "k_proj.weight"], None, dt).view(T, KVH, D) + rows[:, None, :], dt)
+        vv = P.linear(h, w[a + "v_proj.weight"], None, dt).view(T, KVH, D)
+        att = P.causal_attention(qq, kk, vv, D ** -0.5, dt)
+        x = x + P.linear(att.reshape(T, H * D), w[a + "o_proj.weight"], None, dt)
+        h = P.rms_norm(x, w[p + "post_attention_layernorm.weight"], 1e-6, dt)
+        m = p + "mlp."
+        if i % 2 == 0:
+            probs = torch.softmax(P.linear(h, w[m + "router.weight"], None, dt, out_dt=torch.float32), dim=-1)
+            top2 = probs.topk(2, dim=-1).values
+            margin = min(margin, float((top2[:, 0] - top2[:, 1]).min()))
+            weight, choice = probs.max(dim=-1)
+            delta = torch.zeros(T, hidden)
+            for t in range(T):
+                y = P.mlp_block(h[t:t + 1], w, m + f"experts.{int(choice[t])}.", dt)
+                delta[t] = P.rnd(weight[t] * y[0], dt)
+            x = x + delta
+        else:
+            x = x + P.mlp_block(h, w, m, dt)
+    h = P.rms_norm(x, w["model.norm.weight"], 1e-6, dt)
+    return P.linear(h, w["lm_head.weight"], None, dt, out_dt=torch.float32), margin
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_routed_experts_and_added_positions_are_registered_built_and_stepped(tmp_path, dtype_name):
+    """A feed-forward with routing and another position encoding, both defined in this file, go through
+    registry, random weights, loader, cache manager, step function and replay unchanged; the positions
+    enter only through the table, so cutting a request anywhere must give the same logits."""
+    from tokenmill_amd.config import register_architecture
+    from tokenmill_amd.replay import ReplaySession
+    from tokenmill_amd.weights import write_random_model
+    from test_gpu_replay import mixed, portions, prefill_then_decode, run_trace
+
+    register_architecture("ToyRoutedLM", ToyRoutedConfig.from_dict, build_toy_routed_model, replace=True)
+    cfg = {"architectures": ["ToyRoutedLM"], "vocab_size": 180, "hidden_size": 80, "num_hidden_layers": 3,
+           "num_experts": 3, "max_positions": 128}
+    d = write_random_model(cfg, tmp_path / "toyr", seed=5, std=0.05, norm_std=0.1)
+    plant_routing_signal(d, 3)
+    dt = {"float32": torch.float32, "bfloat16": torch.bfloat16}[dtype_name]
+    w = P.read_weights(d)
+    assert sum("experts." in k for k in w) == 2 * 3 * 3 and "model.layers.0.self_attn.pos_table.weight" in w
+    session = ReplaySession(d, dtype_name, 4 * 128)
+    reqs = {f"r{i}": random_ids(n, 180, 500 + i) for i, n in enumerate([60, 35, 47, 90, 21])}
+    want = {}
+    for rid, ids in reqs.items():
+        want[rid], margin = plain_toy_routed_logits(w, cfg, ids, dt)
+        assert margin > 0.5, f"{rid}: a router decision is too close to call ({margin})"
+    for name, steps in (("prefill+decode", prefill_then_decode(reqs)), ("portions", portions(reqs)),
+                        ("mixed", mixed(reqs, seed=10))):
+        got = run_trace(session, steps)
+        assert len(got) == sum(len(v) for v in reqs.values()) or name == "prefill+decode"
+        for (rid, p), row in got.items():
+            assert_logits_close(row, want[rid][p], dt, f"toy routed model, {name}, {rid} position {p}")
+        session.manager.check_invariants()
+        assert not session.manager.live
