@@ -63,6 +63,8 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (named in config)")
+    ap.add_argument("--prompt-len", type=int, default=PROMPT_LEN,
+                    help="tokens of every prompt: the prefill's length and the context the decode steps start from")
     ap.add_argument("--config", default=None, help="a config.json: run its shape instead of the 0.5B shape")
     ap.add_argument("--no-graphs", action="store_true", help="launch decode steps kernel by kernel")
     ap.add_argument("--no-tune", action="store_true", help="keep the library's first choice of matrix-product algorithm")
@@ -70,6 +72,8 @@ def main() -> int:
     ap.add_argument("--part", default="all", choices=["all", "decode", "prefill"],
                     help="run only the decode steps or only the prefill (for profiling one of them)")
     args = ap.parse_args()
+    prompt_len = args.prompt_len
+    max_model_len = max(MAX_MODEL_LEN, prompt_len + args.steps + args.warmup + 128)
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
@@ -88,17 +92,17 @@ def main() -> int:
     layers_full = shape["num_hidden_layers"]
     if args.layers:
         shape["num_hidden_layers"] = args.layers
-    model = load_random_model(shape, seed=0, dtype=dtype, device=device, max_positions=MAX_MODEL_LEN)
+    model = load_random_model(shape, seed=0, dtype=dtype, device=device, max_positions=max_model_len)
     elem = 2 if dtype == torch.bfloat16 else 4
     gen = torch.Generator().manual_seed(0)
 
     def prompts(n):
-        return [torch.randint(0, shape["vocab_size"], (PROMPT_LEN,), generator=gen).tolist() for _ in range(n)]
+        return [torch.randint(0, shape["vocab_size"], (prompt_len,), generator=gen).tolist() for _ in range(n)]
 
     def engine_for(batch):
-        pages = batch * (-(-(PROMPT_LEN + args.steps + args.warmup + 64) // BLOCK_SIZE)) + 8
-        cfg = EngineConfig(dtype=args.dtype, block_size=BLOCK_SIZE, num_blocks=pages, max_model_len=MAX_MODEL_LEN,
-                           max_num_seqs=max(batch, 1), max_num_batched_tokens=max(PROMPT_LEN, batch),
+        pages = batch * (-(-(prompt_len + args.steps + args.warmup + 64) // BLOCK_SIZE)) + 8
+        cfg = EngineConfig(dtype=args.dtype, block_size=BLOCK_SIZE, num_blocks=pages, max_model_len=max_model_len,
+                           max_num_seqs=max(batch, 1), max_num_batched_tokens=max(prompt_len, batch),
                            watermark=0.0, hip_graphs=not args.no_graphs, tune_gemm=not args.no_tune)
         return LLMEngine(cfg, model=model)
 
@@ -118,7 +122,7 @@ def main() -> int:
             assert len(outs) == batch
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
-        context = PROMPT_LEN + warmup + steps // 2
+        context = prompt_len + warmup + steps // 2
         for s in list(eng.seqs):
             eng.abort_request(s)
         del eng
@@ -140,7 +144,7 @@ def main() -> int:
 
     if args.part == "prefill":
         prefill_s = time_prefill()
-        print(json.dumps({"prefill": {"value": round(PROMPT_LEN / prefill_s, 1), "tokens": PROMPT_LEN,
+        print(json.dumps({"prefill": {"value": round(prompt_len / prefill_s, 1), "tokens": prompt_len,
                                       "ms": round(prefill_s * 1e3, 3)}}))
         return 0
     step_s, context = time_decode(args.batch, args.steps, args.warmup)
@@ -156,9 +160,9 @@ def main() -> int:
             points[f"decode_b{b}"] = round(b / s, 1)
     nbytes = decode_bytes(shape, args.batch, context, elem)
     achieved = nbytes / step_s / 1e9
-    flops = prefill_flops(shape, PROMPT_LEN)
+    flops = prefill_flops(shape, prompt_len)
     line = {
-        "metric": f"decode tok/s at batch {args.batch}, context 2048 ({shape_name}); prefill and batch 1/64 alongside",
+        "metric": f"decode tok/s at batch {args.batch}, context {prompt_len} ({shape_name}); prefill and batch 1/64 alongside",
         "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if dtype == torch.bfloat16 else "fp32", "data": "synthetic token ids, random weights",
@@ -168,10 +172,10 @@ def main() -> int:
                    "head_dim": shape["hidden_size"] // shape["num_attention_heads"],
                    "intermediate": shape["intermediate_size"], "vocab": shape["vocab_size"],
                    "tied": bool(shape.get("tie_word_embeddings", False)),
-                   "global_batch": args.batch, "seq_len": PROMPT_LEN, "context": context,
-                   "max_model_len": MAX_MODEL_LEN, "block_size": BLOCK_SIZE, "parallelism": "single GPU",
+                   "global_batch": args.batch, "seq_len": prompt_len, "context": context,
+                   "max_model_len": max_model_len, "block_size": BLOCK_SIZE, "parallelism": "single GPU",
                    "hip_graphs": not args.no_graphs, "tune_gemm": not args.no_tune},
-        "prefill": {"value": round(PROMPT_LEN / prefill_s, 1), "tokens": PROMPT_LEN, "ms": round(prefill_s * 1e3, 3),
+        "prefill": {"value": round(prompt_len / prefill_s, 1), "tokens": prompt_len, "ms": round(prefill_s * 1e3, 3),
                     "frac": round(flops / prefill_s / PEAK_FLOPS[args.dtype], 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / PEAK_HBM_GBS, 4)},

@@ -302,28 +302,60 @@ __global__ __launch_bounds__(256) void attn_decode_split_kernel(
     }
 }
 
-// out[s, h, :] = sum over the visible chunks (ascending) of partial values, normalised.
-__global__ void attn_decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                         const int* __restrict__ context_lens, bf16_t* __restrict__ out,
-                                         int out_stride, int max_chunks, int H, int D, int window) {
+// out[s, h, :] = the partial values of the visible chunks, weighted and normalised. Four wavefronts
+// share a (request, head): wavefront w adds the chunks c0 + w, c0 + w + 4, ... in ascending order and
+// the four sums are added in wavefront order, so the order of additions depends on the context
+// length and the window only. A lane holds elements d = lane and lane + 64 of the head.
+#define AD_MERGE_WAVES 4
+__global__ __launch_bounds__(64 * AD_MERGE_WAVES) void attn_decode_merge_kernel(
+    const float* __restrict__ part_o, const float* __restrict__ part_ml, const int* __restrict__ context_lens,
+    bf16_t* __restrict__ out, int out_stride, int max_chunks, int H, int D, int window) {
+    __shared__ float s_m[AD_MERGE_WAVES], s_l[AD_MERGE_WAVES], s_o[AD_MERGE_WAVES][128];
     const int s = blockIdx.x, h = blockIdx.y;
+    const int wave = threadIdx.x / TM_WAVE, lane = threadIdx.x % TM_WAVE;
     const int ctx = context_lens[s];
     const int p = ctx - 1;
     const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
     const int c0 = lo / AD_CHUNK, c1 = (ctx - 1) / AD_CHUNK;
     const size_t base = ((size_t)s * H + h) * max_chunks;
     float mm = -INFINITY;
-    for (int c = c0; c <= c1; ++c) mm = fmaxf(mm, part_ml[(base + c) * 2]);
-    for (int d = threadIdx.x; d < D; d += blockDim.x) {
-        float ll = 0.f, oo = 0.f;
-        for (int c = c0; c <= c1; ++c) {
-            const float mc = part_ml[(base + c) * 2];
-            const float f = (mc == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mc - mm);
-            ll += part_ml[(base + c) * 2 + 1] * f;
-            oo += part_o[(base + c) * D + d] * f;
-        }
-        out[(size_t)s * out_stride + (size_t)h * D + d] = f32_to_bf16(oo / ll);
+    for (int c = c0 + (int)threadIdx.x; c <= c1; c += 64 * AD_MERGE_WAVES) mm = fmaxf(mm, part_ml[(base + c) * 2]);
+    mm = wave_max(mm);
+    if (lane == 0) s_m[wave] = mm;
+    __syncthreads();
+    mm = s_m[0];
+#pragma unroll
+    for (int w = 1; w < AD_MERGE_WAVES; ++w) mm = fmaxf(mm, s_m[w]);
+    const bool two = lane + 64 < D;
+    float ll = 0.f, o0 = 0.f, o1 = 0.f;
+#pragma unroll 4
+    for (int c = c0 + wave; c <= c1; c += AD_MERGE_WAVES) {
+        const float mc = part_ml[(base + c) * 2];
+        const float lc = part_ml[(base + c) * 2 + 1];
+        const float a0 = lane < D ? part_o[(base + c) * D + lane] : 0.f;
+        const float a1 = two ? part_o[(base + c) * D + lane + 64] : 0.f;
+        const float f = (mc == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mc - mm);
+        ll = fmaf(lc, f, ll);
+        o0 = fmaf(a0, f, o0);
+        o1 = fmaf(a1, f, o1);
     }
+    if (lane == 0) s_l[wave] = ll;
+    s_o[wave][lane] = o0;
+    s_o[wave][lane + 64] = o1;
+    __syncthreads();
+    if (wave != 0) return;
+    ll = s_l[0];
+    o0 = s_o[0][lane];
+    o1 = s_o[0][lane + 64];
+#pragma unroll
+    for (int w = 1; w < AD_MERGE_WAVES; ++w) {
+        ll += s_l[w];
+        o0 += s_o[w][lane];
+        o1 += s_o[w][lane + 64];
+    }
+    bf16_t* orow = out + (size_t)s * out_stride + (size_t)h * D;
+    if (lane < D) orow[lane] = f32_to_bf16(o0 / ll);
+    if (two) orow[lane + 64] = f32_to_bf16(o1 / ll);
 }
 
 template <int D>
@@ -349,8 +381,8 @@ static int launch_decode(const void* q, int q_stride, void* out, int out_stride,
         (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, block_tables, table_width,
         context_lens, part_o, part_ml, max_chunks, H, KVH, page_shift, scale_log2, window);
     TM_CHECK_LAUNCH();
-    attn_decode_merge_kernel<<<dim3(S, H), 64, 0, stream>>>(part_o, part_ml, context_lens, (bf16_t*)out, out_stride,
-                                                            max_chunks, H, D, window);
+    attn_decode_merge_kernel<<<dim3(S, H), 64 * AD_MERGE_WAVES, 0, stream>>>(
+        part_o, part_ml, context_lens, (bf16_t*)out, out_stride, max_chunks, H, D, window);
     TM_CHECK_LAUNCH();
     return TM_OK;
 }
