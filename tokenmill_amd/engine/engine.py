@@ -117,7 +117,7 @@ class LLMEngine:
         if request_id in self.seqs:
             raise RequestRejected(f"duplicate request id {request_id}")
         vocab = self.runner.vocab
-        if any((not 0 <= t < vocab) for t in prompt_ids):
+        if min(prompt_ids) < 0 or max(prompt_ids) >= vocab:
             raise RequestRejected(f"a prompt token is outside the vocabulary of {vocab}")
         seq = Sequence(request_id, list(prompt_ids), params,
                        arrival_time=time.monotonic() if arrival_time is None else arrival_time)

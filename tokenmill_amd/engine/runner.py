@@ -140,9 +140,13 @@ class ModelRunner:
                 tab[:widths[i]] = np.where(table == RELEASED, 0, table)   # never read: below the window
                 tab[widths[i]:] = 0                                       # padding: never read either
             if n > 1:
-                for j in range(0, n, 16):
-                    tiles[4 * tile_i:4 * tile_i + 4] = (s, row0 + j, min(16, n - j), e.start + j)
-                    tile_i += 1
+                first = np.arange(0, n, 16, dtype=np.int64)                      # first token of each tile
+                t = tiles[4 * tile_i:4 * (tile_i + len(first))].reshape(len(first), 4)
+                t[:, 0] = s
+                t[:, 1] = row0 + first
+                t[:, 2] = np.minimum(16, n - first)
+                t[:, 3] = e.start + first
+                tile_i += len(first)
             first_row[i] = row0
             q_lens.append(n)
             starts.append(e.start)
