@@ -193,6 +193,30 @@ def paged_truth(case, lens, q_lens, scale, dt, window=None):
     return torch.cat(outs)
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 307, 120), (8, 896, 4864), (16, 1153, 896), (5, 6, 4), (3, 9728, 896)])
+def test_gemv_f32(ops, M, N, K):
+    """The 32-bit matrix-vector kernel of decode steps: against a 64-bit product, with and without
+    bias, a strided input, and a row alone giving the same bits as among others."""
+    torch.manual_seed(13)
+    a, w, b = torch.randn(M, K), torch.randn(N, K) * 0.1, torch.randn(N)
+    want = (a.double() @ w.double().t()).float()
+    da, dw, db = a.to(DEV), w.to(DEV), b.to(DEV)
+    out = torch.full((M, N), 7.0, device=DEV)
+    ops.gemv_f32(da, dw, db, out)
+    torch.testing.assert_close(out.cpu(), want + b, rtol=1e-5, atol=1e-5 * K ** 0.5)
+    ops.gemv_f32(da, dw, None, out)
+    torch.testing.assert_close(out.cpu(), want, rtol=1e-5, atol=1e-5 * K ** 0.5)
+    one = torch.empty(1, N, device=DEV)
+    ops.gemv_f32(da[M - 1:], dw, None, one)
+    assert torch.equal(one[0], out[M - 1])
+    wide = torch.zeros(M, K + 12, device=DEV)
+    wide[:, :K] = da
+    out_s = torch.empty(M, N, device=DEV)
+    ops.gemv_f32(wide[:, :K], dw, None, out_s)
+    assert torch.equal(out_s, out)
+    assert not ops.gemv_f32_ok(torch.zeros(17, K, device=DEV), dw, None, torch.zeros(17, N, device=DEV))
+
+
 @pytest.mark.parametrize("dt", DTS)
 @pytest.mark.parametrize("H,KVH,D,page", [(4, 2, 16, 16), (6, 1, 32, 8), (14, 2, 64, 16), (5, 5, 48, 4), (3, 1, 128, 16),
                                            (8, 2, 80, 16)])
@@ -215,6 +239,32 @@ def test_paged_attention_generic(ops, dt, H, KVH, D, page):
     got_last = out.float().cpu()[-1].view(H, D)
     for h in range(H):
         torch.testing.assert_close(got_last[h], v_far[h // (H // KVH)], rtol=0, atol=5e-2)
+
+
+@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("window", [0, 40])
+def test_paged_attention_generic_many_tokens(ops, dt, window):
+    """A step with many (token, head) pairs runs one wavefront a pair, a small one lets the
+    wavefronts of a block share a pair's keys: both against the plain attention, and against each
+    other (the same rows computed in a large and in a small call differ by rounding only)."""
+    H, KVH, D, page = 4, 2, 32, 16
+    lens, q_lens = [300, 210], [300, 210]
+    case = paged_case(dt, lens, q_lens, H, KVH, D, page, seed=14)
+    scale = D ** -0.5
+    T = case["q"].shape[0]
+    assert T * H >= 1024
+    dev = {k: (v_layout(case[k]) if k == "vp" else case[k]).to(DEV) for k in ("kp", "vp", "tables", "seq_of", "pos")}
+    q = case["q"].reshape(T, H * D).to(DEV)
+    out = torch.empty(T, H * D, dtype=dt, device=DEV)
+    ops.attn_paged_generic(q, out, dev["kp"], dev["vp"], dev["tables"], dev["seq_of"], dev["pos"], H, KVH, D, scale, window)
+    want = paged_truth(case, lens, q_lens, scale, dt, window or None).reshape(T, H * D)
+    torch.testing.assert_close(out.float().cpu(), want, **tol(dt))
+    few = slice(280, 300)                        # the last rows of the first request, alone
+    out_few = torch.empty(20, H * D, dtype=dt, device=DEV)
+    ops.attn_paged_generic(q[few], out_few, dev["kp"], dev["vp"], dev["tables"], dev["seq_of"][few], dev["pos"][few],
+                           H, KVH, D, scale, window)
+    torch.testing.assert_close(out_few.float().cpu(), want[few], **tol(dt))
+    torch.testing.assert_close(out_few.float(), out[few].float(), **tol(dt))
 
 
 @pytest.mark.parametrize("dt", DTS)

@@ -13,23 +13,46 @@
 // It takes every head size that is a multiple of 4 up to 256 and any q length and start position,
 // in 32-bit and in bfloat16; it is the attention of the true 32-bit path, and the bfloat16 path
 // uses it for shapes its MFMA kernels refuse. Keys are visited in ascending position in groups of
-// 64 starting at lo, whatever else the batch holds, so a token's result depends on nothing but its
-// own request.
+// 64 starting at lo, so a token's result depends on its own request only (and, in the last bits, on
+// whether the step was small enough for the wavefronts of a block to share a token's keys).
 #include "common.h"
 #include "api.h"
 
 #define AG_WAVES 4
+#define AG_SPLIT_WAVES 8
 #define AG_MAXD 256
 
-template <typename T>
-__global__ __launch_bounds__(AG_WAVES * TM_WAVE) void attn_paged_generic_kernel(
+// four consecutive elements as 32-bit floats
+__device__ __forceinline__ void ag_load4(const float* p, float (&v)[4]) {
+    const float4 t = *(const float4*)p;
+    v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+}
+__device__ __forceinline__ void ag_load4(const bf16_t* p, float (&v)[4]) {
+    const uint2 t = *(const uint2*)p;
+    v[0] = __uint_as_float(t.x << 16);
+    v[1] = __uint_as_float(t.x & 0xffff0000u);
+    v[2] = __uint_as_float(t.y << 16);
+    v[3] = __uint_as_float(t.y & 0xffff0000u);
+}
+
+// SPLIT = false: a block is AG_WAVES (token, head) pairs, one per wavefront (steps with many tokens).
+// SPLIT = true : a block is one (token, head) pair; its AG_SPLIT_WAVES wavefronts take the groups of 64
+//                keys in turn (group i goes to wavefront i % AG_SPLIT_WAVES) and their partial results
+//                are merged through LDS in wavefront order (steps with few tokens, where the pairs
+//                alone would leave most of the chip idle). Which keys a wavefront takes depends on
+//                the token's own position and window only.
+template <typename T, bool SPLIT>
+__global__ __launch_bounds__((SPLIT ? AG_SPLIT_WAVES : AG_WAVES) * TM_WAVE) void attn_paged_generic_kernel(
     const T* __restrict__ q, int q_stride, T* __restrict__ out, int out_stride,
     const T* __restrict__ k_pool, const T* __restrict__ v_pool, const int* __restrict__ block_tables,
     int table_width, const int* __restrict__ seq_of_token, const int* __restrict__ positions, int T_tokens,
     int H, int KVH, int D, int page, float scale, int window) {
-    __shared__ float q_s[AG_WAVES][AG_MAXD];
+    constexpr int WAVES = SPLIT ? AG_SPLIT_WAVES : AG_WAVES;
+    __shared__ float q_s[SPLIT ? 1 : AG_WAVES][AG_MAXD];
+    __shared__ float s_m[SPLIT ? AG_SPLIT_WAVES : 1], s_l[SPLIT ? AG_SPLIT_WAVES : 1];
+    __shared__ float s_acc[SPLIT ? AG_SPLIT_WAVES : 1][SPLIT ? AG_MAXD : 1];
     const int wave = threadIdx.x / TM_WAVE, lane = threadIdx.x % TM_WAVE;
-    const long long w = (long long)blockIdx.x * AG_WAVES + wave;
+    const long long w = SPLIT ? (long long)blockIdx.x : (long long)blockIdx.x * AG_WAVES + wave;
     const bool active = w < (long long)T_tokens * H;
     const int t = active ? (int)(w / H) : 0, h = active ? (int)(w % H) : 0;
     const int kvh = h / (H / KVH);
@@ -37,9 +60,14 @@ __global__ __launch_bounds__(AG_WAVES * TM_WAVE) void attn_paged_generic_kernel(
     const int p = positions[t];
     const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
     const int* table = block_tables + (size_t)s * table_width;
+    float* qs = q_s[SPLIT ? 0 : wave];
 
     const T* qrow = q + (size_t)t * q_stride + (size_t)h * D;
-    for (int d = lane; d < D; d += TM_WAVE) q_s[wave][d] = Elem<T>::load(qrow + d);
+    if (SPLIT) {
+        for (int d = threadIdx.x; d < D; d += WAVES * TM_WAVE) qs[d] = Elem<T>::load(qrow + d);
+    } else {
+        for (int d = lane; d < D; d += TM_WAVE) qs[d] = Elem<T>::load(qrow + d);
+    }
     __syncthreads();
     if (!active) return;
 
@@ -48,7 +76,9 @@ __global__ __launch_bounds__(AG_WAVES * TM_WAVE) void attn_paged_generic_kernel(
 #pragma unroll
     for (int i = 0; i < AG_MAXD / TM_WAVE; ++i) acc[i] = 0.f;
 
-    for (int j0 = lo; j0 <= p; j0 += TM_WAVE) {
+    const int first = SPLIT ? lo + wave * TM_WAVE : lo;
+    const int stride = SPLIT ? WAVES * TM_WAVE : TM_WAVE;
+    for (int j0 = first; j0 <= p; j0 += stride) {
         const int j = j0 + lane;
         const bool valid = j <= p;
         long long row = 0;
@@ -58,10 +88,12 @@ __global__ __launch_bounds__(AG_WAVES * TM_WAVE) void attn_paged_generic_kernel(
             const T* kr = k_pool + ((size_t)row * KVH + kvh) * D;
             float dot = 0.f;
             for (int d = 0; d < D; d += 4) {
-                dot = fmaf(q_s[wave][d + 0], Elem<T>::load(kr + d + 0), dot);
-                dot = fmaf(q_s[wave][d + 1], Elem<T>::load(kr + d + 1), dot);
-                dot = fmaf(q_s[wave][d + 2], Elem<T>::load(kr + d + 2), dot);
-                dot = fmaf(q_s[wave][d + 3], Elem<T>::load(kr + d + 3), dot);
+                float kv[4];
+                ag_load4(kr + d, kv);
+                dot = fmaf(qs[d + 0], kv[0], dot);
+                dot = fmaf(qs[d + 1], kv[1], dot);
+                dot = fmaf(qs[d + 2], kv[2], dot);
+                dot = fmaf(qs[d + 3], kv[3], dot);
             }
             sc = dot * scale;
         }
@@ -86,12 +118,55 @@ __global__ __launch_bounds__(AG_WAVES * TM_WAVE) void attn_paged_generic_kernel(
         }
     }
     T* orow = out + (size_t)t * out_stride + (size_t)h * D;
-    const float inv = 1.f / l;
+    if (!SPLIT) {
+        const float inv = 1.f / l;
+#pragma unroll
+        for (int i = 0; i < AG_MAXD / TM_WAVE; ++i) {
+            const int d = lane + i * TM_WAVE;
+            if (d < D) Elem<T>::store(orow + d, acc[i] * inv);
+        }
+        return;
+    }
+    // the wavefronts' partial results, merged in wavefront order (one that saw no key has m = -inf, l = 0)
+    if (lane == 0) {
+        s_m[wave] = m;
+        s_l[wave] = l;
+    }
 #pragma unroll
     for (int i = 0; i < AG_MAXD / TM_WAVE; ++i) {
         const int d = lane + i * TM_WAVE;
-        if (d < D) Elem<T>::store(orow + d, acc[i] * inv);
+        if (d < D) s_acc[wave][d] = acc[i];
     }
+    __syncthreads();
+    float mm = s_m[0];
+#pragma unroll
+    for (int ww = 1; ww < WAVES; ++ww) mm = fmaxf(mm, s_m[ww]);
+    float ll = 0.f;
+#pragma unroll
+    for (int ww = 0; ww < WAVES; ++ww) ll += (s_m[ww] == -INFINITY) ? 0.f : s_l[ww] * expf(s_m[ww] - mm);
+    for (int d = threadIdx.x; d < D; d += WAVES * TM_WAVE) {
+        float oo = 0.f;
+#pragma unroll
+        for (int ww = 0; ww < WAVES; ++ww) oo += (s_m[ww] == -INFINITY) ? 0.f : s_acc[ww][d] * expf(s_m[ww] - mm);
+        Elem<T>::store(orow + d, oo / ll);
+    }
+}
+
+template <typename T>
+static void launch_generic(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
+                           const void* v_pool, const int* block_tables, int table_width, const int* seq_of_token,
+                           const int* positions, int T_tokens, int H, int KVH, int D, int page, float scale,
+                           int window, hipStream_t stream) {
+    const long long pairs = (long long)T_tokens * H;
+    if (pairs < 1024)           // too few (token, head) pairs to fill the chip: the wavefronts of a block split the keys
+        attn_paged_generic_kernel<T, true><<<(unsigned)pairs, AG_SPLIT_WAVES * TM_WAVE, 0, stream>>>(
+            (const T*)q, q_stride, (T*)out, out_stride, (const T*)k_pool, (const T*)v_pool, block_tables,
+            table_width, seq_of_token, positions, T_tokens, H, KVH, D, page, scale, window);
+    else
+        attn_paged_generic_kernel<T, false><<<(unsigned)((pairs + AG_WAVES - 1) / AG_WAVES), AG_WAVES * TM_WAVE, 0,
+                                              stream>>>(
+            (const T*)q, q_stride, (T*)out, out_stride, (const T*)k_pool, (const T*)v_pool, block_tables,
+            table_width, seq_of_token, positions, T_tokens, H, KVH, D, page, scale, window);
 }
 
 extern "C" int tm_attn_paged_generic(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
@@ -102,19 +177,18 @@ extern "C" int tm_attn_paged_generic(const void* q, int q_stride, void* out, int
     if (H <= 0 || KVH <= 0 || H % KVH || D <= 0 || D > AG_MAXD || D % 4 || page <= 0 || table_width <= 0 ||
         window < 0 || q_stride < H * D || out_stride < H * D)
         return TM_ERR_ARG;
-    const long long waves = (long long)T * H;
-    const long long blocks = (waves + AG_WAVES - 1) / AG_WAVES;
-    if (blocks > 0x7fffffffLL) return TM_ERR_ARG;
-    if (dtype == TM_F32)
-        attn_paged_generic_kernel<float><<<(unsigned)blocks, AG_WAVES * TM_WAVE, 0, stream>>>(
-            (const float*)q, q_stride, (float*)out, out_stride, (const float*)k_pool, (const float*)v_pool,
-            block_tables, table_width, seq_of_token, positions, T, H, KVH, D, page, scale, window);
-    else if (dtype == TM_BF16)
-        attn_paged_generic_kernel<bf16_t><<<(unsigned)blocks, AG_WAVES * TM_WAVE, 0, stream>>>(
-            (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool,
-            block_tables, table_width, seq_of_token, positions, T, H, KVH, D, page, scale, window);
-    else
+    if (((long long)T * H + AG_WAVES - 1) / AG_WAVES > 0x7fffffffLL) return TM_ERR_ARG;
+    if (dtype == TM_F32) {
+        if (((uintptr_t)k_pool % 16)) return TM_ERR_ARG;
+        launch_generic<float>(q, q_stride, out, out_stride, k_pool, v_pool, block_tables, table_width, seq_of_token,
+                              positions, T, H, KVH, D, page, scale, window, stream);
+    } else if (dtype == TM_BF16) {
+        if (((uintptr_t)k_pool % 8)) return TM_ERR_ARG;
+        launch_generic<bf16_t>(q, q_stride, out, out_stride, k_pool, v_pool, block_tables, table_width, seq_of_token,
+                               positions, T, H, KVH, D, page, scale, window, stream);
+    } else {
         return TM_ERR_ARG;
+    }
     TM_CHECK_LAUNCH();
     return TM_OK;
 }

@@ -83,6 +83,88 @@ static int launch_tiled(const void* A, int lda, const void* W, const void* bias,
     return TM_OK;
 }
 
+// gemv_f32: the same product for at most 16 rows of A in 32-bit (a decode step of the true 32-bit
+// path), bound by reading W once. A block of four wavefronts takes GV_ROWS rows of W; the
+// wavefronts split K into four contiguous ranges, a lane takes the slices k = 256 i + 4 lane .. + 3
+// of its wavefront's range in ascending i, the lanes' sums are added by a fixed tree and the
+// wavefronts' in wavefront order: the order of additions depends on K only, so a row's result
+// does not depend on the other rows of the call. 32-bit multiply-adds only.
+#define GV_ROWS 4
+
+typedef float gv_f32x4 __attribute__((ext_vector_type(4)));
+
+template <int MT>
+__global__ __launch_bounds__(256) void gemv_f32_kernel(const float* __restrict__ A, int lda,
+                                                       const float* __restrict__ W,
+                                                       const float* __restrict__ bias, float* __restrict__ C,
+                                                       int ldc, int M, int N, int K) {
+    __shared__ float red[4][GV_ROWS][MT];
+    const int wave = threadIdx.x / TM_WAVE, lane = threadIdx.x % TM_WAVE;
+    const int n0 = blockIdx.x * GV_ROWS;
+    const int slices = (K + 255) / 256;                     // 256 = 64 lanes x 4 elements
+    const int per = (slices + 3) / 4;
+    const int s0 = wave * per, s1 = s0 + per < slices ? s0 + per : slices;
+    float acc[GV_ROWS][MT];
+#pragma unroll
+    for (int r = 0; r < GV_ROWS; ++r)
+#pragma unroll
+        for (int m = 0; m < MT; ++m) acc[r][m] = 0.f;
+    for (int sl = s0; sl < s1; ++sl) {
+        const int k = sl * 256 + 4 * lane;
+        if (k >= K) continue;                               // K is a multiple of 4: a slice is whole or absent
+        gv_f32x4 w[GV_ROWS];
+#pragma unroll
+        for (int r = 0; r < GV_ROWS; ++r)
+            w[r] = n0 + r < N ? *(const gv_f32x4*)(W + (size_t)(n0 + r) * K + k) : gv_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            const gv_f32x4 a = m < M ? *(const gv_f32x4*)(A + (size_t)m * lda + k) : gv_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int r = 0; r < GV_ROWS; ++r) {
+                float v = acc[r][m];
+                v = fmaf(a[0], w[r][0], v);
+                v = fmaf(a[1], w[r][1], v);
+                v = fmaf(a[2], w[r][2], v);
+                v = fmaf(a[3], w[r][3], v);
+                acc[r][m] = v;
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < GV_ROWS; ++r)
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            const float v = wave_sum(acc[r][m]);
+            if (lane == 0) red[wave][r][m] = v;
+        }
+    __syncthreads();
+    const int r = threadIdx.x / MT, m = threadIdx.x % MT;
+    if (r < GV_ROWS && m < M && n0 + r < N) {
+        float v = red[0][r][m] + red[1][r][m];
+        v += red[2][r][m];
+        v += red[3][r][m];
+        if (bias) v += bias[n0 + r];
+        C[(size_t)m * ldc + n0 + r] = v;
+    }
+}
+
+// C[M, N] (float32) = A[M, K] W[N, K]^T + bias, all float32, M <= 16, K % 4 == 0, 16-byte aligned rows.
+extern "C" int tm_gemv_f32(const float* A, int lda, const float* W, const float* bias, float* C, int ldc, int M,
+                           int N, int K, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return TM_OK;
+    if (M > 16 || K <= 0 || (K % 4) || (lda % 4) || lda < K || ldc < N || ((uintptr_t)A % 16) || ((uintptr_t)W % 16))
+        return TM_ERR_ARG;
+    const unsigned blocks = (unsigned)((N + GV_ROWS - 1) / GV_ROWS);
+    if (M <= 4)
+        gemv_f32_kernel<4><<<blocks, 256, 0, stream>>>(A, lda, W, bias, C, ldc, M, N, K);
+    else if (M <= 8)
+        gemv_f32_kernel<8><<<blocks, 256, 0, stream>>>(A, lda, W, bias, C, ldc, M, N, K);
+    else
+        gemv_f32_kernel<16><<<blocks, 256, 0, stream>>>(A, lda, W, bias, C, ldc, M, N, K);
+    TM_CHECK_LAUNCH();
+    return TM_OK;
+}
+
 extern "C" int tm_gemm_nt_tiled(const void* A, int lda, const void* W, const void* bias, int bias_dtype,
                                 void* C, int ldc, int M, int N, int K, int in_dtype, int out_dtype,
                                 hipStream_t stream) {

@@ -1,7 +1,7 @@
 """Which matrix-product kernel a Linear runs.
 
 float32: the LDS-tiled kernel with 32-bit multiply-adds (a true 32-bit product, fixed summation
-order). bfloat16: up to 16 rows (decode steps) the MFMA kernels of this library that stream the
+order), or up to 16 rows a matrix-vector kernel of the same kind that streams the matrix once. bfloat16: up to 16 rows (decode steps) the MFMA kernels of this library that stream the
 matrix once and carry the layer's epilogue (bias, rotary + cache write, SiLU·up, residual add) or
 start at the norm; above that the library's matrix product (hipBLASLt, called from this package's
 own library with the plan of every shape kept), as the reference's engine uses a library
@@ -32,6 +32,8 @@ def linear(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, out: tor
     if M == 0:
         return out
     if x.dtype != torch.bfloat16:
+        if ops.gemv_f32_ok(x, w, bias, out):                    # a decode step of the 32-bit path
+            return ops.gemv_f32(x, w, bias, out)
         return ops.gemm_nt_tiled(x, w, bias, out)
     skinny = _skinny_ok(x, w)
     library = w.dtype == torch.bfloat16 and x.stride(1) == 1 and out.stride(1) == 1

@@ -224,6 +224,35 @@ def gemm_library(a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, ou
     return True
 
 
+GEMV_F32_ROWS = 16          # most rows the 32-bit matrix-vector kernel takes
+
+
+def gemv_f32_ok(a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, out: torch.Tensor) -> bool:
+    M, K = a.shape
+    lda = a.stride(0) if M > 1 else max(K, a.stride(0))
+    return (a.dtype == torch.float32 and w.dtype == torch.float32 and out.dtype == torch.float32
+            and (bias is None or bias.dtype == torch.float32) and 0 < M <= GEMV_F32_ROWS and K % 4 == 0
+            and lda % 4 == 0 and a.stride(1) == 1 and out.stride(1) == 1 and a.data_ptr() % 16 == 0
+            and w.data_ptr() % 16 == 0)
+
+
+def gemv_f32(a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, out: torch.Tensor) -> torch.Tensor:
+    """out[M, N] = a[M, K] @ w[N, K]^T (+ bias[N]), everything float32, M <= 16: 32-bit multiply-adds
+    in an order that depends on K only."""
+    _gpu(a, w, bias, out)
+    M, K = a.shape
+    N = w.shape[0]
+    _need(gemv_f32_ok(a, w, bias, out), "gemv_f32: float32 operands, at most 16 rows, K a multiple of 4, 16-byte aligned")
+    _need(w.shape[1] == K and w.is_contiguous() and tuple(out.shape) == (M, N), "gemv_f32: w [N, K] contiguous, out [M, N]")
+    if bias is not None:
+        _need(tuple(bias.shape) == (N,) and bias.is_contiguous(), "gemv_f32: bias must be [N]")
+    lda = a.stride(0) if M > 1 else max(K, a.stride(0))
+    ldc = out.stride(0) if M > 1 else max(N, out.stride(0))
+    _check(library().tm_gemv_f32(_p(a), c_int(lda), _p(w), _p(bias), _p(out), c_int(ldc), c_int(M), c_int(N),
+                                 c_int(K), _stream()), "gemv_f32")
+    return out
+
+
 def attn_paged_generic(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                        block_tables: torch.Tensor, seq_of_token: torch.Tensor, positions: torch.Tensor,
                        H: int, KVH: int, D: int, scale: float, window: int = 0) -> torch.Tensor:
