@@ -18,7 +18,7 @@ from pathlib import Path
 
 sys.path.insert(0, str(Path(__file__).resolve().parent))
 
-# BASELINE configuration 3: the Qwen2.5-0.5B shape
+# the headline configuration: the Qwen2.5-0.5B shape
 SHAPE = {"architectures": ["Qwen2ForCausalLM"], "num_hidden_layers": 24, "hidden_size": 896,
          "num_attention_heads": 14, "num_key_value_heads": 2, "intermediate_size": 4864, "vocab_size": 151936,
          "rope_theta": 1e6, "rms_norm_eps": 1e-6, "tie_word_embeddings": True, "max_position_embeddings": 32768,

@@ -46,7 +46,7 @@ def verify(plain, prompt, out, dt, params=None, seed=0):
 
 @pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
 def test_greedy_generation_whole_prompts(model_dirs, plains, dtype_name):
-    """BASELINE configuration A: prompts of 5 / 17 / 33 ids, whole-prompt prefill, 16 greedy tokens."""
+    """The first tiny configuration: prompts of 5 / 17 / 33 ids, whole-prompt prefill, 16 greedy tokens."""
     from tokenmill_amd import SamplingParams
     eng = make_engine(model_dirs["A"], dtype_name)
     prompts = [random_ids(n, 256, 20 + i) for i, n in enumerate((5, 17, 33))]
@@ -60,7 +60,7 @@ def test_greedy_generation_whole_prompts(model_dirs, plains, dtype_name):
 
 @pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
 def test_sampled_generation_chunked_and_mixed(model_dirs, plains, dtype_name):
-    """BASELINE configuration B: page size 8, prefill in portions of 12 mixed with decodes,
+    """The second tiny configuration: page size 8, prefill in portions of 12 mixed with decodes,
     temperature 0.8 with a fixed seed, prompts of 1 / 9 / 24 / 40 ids, 20 tokens."""
     from tokenmill_amd import SamplingParams
     eng = make_engine(model_dirs["B"], dtype_name, block_size=8, enable_chunked_prefill=True,
