@@ -533,6 +533,47 @@ def test_paged_attention_prefill_mfma(ops, H, KVH, D, page, window):
     assert torch.equal(out2[first:first + 200], out[first:first + 200])
 
 
+@pytest.mark.parametrize("H,KVH,D,page", [(14, 2, 64, 16), (6, 1, 32, 16), (5, 5, 128, 32), (3, 1, 48, 16), (8, 2, 80, 64),
+                                           (4, 2, 16, 16)])
+@pytest.mark.parametrize("window", [0, 40])
+def test_paged_attention_prefill_f32(ops, H, KVH, D, page, window):
+    """The 32-bit MFMA attention of prompt portions, at 32-bit tolerance: whole prompts, portions that
+    start and end mid-page, a far key that carries a query, pages behind the window never read, and
+    the same bits when a request is cut into other portions."""
+    dt = torch.float32
+    lens = [2, 37, 130, 64, 5, 300, 33, 200]
+    q_lens = [2, 37, 2, 64, 3, 45, 17, 200]
+    case = paged_case(dt, lens, q_lens, H, KVH, D, page, seed=15, spike=(5, 3) if not window else None)
+    if window:
+        for s, (n, ql) in enumerate(zip(lens, q_lens)):
+            for i in range(max(0, n - ql - window + 1) // page):
+                case["kp"][case["tables"][s, i]] = float("nan")
+                case["vp"][case["tables"][s, i]] = float("nan")
+    T = case["q"].shape[0]
+    scale = D ** -0.5
+    wide = torch.zeros(T, (H + 2 * KVH) * D, dtype=dt, device=DEV)
+    wide[:, :H * D] = case["q"].reshape(T, H * D).to(DEV)
+    out = torch.full((T, H * D), 3.0, dtype=dt, device=DEV)
+    k_dev, v_dev = case["kp"].to(DEV), v_layout(case["vp"]).to(DEV)
+    ops.attn_prefill_f32(wide, out, k_dev, v_dev, case["tables"].to(DEV), tiles_for(lens, q_lens).to(DEV), H, KVH, D,
+                         scale, window)
+    want = paged_truth(case, lens, q_lens, scale, dt, window or None).reshape(T, H * D)
+    torch.testing.assert_close(out.cpu(), want, rtol=2e-5, atol=2e-5)
+    if not window:
+        row = sum(q_lens[:6]) - 1
+        v_far = case["v"][5][3].float()
+        got = out.cpu()[row].view(H, D)
+        for h in range(H):
+            torch.testing.assert_close(got[h], v_far[h // (H // KVH)], rtol=0, atol=2e-2)
+    s = 7
+    first = sum(q_lens[:s])
+    out2 = torch.empty(T, H * D, dtype=dt, device=DEV)
+    t2 = torch.tensor([(s, first + j, min(16, 77 - j), j) for j in range(0, 77, 16)] +
+                      [(s, first + 77 + j, min(16, 123 - j), 77 + j) for j in range(0, 123, 16)], dtype=torch.int32)
+    ops.attn_prefill_f32(wide, out2, k_dev, v_dev, case["tables"].to(DEV), t2.to(DEV), H, KVH, D, scale, window)
+    assert torch.equal(out2[first:first + 200], out[first:first + 200])
+
+
 # ----------------------------------------------------------------------------------------------- fused decode kernels
 
 @pytest.mark.parametrize("M,K,H,KVH,D,page", [(8, 896, 14, 2, 64, 16), (1, 192, 6, 1, 32, 16), (16, 3584, 4, 4, 128, 32),

@@ -55,6 +55,10 @@ int tm_gemm_library_tune(int n);
 int tm_gemm_library(const void* A, int lda, const void* W, int ldw, const void* bias, int bias_dtype, void* C, int ldc,
                     int out_f32, int M, int N, int K, void* workspace, size_t workspace_bytes, hipStream_t stream);
 
+int tm_attn_prefill_f32(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
+                        const void* v_pool, const int* block_tables, int table_width, const int* tiles, int n_tiles,
+                        int H, int KVH, int D, int page, float scale, int window, hipStream_t stream);
+
 int tm_argmax_work_chunks(int V);
 int tm_argmax_rows(const float* logits, int R, int V, int* out, float* work_v, int* work_i, hipStream_t stream);
 

@@ -2,8 +2,8 @@
 
 The step's entries are ordered with the single-token entries last. In bfloat16, when the head
 size and page size allow, prompt portions go to the flash-style MFMA kernel and single tokens to
-the split-context MFMA decode kernel; everything else (the true 32-bit path, unusual shapes) goes
-to the generic kernel.
+the split-context MFMA decode kernel. In float32 prompt portions go to the flash-style kernel on
+the 32-bit MFMA. Everything else (single tokens in float32, unusual shapes) goes to the generic kernel.
 """
 from __future__ import annotations
 
@@ -23,6 +23,10 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, cache: KVCacheView, st
     done_prefill = done_decode = False
     if tp and step.prefill_tiles is not None and ops.attn_prefill_mfma_supported(qkv.dtype, H, KVH, D, page):
         ops.attn_prefill_mfma(qkv, out, cache.k, cache.v, g.block_tables, step.prefill_tiles, H, KVH, D, scale, window)
+        done_prefill = True
+    elif tp and step.prefill_tiles is not None and ops.attn_prefill_f32_supported(qkv.dtype, H, KVH, D, page) \
+            and qkv.stride(0) % 4 == 0 and qkv.data_ptr() % 16 == 0:
+        ops.attn_prefill_f32(qkv, out, cache.k, cache.v, g.block_tables, step.prefill_tiles, H, KVH, D, scale, window)
         done_prefill = True
     if nd and ops.attn_decode_mfma_supported(qkv.dtype, H, KVH, D, page):
         ops.attn_decode_mfma(qkv[tp:], out[tp:], cache.k, cache.v, g.block_tables[S - nd:], step.context_lens[S - nd:],

@@ -439,6 +439,37 @@ def attn_prefill_mfma(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, 
     return out
 
 
+def attn_prefill_f32_supported(dtype, H: int, KVH: int, D: int, page: int) -> bool:
+    return (dtype == torch.float32 and D % 16 == 0 and 16 <= D <= 128 and page >= 16 and page & (page - 1) == 0
+            and H % KVH == 0)
+
+
+def attn_prefill_f32(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
+                     block_tables: torch.Tensor, tiles: torch.Tensor, H: int, KVH: int, D: int, scale: float,
+                     window: int) -> torch.Tensor:
+    """Attention of prompt portions over the cache in true 32-bit (32-bit MFMA). Operands as for
+    ``attn_prefill_mfma``, all float32."""
+    _gpu(q, out, k_pool, v_pool, block_tables, tiles)
+    T = q.shape[0]
+    page = _check_pools(k_pool, v_pool, KVH, D, torch.float32, "attn_prefill_f32")
+    _need(attn_prefill_f32_supported(q.dtype, H, KVH, D, page), "attn_prefill_f32: unsupported head size or page size")
+    _need(q.stride(1) == 1 and out.stride(1) == 1 and out.dtype == torch.float32 and out.shape[0] == T
+          and q.shape[1] >= H * D and out.shape[1] >= H * D, "attn_prefill_f32: q, out [T, >= H*D] with unit inner stride")
+    q_stride = q.stride(0) if T > 1 else max(q.stride(0), H * D)
+    out_stride = out.stride(0) if T > 1 else max(out.stride(0), H * D)
+    _need(q_stride % 4 == 0 and out_stride % 4 == 0 and q.data_ptr() % 16 == 0 and out.data_ptr() % 16 == 0,
+          "attn_prefill_f32: q and out rows must be 16-byte aligned")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous(),
+          "attn_prefill_f32: block_tables must be contiguous int32 [S, W]")
+    _need(tiles.dtype == torch.int32 and tiles.dim() == 2 and tiles.shape[1] == 4 and tiles.is_contiguous(),
+          "attn_prefill_f32: tiles must be contiguous int32 [n, 4]")
+    _check(library().tm_attn_prefill_f32(_p(q), c_int(q_stride), _p(out), c_int(out_stride), _p(k_pool), _p(v_pool),
+                                         _p(block_tables), c_int(block_tables.shape[1]), _p(tiles),
+                                         c_int(tiles.shape[0]), c_int(H), c_int(KVH), c_int(D), c_int(page),
+                                         c_float(scale), c_int(window), _stream()), "attn_prefill_f32")
+    return out
+
+
 FUSED_DECODE_ROWS = 16      # most tokens the norm-fused decode products take
 
 
