@@ -215,3 +215,30 @@ def test_decode_steps_replayed_from_hip_graphs(model_dirs, plains, dtype_name):
     for p, o in zip(prompts, outs[True]):
         verify(plains["B"], p, o, DTYPES[dtype_name])
     assert outs[True] == outs[False]
+
+
+@pytest.mark.parametrize("portion", [16, 48])
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_prompt_portions_replayed_from_hip_graphs(model_dirs, plains, dtype_name, portion):
+    """Long prompts cut into portions of 16 tokens (this library's own products) or 48 (the library
+    products, which then are nodes of the graph), one request at a time: the second portion of a
+    length captures a graph, the later ones (of this prompt and of the next prompts, at other
+    positions and on other pages) replay it, with eager steps (the last, shorter portion; the decode
+    steps of other sizes) and synchronisations in between. Every replay must give what the eager
+    engine gives, and what the plain implementation gives."""
+    from tokenmill_amd import SamplingParams
+    lengths = [100, 77, 33, 120] if portion == 16 else [200, 150, 97, 240]
+    prompts = [random_ids(n, 384, 190 + i) for i, n in enumerate(lengths)]
+    sp = SamplingParams(max_tokens=5, ignore_eos=True)
+    outs = {}
+    for graphs in (False, True):
+        eng = make_engine(model_dirs["B"], dtype_name, block_size=16, hip_graphs=graphs, max_num_seqs=2,
+                          max_num_batched_tokens=portion, enable_chunked_prefill=True, max_model_len=256)
+        outs[graphs] = [eng.generate([p], sp)[0] for p in prompts]
+        if graphs:
+            pg = eng.runner.portion_graphs
+            assert pg.replays >= (15 if portion == 16 else 8) and (portion, False) in pg.portions
+        assert eng.cache.num_free_pages == eng.cache.num_pages
+    for p, o in zip(prompts, outs[True]):
+        verify(plains["B"], p, o, DTYPES[dtype_name])
+    assert outs[True] == outs[False]

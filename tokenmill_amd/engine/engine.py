@@ -72,8 +72,9 @@ class LLMEngine:
         self.cache = CacheManager(self.pools.windows, pages, cfg.block_size, cfg.max_num_seqs, cfg.watermark)
         self.runner = ModelRunner(model, self.pools, max_positions=cfg.max_model_len)
         if cfg.hip_graphs:
-            from tokenmill_amd.engine.graphs import DecodeGraphs
+            from tokenmill_amd.engine.graphs import DecodeGraphs, PortionGraphs
             self.runner.graphs = DecodeGraphs(self.runner, cfg)
+            self.runner.portion_graphs = PortionGraphs(self.runner)
         self.scheduler = Scheduler(cfg, self.cache)
         self.sampler = Sampler(self.device)
         self.seqs: dict[str, Sequence] = {}

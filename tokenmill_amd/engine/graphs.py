@@ -1,4 +1,4 @@
-"""HIP graphs for decode steps.
+"""HIP graphs for decode steps, and for prompt portions of a repeated length.
 
 A step in which every request decodes one token launches the same kernels with the same grids
 whatever the requests are, once the batch is padded to a bucket size and the block tables to the
@@ -9,6 +9,10 @@ profile of where an eager decode step's time goes, bench/results/profile/decode_
 
 Padding rows carry token 0 at position 0, a context of one key, and cache slot -1, which the cache
 write skips; their logits are never looked at. The graphs hold no memset node.
+
+A step that is one portion of one prompt launches the same kernels with the same grids as any other
+portion of that length (its positions, pages and tiles are data), so a long prompt cut into equal
+portions, or prompts of one length arriving one after the other, replay one graph: ``PortionGraphs``.
 """
 from __future__ import annotations
 
@@ -157,3 +161,69 @@ class DecodeGraphs:
         with torch.cuda.graph(graph):
             bk.logits = runner.model.forward(step, runner.pools.views)
         bk.graph = graph
+
+
+class _Portion:
+    def __init__(self):
+        self.dev: torch.Tensor | None = None
+        self.graph: torch.cuda.CUDAGraph | None = None
+        self.logits: torch.Tensor | None = None
+
+
+class PortionGraphs:
+    """Graphs for steps of exactly one entry with several tokens (a prompt or a portion of one) that
+    wants no logits or those of its last token. A shape (tokens, wants logits) is captured when it
+    comes the second time; the most recently used ``max_graphs`` shapes are kept (each holds the
+    activations of a step of its size)."""
+
+    def __init__(self, runner, max_graphs: int = 4):
+        self.runner = runner
+        ops.library_workspace(runner.device)
+        self.W = -(-runner.max_positions // runner.page_size)
+        self.max_graphs = max_graphs
+        self.seen: dict[tuple, int] = {}
+        self.portions: dict[tuple, _Portion] = {}          # insertion order = least recently used first
+        self.replays = 0
+
+    def can_run(self, entries) -> bool:
+        if len(entries) != 1 or self.runner.pools.states:
+            return False
+        e = entries[0]
+        return len(e.tokens) > 1 and list(e.want) in ([], [len(e.tokens) - 1])
+
+    @torch.inference_mode()
+    def run(self, entries) -> torch.Tensor | None:
+        """The step's logits ([1, vocab] or [0, vocab]), or None if this shape has no graph yet (the
+        caller then runs the step kernel by kernel)."""
+        runner = self.runner
+        e = entries[0]
+        key = (len(e.tokens), bool(e.want))
+        slot = self.portions.pop(key, None)
+        if slot is None:
+            self.seen[key] = self.seen.get(key, 0) + 1
+            if self.seen[key] < 2:
+                return None
+            slot = _Portion()
+            T, n_groups = len(e.tokens), len(runner.pools.groups)
+            n_ints = 3 * T + 2 + 2 + 1 + n_groups * (T + self.W) + 4 * (-(-T // 16))
+            slot.dev = torch.zeros(n_ints, dtype=torch.int32, device=runner.device)
+            step, _ = runner.prepare(entries, into=slot.dev, table_width=self.W)
+            torch.cuda.synchronize()
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):                   # a first run outside the graph: lazy set-up happens here
+                runner.model.forward(step, runner.pools.views)
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                slot.logits = runner.model.forward(step, runner.pools.views)
+            slot.graph = graph
+            while len(self.portions) >= self.max_graphs:    # the least recently used shape gives its memory back
+                self.portions.pop(next(iter(self.portions)))
+        else:
+            runner.prepare(entries, into=slot.dev, table_width=self.W)
+        self.portions[key] = slot
+        slot.graph.replay()
+        self.replays += 1
+        return slot.logits

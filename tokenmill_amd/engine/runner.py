@@ -46,6 +46,7 @@ class ModelRunner:
         self._copied = torch.cuda.Event()
         self._copy_pending = False
         self.graphs = None                        # DecodeGraphs when the engine runs with --hip-graphs
+        self.portion_graphs = None                # PortionGraphs likewise
 
     # ------------------------------------------------------------------------------------------------
 
@@ -57,10 +58,13 @@ class ModelRunner:
             self._pinned = torch.empty(max(n, 2 * self._pinned.numel()), dtype=torch.int32, pin_memory=True)
         return self._pinned.numpy()
 
-    def prepare(self, entries: list[StepEntry]) -> tuple[StepContext, list[int]]:
+    def prepare(self, entries: list[StepEntry], into: torch.Tensor | None = None,
+                table_width: int | None = None) -> tuple[StepContext, list[int]]:
         """Flatten the entries into device metadata. Returns the context and, for each wanted logit
         in the caller's order (entries in the given order, ``want`` in its order), its row in the
-        step's logits."""
+        step's logits. ``into``: a device int32 buffer to hold the metadata (a captured graph reads
+        it at a fixed address; steps of the same shape lay it out the same way); ``table_width``:
+        pad the block tables to this width instead of the widest of the step."""
         if not entries:
             raise StepError("a step needs at least one entry")
         page = self.page_size
@@ -87,6 +91,10 @@ class ModelRunner:
                 if not 0 <= w < len(e.tokens):
                     raise StepError(f"{e.cache.request_id}: wanted place {w} is not among its {len(e.tokens)} tokens")
         W = max(widths)
+        if table_width is not None:
+            if table_width < W:
+                raise StepError(f"block tables of {W} pages do not fit the width {table_width}")
+            W = table_width
         n_tiles = sum(-(-len(e.tokens) // 16) for e in entries if len(e.tokens) > 1)
         n_ints = 3 * T + (S + 1) + 2 * S + max(R, 1) + n_groups * (T + S * W) + 4 * n_tiles
         buf = self._staging(n_ints)
@@ -164,7 +172,13 @@ class ModelRunner:
         if R == 0:
             rows[0] = 0
 
-        dev = self._pinned[:off].to(self.device, non_blocking=True)
+        if into is None:
+            dev = self._pinned[:off].to(self.device, non_blocking=True)
+        else:
+            if into.numel() < off or into.dtype != torch.int32:
+                raise StepError("the metadata buffer is too small for this step")
+            dev = into[:off]
+            dev.copy_(self._pinned[:off], non_blocking=True)
         self._copied.record()
         self._copy_pending = True
 
@@ -193,5 +207,9 @@ class ModelRunner:
                 e.cache.fresh = False
         if self.graphs is not None and self.graphs.can_run(entries):
             return self.graphs.run(entries)
+        if self.portion_graphs is not None and self.portion_graphs.can_run(entries):
+            logits = self.portion_graphs.run(entries)
+            if logits is not None:
+                return logits
         ctx, _ = self.prepare(entries)
         return self.model.forward(ctx, self.pools.views)
