@@ -120,7 +120,15 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
         // KCH k-steps at a time with every load issued before the first product: a wavefront's whole
         // K range is at most one or two such groups, so it waits for memory once or twice, not per step.
         for (int base = ks0; base < ks1; base += KCH) {
-            Frag wf[KCH], uf[SILU ? KCH : 1];
+            // With one tile of tokens (decode steps) the activations are asked for first: loads come back
+            // in the order they were issued, and these few rows come from the cache long before the
+            // matrix arrives from HBM. With more tiles there are no registers for that.
+            Frag af[NT == 1 ? KCH : 1], wf[KCH], uf[SILU ? KCH : 1];
+            if constexpr (NT == 1) {
+#pragma unroll
+                for (int j = 0; j < KCH; ++j)
+                    af[j] = load_frag(arow[0], (base + j) * 32, K - 8 * g, a_ok[0] && base + j < ks1);
+            }
 #pragma unroll
             for (int j = 0; j < KCH; ++j) {
                 const bool in = base + j < ks1;
@@ -132,9 +140,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
                 const bool in = base + j < ks1;
 #pragma unroll
                 for (int t = 0; t < NT; ++t) {
-                    const Frag af = load_frag(arow[t], (base + j) * 32, K - 8 * g, a_ok[t] && in);
-                    acc[0][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[j].b, af.b, acc[0][t], 0, 0, 0);
-                    if (SILU) acc[1][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[j].b, af.b, acc[1][t], 0, 0, 0);
+                    Frag a1;
+                    if constexpr (NT == 1) a1 = af[j];
+                    else a1 = load_frag(arow[t], (base + j) * 32, K - 8 * g, a_ok[t] && in);
+                    acc[0][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[j].b, a1.b, acc[0][t], 0, 0, 0);
+                    if (SILU) acc[1][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[j].b, a1.b, acc[1][t], 0, 0, 0);
                 }
             }
         }
