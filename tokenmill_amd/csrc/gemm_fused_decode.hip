@@ -142,6 +142,42 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void fused_norm_gem
     load_group(fa, fb, ks0, cu.rows_ok);
     if constexpr (PIPE) load_group(fa2, fb2, ks0 + KCH, cu.rows_ok);
 
+    // What the epilogue will need from memory is asked for now, long before it is used: its address
+    // depends on a value that has to be loaded first (the token's position), two trips to memory that
+    // must not stand between the norm and the products.
+    struct EpilogueInputs {
+        float bias[2][4];
+        float cos[4], sin[4];
+        int slot;
+    };
+    const int tok = r;                                               // the epilogue's token of this lane
+    const bool epi_lane = wave == 0 && tok < M && 4 * g < ROWS;
+    auto epilogue_inputs = [&](const FusedUnit& t) {
+        EpilogueInputs e = {{{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}, {1.f, 1.f, 1.f, 1.f}, {0.f, 0.f, 0.f, 0.f}, -1};
+        if (EPI == FD_EPI_QKV && epi_lane) {
+            if (a.bias) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int ia = t.nA + 4 * g + i, ib = t.nB + 4 * g + i;
+                    e.bias[0][i] = a.bias_f32 ? ((const float*)a.bias)[ia] : bf16_to_f32(((const bf16_t*)a.bias)[ia]);
+                    e.bias[1][i] = a.bias_f32 ? ((const float*)a.bias)[ib] : bf16_to_f32(((const bf16_t*)a.bias)[ib]);
+                }
+            }
+            e.slot = a.slots ? a.slots[tok] : -1;
+            if (t.head < a.H + a.KVH) {
+                const size_t at = (size_t)a.positions[tok] * (a.D / 2) + ROWS * t.jt + 4 * g;
+                const f32x4_t cv = *(const f32x4_t*)(a.cos_t + at), sv = *(const f32x4_t*)(a.sin_t + at);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    e.cos[i] = cv[i];
+                    e.sin[i] = sv[i];
+                }
+            }
+        }
+        return e;
+    };
+    EpilogueInputs e_next = epilogue_inputs(cu);
+
     // x = norm(resid) into LDS. A row is shared by TPR threads of one wavefront (256 threads: 16 rows x 16
     // threads, 8 x 32, or 4 x 64); each keeps its first FD_RC vectors in registers between the two passes.
     const int mpad = fused_rows(M);
@@ -235,35 +271,8 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void fused_norm_gem
             accB = __builtin_amdgcn_mfma_f32_16x16x32_bf16(gb[j].b, xf.b, accB, 0, 0, 0);
         }
     };
-    const int tok = r;                                               // the epilogue's token of this lane
-    const bool epi_lane = wave == 0 && tok < M && 4 * g < ROWS;
-
     for (;;) {
-        // what the epilogue will need from memory is asked for now, long before it is used
-        float e_bias[2][4] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
-        float e_cos[4] = {1.f, 1.f, 1.f, 1.f}, e_sin[4] = {0.f, 0.f, 0.f, 0.f};
-        int e_slot = -1;
-        if (EPI == FD_EPI_QKV && epi_lane) {
-            if (a.bias) {
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int ia = cu.nA + 4 * g + i, ib = cu.nB + 4 * g + i;
-                    e_bias[0][i] = a.bias_f32 ? ((const float*)a.bias)[ia] : bf16_to_f32(((const bf16_t*)a.bias)[ia]);
-                    e_bias[1][i] = a.bias_f32 ? ((const float*)a.bias)[ib] : bf16_to_f32(((const bf16_t*)a.bias)[ib]);
-                }
-            }
-            e_slot = a.slots ? a.slots[tok] : -1;
-            if (cu.head < a.H + a.KVH) {
-                const size_t at = (size_t)a.positions[tok] * (a.D / 2) + ROWS * cu.jt + 4 * g;
-                const f32x4_t cv = *(const f32x4_t*)(a.cos_t + at), sv = *(const f32x4_t*)(a.sin_t + at);
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    e_cos[i] = cv[i];
-                    e_sin[i] = sv[i];
-                }
-            }
-        }
-
+        const EpilogueInputs e = e_next;                                 // asked for before this unit's products began
         accA = f32x4_t{0.f, 0.f, 0.f, 0.f};
         accB = f32x4_t{0.f, 0.f, 0.f, 0.f};
         if constexpr (PIPE) {
@@ -300,6 +309,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void fused_norm_gem
             wB = a.W + (size_t)(cu.nB + r) * K + 8 * g;
             load_group(fa, fb, ks0, cu.rows_ok);
             if constexpr (PIPE) load_group(fa2, fb2, ks0 + KCH, cu.rows_ok);
+            e_next = epilogue_inputs(cu);
         }
 
         if (epi_lane) {
@@ -335,18 +345,18 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void fused_norm_gem
                 float xA[4], xB[4];
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    xA[i] = fd_round(accA[i] + e_bias[0][i]);
-                    xB[i] = fd_round(accB[i] + e_bias[1][i]);
+                    xA[i] = fd_round(accA[i] + e.bias[0][i]);
+                    xB[i] = fd_round(accB[i] + e.bias[1][i]);
                 }
-                const int slot = e_slot;
+                const int slot = e.slot;
                 if (done.head < a.H + a.KVH) {
                     const int half = a.D / 2;
                     const int j0 = ROWS * done.jt + 4 * g;                       // pair index of element 0
                     float y1[4], y2[4];
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
-                        y1[i] = xA[i] * e_cos[i] - xB[i] * e_sin[i];
-                        y2[i] = xB[i] * e_cos[i] + xA[i] * e_sin[i];
+                        y1[i] = xA[i] * e.cos[i] - xB[i] * e.sin[i];
+                        y2[i] = xB[i] * e.cos[i] + xA[i] * e.sin[i];
                     }
                     bf16_t* dst = nullptr;
                     if (done.head < a.H)
