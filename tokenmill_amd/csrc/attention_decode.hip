@@ -248,7 +248,7 @@ __global__ __launch_bounds__(64 * WAVES) void attn_decode_block_kernel(
 // split kernels: grid (S, KVH, chunks) with four wavefronts, then the merge
 // ------------------------------------------------------------------------------------------------
 template <int D>
-__global__ __launch_bounds__(256) void attn_decode_split_kernel(
+__global__ __launch_bounds__(256, D <= 64 ? 4 : 2) void attn_decode_split_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_pool,
     const bf16_t* __restrict__ v_pool, const int* __restrict__ block_tables, int table_width,
     const int* __restrict__ context_lens, float* __restrict__ part_o, float* __restrict__ part_ml,

@@ -67,9 +67,29 @@ struct Operands {
     hipStream_t stream;
 };
 
-// Mean time of a few runs of one algorithm on the caller's own operands (the result is the same
-// whichever algorithm wrote it last, up to rounding); negative if it fails.
-float time_algo(hipblasLtHandle_t handle, const Plan& p, const hipblasLtMatmulAlgo_t& algo, const Operands& op) {
+// What the timed runs evict the caches with: larger than the last-level cache, so that every timed
+// product finds its matrix in HBM, as it does inside a step (a decode step reads about a gigabyte of
+// other matrices between two uses of this one). Made when the first shape is timed, never freed.
+constexpr size_t FLUSH_BYTES = (size_t)768 << 20;
+std::unordered_map<int, void*> g_flush;                      // per device; nullptr: could not be allocated
+
+void* flush_buffer(int device) {
+    auto it = g_flush.find(device);
+    if (it != g_flush.end()) return it->second;
+    void* buf = nullptr;
+    if (hipMalloc(&buf, FLUSH_BYTES) != hipSuccess) {
+        (void)hipGetLastError();
+        buf = nullptr;
+    }
+    g_flush[device] = buf;
+    return buf;
+}
+
+// Mean time of a few runs of one algorithm on the caller's own operands, each run after the caches
+// were flushed (the result is the same whichever algorithm wrote it last, up to rounding);
+// negative if it fails.
+float time_algo(hipblasLtHandle_t handle, const Plan& p, const hipblasLtMatmulAlgo_t& algo, const Operands& op,
+                void* flush) {
     const float one = 1.f, zero = 0.f;
     hipEvent_t t0, t1;
     if (hipEventCreate(&t0) != hipSuccess) return -1.f;
@@ -77,19 +97,22 @@ float time_algo(hipblasLtHandle_t handle, const Plan& p, const hipblasLtMatmulAl
         hipEventDestroy(t0);
         return -1.f;
     }
-    float ms = -1.f;
+    constexpr int WARM = 1, TIMED = 4;
+    float total = 0.f;
     bool ok = true;
-    for (int i = 0; i < 2 + 5 && ok; ++i) {
-        if (i == 2) hipEventRecord(t0, op.stream);
-        ok = hipblasLtMatmul(handle, p.desc, &one, op.W, p.w, op.A, p.a, &zero, op.C, p.c, op.C, p.c, &algo, op.workspace,
-                             op.workspace_bytes, op.stream) == HIPBLAS_STATUS_SUCCESS;
+    for (int i = 0; i < WARM + TIMED && ok; ++i) {
+        if (flush) ok = hipMemsetAsync(flush, i, FLUSH_BYTES, op.stream) == hipSuccess;
+        hipEventRecord(t0, op.stream);
+        ok = ok && hipblasLtMatmul(handle, p.desc, &one, op.W, p.w, op.A, p.a, &zero, op.C, p.c, op.C, p.c, &algo,
+                                   op.workspace, op.workspace_bytes, op.stream) == HIPBLAS_STATUS_SUCCESS;
+        hipEventRecord(t1, op.stream);
+        float ms = 0.f;
+        ok = ok && hipEventSynchronize(t1) == hipSuccess && hipEventElapsedTime(&ms, t0, t1) == hipSuccess;
+        if (i >= WARM) total += ms;
     }
-    hipEventRecord(t1, op.stream);
-    if (hipEventSynchronize(t1) == hipSuccess && ok && hipEventElapsedTime(&ms, t0, t1) == hipSuccess) ms /= 5.f;
-    else ms = -1.f;
     hipEventDestroy(t0);
     hipEventDestroy(t1);
-    return ms;
+    return ok ? total / TIMED : -1.f;
 }
 
 bool make_plan(hipblasLtHandle_t handle, const PlanKey& k, const Operands& op, Plan& p) {
@@ -129,14 +152,19 @@ bool make_plan(hipblasLtHandle_t handle, const PlanKey& k, const Operands& op, P
     if (want > 1) {
         if (k.bias_dtype != TM_NONE)
             hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &op.bias, sizeof(op.bias));
-        // The heuristic's first choice stays unless another candidate beats it clearly: the runs
-        // timed here follow each other with the operands in cache, which flatters some candidates
-        // by a few percent against the cold matrices of a real step.
+        // The heuristic's first choice stays unless another candidate beats it clearly (timings of a
+        // few runs scatter by some percent).
+        // Flushed where the matrix is the larger part of what the product reads and writes (few
+        // rows: the matrix comes from HBM in a real step); with many rows the activations, which the
+        // kernel before has just written, are the larger part, and those are in cache in a step too.
+        const size_t out_size = k.out_f32 ? 4 : 2;
+        const bool cold = (size_t)k.N * k.K * 2 > (size_t)k.M * k.K * 2 + (size_t)k.M * k.N * out_size;
+        void* flush = cold ? flush_buffer(k.device) : nullptr;
         float best_ms = 0.f, first_ms = -1.f;
         int first = -1;
         for (int i = 0; i < n_found; ++i) {
             if (found[i].state != HIPBLAS_STATUS_SUCCESS || found[i].workspaceSize > workspace_bytes) continue;
-            const float ms = time_algo(handle, p, found[i].algo, op);
+            const float ms = time_algo(handle, p, found[i].algo, op, flush);
             if (ms < 0.f) continue;
             if (first < 0) {
                 first = i;
@@ -147,7 +175,7 @@ bool make_plan(hipblasLtHandle_t handle, const PlanKey& k, const Operands& op, P
                 best_ms = ms;
             }
         }
-        if (first >= 0 && best_ms > 0.85f * first_ms) best = first;
+        if (first >= 0 && best_ms > 0.93f * first_ms) best = first;
     }
     if (best < 0) {                         // untimed, or nothing could be timed: the heuristic's first valid choice
         for (int i = 0; i < n_found && best < 0; ++i)
