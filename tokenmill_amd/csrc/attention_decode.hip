@@ -47,46 +47,60 @@ union Bf16x8Bits {
     bf16x8_t b;
 };
 
-// The partial of 64 keys [wbase, wbase + 64) for the (up to 16) query heads of one kv head.
-// Every load is issued before the first product. m is in units of score * scale * log2(e).
+// The keys and values of 64 positions [wbase, wbase + 64) of one kv head as a wavefront holds them
+// between asking for them and using them: four 16-key tiles of MFMA operands.
 template <int D>
-__device__ __forceinline__ void wave_keys64(const Bf16x8Bits (&qreg)[D / 32], const bf16_t* __restrict__ k_pool,
+struct Keys64 {
+    int tile_page[4];                       // page of each tile, -1 if no query may see it (wave-uniform)
+    Bf16x8Bits k[4][D / 32];
+    u32x2_t v[D / 16][4];
+};
+
+// Ask for the keys and values of [wbase, wbase + 64): every load is issued, nothing is waited for.
+template <int D>
+__device__ __forceinline__ void load_keys64(Keys64<D>& kv, const bf16_t* __restrict__ k_pool,
                                             const bf16_t* __restrict__ v_pool, const int* __restrict__ table,
-                                            int wbase, int ctx, int lo, int kvh, int KVH, int page_shift,
-                                            float scale_log2, int r, int g, float& m, float& l,
-                                            f32x4_t (&o)[D / 16]) {
+                                            int wbase, int ctx, int lo, int kvh, int KVH, int page_shift, int r,
+                                            int g) {
     constexpr int NDC = D / 32, NDT = D / 16;
     const int page_mask = (1 << page_shift) - 1;
-    int tile_page[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
         const int tile0 = wbase + 16 * t;
-        tile_page[t] = (tile0 < ctx && tile0 + 16 > lo) ? table[tile0 >> page_shift] : -1;      // wave-uniform
+        kv.tile_page[t] = (tile0 < ctx && tile0 + 16 > lo) ? table[tile0 >> page_shift] : -1;      // wave-uniform
     }
-    Bf16x8Bits kreg[4][NDC];
-    u32x2_t vreg[NDT][4];
+    // Every load is unconditional, so that none of them has to be waited for before the next is
+    // issued: a tile nobody may see reads page 0 instead, and keys beyond the context read the rest of
+    // their page. What such loads bring is never used: their scores are replaced by -inf and their
+    // values are masked bit by bit.
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
         const int tile0 = wbase + 16 * t;
         const int in_page = tile0 & page_mask;
-        const bool have = tile_page[t] >= 0;
-        const size_t pg = have ? (size_t)tile_page[t] : 0;
+        const size_t pg = kv.tile_page[t] >= 0 ? (size_t)kv.tile_page[t] : 0;
         const bf16_t* kr = k_pool + (((pg << page_shift) + in_page + r) * KVH + kvh) * D + 8 * g;
         const bf16_t* vr = v_pool + (((pg * KVH + kvh) * D + r) << page_shift) + in_page + 4 * g;
 #pragma unroll
-        for (int c = 0; c < NDC; ++c)
-            kreg[t][c].u = (have && tile0 + r < ctx) ? *(const u32x4_t*)(kr + 32 * c) : u32x4_t{0, 0, 0, 0};
+        for (int c = 0; c < NDC; ++c) kv.k[t][c].u = *(const u32x4_t*)(kr + 32 * c);
 #pragma unroll
-        for (int dt = 0; dt < NDT; ++dt)
-            vreg[dt][t] = have ? *(const u32x2_t*)(vr + ((size_t)(16 * dt) << page_shift)) : u32x2_t{0, 0};
+        for (int dt = 0; dt < NDT; ++dt) kv.v[dt][t] = *(const u32x2_t*)(vr + ((size_t)(16 * dt) << page_shift));
     }
+}
+
+// The partial of the 64 keys in kv for the (up to 16) query heads of one kv head.
+// m is in units of score * scale * log2(e).
+template <int D>
+__device__ __forceinline__ void attend_keys64(const Keys64<D>& kv, const Bf16x8Bits (&qreg)[D / 32], int wbase, int ctx,
+                                              int lo, float scale_log2, int g, float& m, float& l,
+                                              f32x4_t (&o)[D / 16]) {
+    constexpr int NDC = D / 32, NDT = D / 16;
     float sc[4][4];                                                 // [16-key tile][key 4g+i] for head r
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
         f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int c = 0; c < NDC; ++c)
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[t][c].b, qreg[c].b, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kv.k[t][c].b, qreg[c].b, acc, 0, 0, 0);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int kj = wbase + 16 * t + 4 * g + i;
@@ -117,7 +131,7 @@ __device__ __forceinline__ void wave_keys64(const Bf16x8Bits (&qreg)[D / 32], co
     for (int dt = 0; dt < NDT; ++dt) o[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
-        if (tile_page[2 * b] < 0 && tile_page[2 * b + 1] < 0) continue;
+        if (kv.tile_page[2 * b] < 0 && kv.tile_page[2 * b + 1] < 0) continue;
         Bf16x8Bits pt;
         pt.u = u32x4_t{pack_bf16(pr[2 * b][0], pr[2 * b][1]), pack_bf16(pr[2 * b][2], pr[2 * b][3]),
                        pack_bf16(pr[2 * b + 1][0], pr[2 * b + 1][1]), pack_bf16(pr[2 * b + 1][2], pr[2 * b + 1][3])};
@@ -135,11 +149,23 @@ __device__ __forceinline__ void wave_keys64(const Bf16x8Bits (&qreg)[D / 32], co
 #pragma unroll
         for (int dt = 0; dt < NDT; ++dt) {
             Bf16x8Bits vf;
-            vf.u = u32x4_t{vreg[dt][2 * b][0] & keep[0], vreg[dt][2 * b][1] & keep[1],
-                           vreg[dt][2 * b + 1][0] & keep[2], vreg[dt][2 * b + 1][1] & keep[3]};
+            vf.u = u32x4_t{kv.v[dt][2 * b][0] & keep[0], kv.v[dt][2 * b][1] & keep[1],
+                           kv.v[dt][2 * b + 1][0] & keep[2], kv.v[dt][2 * b + 1][1] & keep[3]};
             o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.b, pt.b, o[dt], 0, 0, 0);
         }
     }
+}
+
+// Load, then attend: the partial of 64 keys [wbase, wbase + 64).
+template <int D>
+__device__ __forceinline__ void wave_keys64(const Bf16x8Bits (&qreg)[D / 32], const bf16_t* __restrict__ k_pool,
+                                            const bf16_t* __restrict__ v_pool, const int* __restrict__ table,
+                                            int wbase, int ctx, int lo, int kvh, int KVH, int page_shift,
+                                            float scale_log2, int r, int g, float& m, float& l,
+                                            f32x4_t (&o)[D / 16]) {
+    Keys64<D> kv;
+    load_keys64<D>(kv, k_pool, v_pool, table, wbase, ctx, lo, kvh, KVH, page_shift, r, g);
+    attend_keys64<D>(kv, qreg, wbase, ctx, lo, scale_log2, g, m, l, o);
 }
 
 template <int D>
@@ -184,10 +210,7 @@ __global__ __launch_bounds__(64 * WAVES) void attn_decode_block_kernel(
 #pragma unroll
     for (int dt = 0; dt < NDT; ++dt) o[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     const int first = (lo / AD_WKEYS) * AD_WKEYS;                   // aligned to 64 positions
-    for (int wbase = first + wave * AD_WKEYS; wbase < ctx; wbase += WAVES * AD_WKEYS) {
-        float mi, li;
-        f32x4_t oi[NDT];
-        wave_keys64<D>(qreg, k_pool, v_pool, table, wbase, ctx, lo, kvh, KVH, page_shift, scale_log2, r, g, mi, li, oi);
+    auto fold = [&](float mi, float li, const f32x4_t (&oi)[NDT]) {  // add a partial to the running one
         const float mn = fmaxf(m, mi);
         const float f0 = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m - mn);
         const float f1 = (mi == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mi - mn);
@@ -197,6 +220,12 @@ __global__ __launch_bounds__(64 * WAVES) void attn_decode_block_kernel(
 #pragma unroll
             for (int i = 0; i < 4; ++i) o[dt][i] = o[dt][i] * f0 + oi[dt][i] * f1;
         m = mn;
+    };
+    for (int wbase = first + wave * AD_WKEYS; wbase < ctx; wbase += WAVES * AD_WKEYS) {
+        float mi, li;
+        f32x4_t oi[NDT];
+        wave_keys64<D>(qreg, k_pool, v_pool, table, wbase, ctx, lo, kvh, KVH, page_shift, scale_log2, r, g, mi, li, oi);
+        fold(mi, li, oi);
     }
     // merge the wavefronts in wavefront order; lane: head r, d = 16 dt + 4 g + i
     if (g == 0) {

@@ -358,7 +358,7 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, out
 
 
 DECODE_CHUNK = 256          # keys per block of the split decode attention
-DECODE_SPLIT_PAIRS = 128    # below this many (request, kv head) pairs the split kernels (with scratch memory) run
+DECODE_SPLIT_PAIRS = 192    # below this many (request, kv head) pairs the split kernels (with scratch memory) run
 
 
 def attn_decode_mfma_supported(dtype, H: int, KVH: int, D: int, page: int) -> bool:
