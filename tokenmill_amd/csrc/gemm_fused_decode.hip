@@ -188,6 +188,23 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void fused_norm_gem
         const int step = 4 * tpr;
         if (row < M) {
             const float* src = a.resid + (size_t)row * K;
+            // The norm's weights of the first group are asked for with the row itself: they depend on
+            // nothing, and asked for after the sum of squares they would cost a trip to memory of their
+            // own. (Two kinds of loads behind one run-time test would each be waited for singly: the
+            // test on the weights' type stands outside the loops.)
+            const bool w16 = !a.norm_w_f32;
+            auto widen = [](const uint2 wv) {
+                return f32x4_t{__uint_as_float(wv.x << 16), __uint_as_float(wv.x & 0xffff0000u),
+                               __uint_as_float(wv.y << 16), __uint_as_float(wv.y & 0xffff0000u)};
+            };
+            uint2 wraw[FD_RC];
+            if (w16) {
+#pragma unroll
+                for (int j = 0; j < FD_RC; ++j) {
+                    const int c = sub * 4 + j * step;
+                    wraw[j] = c < K ? *(const uint2*)((const bf16_t*)a.norm_w + c) : uint2{0u, 0u};
+                }
+            }
             f32x4_t cache[FD_RC];
             float ss = 0.f;
 #pragma unroll
@@ -209,31 +226,23 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void fused_norm_gem
             }
             for (int off = 1; off < tpr; off <<= 1) ss += __shfl_xor(ss, off, TM_WAVE);
             const float rs = rsqrtf(ss / (float)K + a.eps);
-            auto weight_at = [&](int c) {
-                f32x4_t w;
-                if (a.norm_w_f32) {
-                    w = *(const f32x4_t*)((const float*)a.norm_w + c);
-                } else {
-                    const uint2 wv = *(const uint2*)((const bf16_t*)a.norm_w + c);
-                    w = f32x4_t{__uint_as_float(wv.x << 16), __uint_as_float(wv.x & 0xffff0000u),
-                                __uint_as_float(wv.y << 16), __uint_as_float(wv.y & 0xffff0000u)};
-                }
-                return w;
-            };
             auto emit = [&](int c, const f32x4_t v, const f32x4_t w) {
                 uint2 pk;
                 pk.x = fd_pack(w[0] * fd_round(v[0] * rs), w[1] * fd_round(v[1] * rs));
                 pk.y = fd_pack(w[2] * fd_round(v[2] * rs), w[3] * fd_round(v[3] * rs));
                 *(uint2*)(xrow + c) = pk;
             };
-            // the weights of a group are asked for together (and with the row's values where those
-            // are read again), so that a group costs one trip to memory
             {
                 f32x4_t w[FD_RC];
+                if (w16) {
 #pragma unroll
-                for (int j = 0; j < FD_RC; ++j) {
-                    const int c = sub * 4 + j * step;
-                    w[j] = c < K ? weight_at(c) : f32x4_t{0.f, 0.f, 0.f, 0.f};
+                    for (int j = 0; j < FD_RC; ++j) w[j] = widen(wraw[j]);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < FD_RC; ++j) {
+                        const int c = sub * 4 + j * step;
+                        w[j] = c < K ? *(const f32x4_t*)((const float*)a.norm_w + c) : f32x4_t{0.f, 0.f, 0.f, 0.f};
+                    }
                 }
 #pragma unroll
                 for (int j = 0; j < FD_RC; ++j) {
@@ -241,13 +250,26 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void fused_norm_gem
                     if (c < K) emit(c, cache[j], w[j]);
                 }
             }
+            // the rest of a long row: the values again and their weights, a group in flight together
             for (int c0 = sub * 4 + FD_RC * step; c0 < K; c0 += FD_RC * step) {
                 f32x4_t v[FD_RC], w[FD_RC];
+                if (w16) {
+                    uint2 raw[FD_RC];
 #pragma unroll
-                for (int j = 0; j < FD_RC; ++j) {
-                    const bool in = c0 + j * step < K;
-                    v[j] = in ? *(const f32x4_t*)(src + c0 + j * step) : f32x4_t{0.f, 0.f, 0.f, 0.f};
-                    w[j] = in ? weight_at(c0 + j * step) : f32x4_t{0.f, 0.f, 0.f, 0.f};
+                    for (int j = 0; j < FD_RC; ++j) {
+                        const bool in = c0 + j * step < K;
+                        v[j] = in ? *(const f32x4_t*)(src + c0 + j * step) : f32x4_t{0.f, 0.f, 0.f, 0.f};
+                        raw[j] = in ? *(const uint2*)((const bf16_t*)a.norm_w + c0 + j * step) : uint2{0u, 0u};
+                    }
+#pragma unroll
+                    for (int j = 0; j < FD_RC; ++j) w[j] = widen(raw[j]);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < FD_RC; ++j) {
+                        const bool in = c0 + j * step < K;
+                        v[j] = in ? *(const f32x4_t*)(src + c0 + j * step) : f32x4_t{0.f, 0.f, 0.f, 0.f};
+                        w[j] = in ? *(const f32x4_t*)((const float*)a.norm_w + c0 + j * step) : f32x4_t{0.f, 0.f, 0.f, 0.f};
+                    }
                 }
 #pragma unroll
                 for (int j = 0; j < FD_RC; ++j)
