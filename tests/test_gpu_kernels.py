@@ -483,6 +483,21 @@ def test_paged_attention_decode_mfma(ops, H, KVH, D, page, window):
                          case["tables"][sub].contiguous().to(DEV), ctx[sub].contiguous(), H, KVH, D, scale, window,
                          max(lens))
     assert torch.equal(out2, out[sub])
+    # block tables wider than any context (the shape a captured graph has), scratch memory full of NaN
+    # beyond what the step writes: up to 64 chunks the merge reads ahead of the context length, beyond
+    # that another merge kernel runs
+    for max_context in (4096, 20000):
+        width = -(-max_context // page)
+        tables = torch.zeros(S, width, dtype=torch.int32)
+        tables[:, :case["tables"].shape[1]] = case["tables"]
+        chunks = -(-max_context // ops.DECODE_CHUNK)
+        ws = (torch.full((S, H, chunks, D), float("nan"), device=DEV), torch.full((S, H, chunks, 2), float("nan"), device=DEV))
+        out3 = torch.full((S, H * D), 3.0, dtype=dt, device=DEV)
+        ops.attn_decode_mfma(wide, out3, case["kp"].to(DEV), v_layout(case["vp"]).to(DEV), tables.to(DEV), ctx,
+                             H, KVH, D, scale, window, max_context, workspace=ws)
+        torch.testing.assert_close(out3.float().cpu(), want, **tol(dt))
+        if not window:
+            assert torch.equal(out3, out)
 
 
 def tiles_for(lens, q_lens):

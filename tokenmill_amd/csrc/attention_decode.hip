@@ -56,18 +56,29 @@ struct Keys64 {
     u32x2_t v[D / 16][4];
 };
 
+// The block-table entries of the four 16-key tiles of [wbase, wbase + 64), read without a test at an
+// index inside the row (what lies beyond the context is dropped by load_keys64): they depend on
+// nothing but the request, so a kernel can ask for them before it knows the context length.
+__device__ __forceinline__ void load_table_entries(int (&entry)[4], const int* __restrict__ table, int table_width,
+                                                   int wbase, int page_shift) {
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        const int at = (wbase + 16 * t) >> page_shift;
+        entry[t] = table[at < table_width ? at : table_width - 1];
+    }
+}
+
 // Ask for the keys and values of [wbase, wbase + 64): every load is issued, nothing is waited for.
 template <int D>
 __device__ __forceinline__ void load_keys64(Keys64<D>& kv, const bf16_t* __restrict__ k_pool,
-                                            const bf16_t* __restrict__ v_pool, const int* __restrict__ table,
-                                            int wbase, int ctx, int lo, int kvh, int KVH, int page_shift, int r,
-                                            int g) {
+                                            const bf16_t* __restrict__ v_pool, const int (&entry)[4], int wbase,
+                                            int ctx, int lo, int kvh, int KVH, int page_shift, int r, int g) {
     constexpr int NDC = D / 32, NDT = D / 16;
     const int page_mask = (1 << page_shift) - 1;
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
         const int tile0 = wbase + 16 * t;
-        kv.tile_page[t] = (tile0 < ctx && tile0 + 16 > lo) ? table[tile0 >> page_shift] : -1;      // wave-uniform
+        kv.tile_page[t] = (tile0 < ctx && tile0 + 16 > lo) ? entry[t] : -1;                         // wave-uniform
     }
     // Every load is unconditional, so that none of them has to be waited for before the next is
     // issued: a tile nobody may see reads page 0 instead, and keys beyond the context read the rest of
@@ -85,6 +96,9 @@ __device__ __forceinline__ void load_keys64(Keys64<D>& kv, const bf16_t* __restr
 #pragma unroll
         for (int dt = 0; dt < NDT; ++dt) kv.v[dt][t] = *(const u32x2_t*)(vr + ((size_t)(16 * dt) << page_shift));
     }
+    // nothing that uses the keys may be scheduled above the loads of the values: both are on their
+    // way before the first wait
+    __builtin_amdgcn_sched_barrier(0);
 }
 
 // The partial of the 64 keys in kv for the (up to 16) query heads of one kv head.
@@ -131,7 +145,6 @@ __device__ __forceinline__ void attend_keys64(const Keys64<D>& kv, const Bf16x8B
     for (int dt = 0; dt < NDT; ++dt) o[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
-        if (kv.tile_page[2 * b] < 0 && kv.tile_page[2 * b + 1] < 0) continue;
         Bf16x8Bits pt;
         pt.u = u32x4_t{pack_bf16(pr[2 * b][0], pr[2 * b][1]), pack_bf16(pr[2 * b][2], pr[2 * b][3]),
                        pack_bf16(pr[2 * b + 1][0], pr[2 * b + 1][1]), pack_bf16(pr[2 * b + 1][2], pr[2 * b + 1][3])};
@@ -160,11 +173,13 @@ __device__ __forceinline__ void attend_keys64(const Keys64<D>& kv, const Bf16x8B
 template <int D>
 __device__ __forceinline__ void wave_keys64(const Bf16x8Bits (&qreg)[D / 32], const bf16_t* __restrict__ k_pool,
                                             const bf16_t* __restrict__ v_pool, const int* __restrict__ table,
-                                            int wbase, int ctx, int lo, int kvh, int KVH, int page_shift,
-                                            float scale_log2, int r, int g, float& m, float& l,
+                                            int table_width, int wbase, int ctx, int lo, int kvh, int KVH,
+                                            int page_shift, float scale_log2, int r, int g, float& m, float& l,
                                             f32x4_t (&o)[D / 16]) {
+    int entry[4];
+    load_table_entries(entry, table, table_width, wbase, page_shift);
     Keys64<D> kv;
-    load_keys64<D>(kv, k_pool, v_pool, table, wbase, ctx, lo, kvh, KVH, page_shift, r, g);
+    load_keys64<D>(kv, k_pool, v_pool, entry, wbase, ctx, lo, kvh, KVH, page_shift, r, g);
     attend_keys64<D>(kv, qreg, wbase, ctx, lo, scale_log2, g, m, l, o);
 }
 
@@ -224,7 +239,7 @@ __global__ __launch_bounds__(64 * WAVES) void attn_decode_block_kernel(
     for (int wbase = first + wave * AD_WKEYS; wbase < ctx; wbase += WAVES * AD_WKEYS) {
         float mi, li;
         f32x4_t oi[NDT];
-        wave_keys64<D>(qreg, k_pool, v_pool, table, wbase, ctx, lo, kvh, KVH, page_shift, scale_log2, r, g, mi, li, oi);
+        wave_keys64<D>(qreg, k_pool, v_pool, table, table_width, wbase, ctx, lo, kvh, KVH, page_shift, scale_log2, r, g, mi, li, oi);
         fold(mi, li, oi);
     }
     // merge the wavefronts in wavefront order; lane: head r, d = 16 dt + 4 g + i
@@ -277,7 +292,7 @@ __global__ __launch_bounds__(64 * WAVES) void attn_decode_block_kernel(
 // split kernels: grid (S, KVH, chunks) with four wavefronts, then the merge
 // ------------------------------------------------------------------------------------------------
 template <int D>
-__global__ __launch_bounds__(256, D <= 64 ? 4 : 2) void attn_decode_split_kernel(
+__global__ __launch_bounds__(256) void attn_decode_split_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_pool,
     const bf16_t* __restrict__ v_pool, const int* __restrict__ block_tables, int table_width,
     const int* __restrict__ context_lens, float* __restrict__ part_o, float* __restrict__ part_ml,
@@ -287,20 +302,26 @@ __global__ __launch_bounds__(256, D <= 64 ? 4 : 2) void attn_decode_split_kernel
     __shared__ float s_o[4][16][D + 1];
     const int s = blockIdx.x, kvh = blockIdx.y, chunk = blockIdx.z;
     const int G = H / KVH;
-    const int ctx = context_lens[s];
-    const int p = ctx - 1;
-    const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
-    const int chunk_lo = chunk * AD_CHUNK;
-    if (chunk_lo >= ctx || chunk_lo + AD_CHUNK <= lo) return;       // nothing of this chunk is visible
     const int wave = threadIdx.x / TM_WAVE, lane = threadIdx.x % TM_WAVE;
     const int r = lane % 16, g = lane / 16;
-    const int* table = block_tables + (size_t)s * table_width;
+    const int chunk_lo = chunk * AD_CHUNK, wbase = chunk_lo + wave * AD_WKEYS;
+    // the context length, the block-table entries and the query are asked for together: one trip to
+    // memory before the keys, not two
+    const int ctx = context_lens[s];
+    int entry[4];
+    load_table_entries(entry, block_tables + (size_t)s * table_width, table_width, wbase, page_shift);
     Bf16x8Bits qreg[D / 32];
     load_q_operand<D>(qreg, q + (size_t)s * q_stride, G, kvh, r, g);
+    const int p = ctx - 1;
+    const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+    if (chunk_lo >= ctx || chunk_lo + AD_CHUNK <= lo) return;       // nothing of this chunk is visible
     float m, l;
     f32x4_t o[NDT];
-    wave_keys64<D>(qreg, k_pool, v_pool, table, chunk_lo + wave * AD_WKEYS, ctx, lo, kvh, KVH, page_shift, scale_log2,
-                   r, g, m, l, o);
+    {
+        Keys64<D> kv;
+        load_keys64<D>(kv, k_pool, v_pool, entry, wbase, ctx, lo, kvh, KVH, page_shift, r, g);
+        attend_keys64<D>(kv, qreg, wbase, ctx, lo, scale_log2, g, m, l, o);
+    }
     if (g == 0) {
         s_m[wave][r] = m;
         s_l[wave][r] = l;
@@ -332,11 +353,82 @@ __global__ __launch_bounds__(256, D <= 64 ? 4 : 2) void attn_decode_split_kernel
 }
 
 // out[s, h, :] = the partial values of the visible chunks, weighted and normalised. Four wavefronts
-// share a (request, head): wavefront w adds the chunks c0 + w, c0 + w + 4, ... in ascending order and
-// the four sums are added in wavefront order, so the order of additions depends on the context
-// length and the window only. A lane holds elements d = lane and lane + 64 of the head.
+// share a (request, head): wavefront w adds the chunks w, w + 4, ... in ascending order and the four
+// sums are added in wavefront order, so the order of additions depends on the context length and
+// the window only. A lane holds elements d = lane and lane + 64 of the head.
+// For up to 64 chunks: lane c of every wavefront holds (max, sum) of chunk c, and those and the
+// values of the first 16 chunks are asked for together with the context length, before it is known
+// which of them count (scratch memory beyond the context holds anything: it is dropped by selects,
+// never multiplied): one trip to memory for contexts up to 4,096.
 #define AD_MERGE_WAVES 4
 __global__ __launch_bounds__(64 * AD_MERGE_WAVES) void attn_decode_merge_kernel(
+    const float* __restrict__ part_o, const float* __restrict__ part_ml, const int* __restrict__ context_lens,
+    bf16_t* __restrict__ out, int out_stride, int max_chunks, int H, int D, int window) {
+    __shared__ float s_l[AD_MERGE_WAVES], s_o[AD_MERGE_WAVES][128];
+    const int s = blockIdx.x, h = blockIdx.y;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / TM_WAVE), lane = threadIdx.x % TM_WAVE;
+    const size_t base = ((size_t)s * H + h) * max_chunks;
+    const int last = max_chunks - 1;
+    const int ctx = context_lens[s];
+    const f32x2_t ml = *(const f32x2_t*)(part_ml + (base + (lane < last ? lane : last)) * 2);
+    const int d0 = lane < D ? lane : D - 1, d1 = lane + 64 < D ? lane + 64 : D - 1;
+    float a0[4], a1[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int c = wave + AD_MERGE_WAVES * i;
+        const float* src = part_o + (base + (c < last ? c : last)) * D;
+        a0[i] = src[d0];
+        a1[i] = src[d1];
+    }
+    const int p = ctx - 1;
+    const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+    const int c0 = lo / AD_CHUNK, c1 = (ctx - 1) / AD_CHUNK;
+    const float mm = wave_max((lane >= c0 && lane <= c1) ? ml[0] : -INFINITY);
+    float ll = 0.f, o0 = 0.f, o1 = 0.f;
+    auto add_chunk = [&](int c, float v0, float v1) {               // c is the same in every lane
+        const float mc = __shfl(ml[0], c, TM_WAVE), lc = __shfl(ml[1], c, TM_WAVE);
+        const bool in = c >= c0 && c <= c1 && mc != -INFINITY;
+        const float f = in ? __builtin_amdgcn_exp2f(mc - mm) : 0.f;
+        ll = fmaf(in ? lc : 0.f, f, ll);
+        o0 = fmaf(in ? v0 : 0.f, f, o0);
+        o1 = fmaf(in ? v1 : 0.f, f, o1);
+    };
+#pragma unroll
+    for (int i = 0; i < 4; ++i) add_chunk(wave + AD_MERGE_WAVES * i, a0[i], a1[i]);
+    // chunks from 16 on (contexts beyond 4,096), four to a wavefront at a time
+    for (int cb = 4 * AD_MERGE_WAVES; cb <= c1; cb += 4 * AD_MERGE_WAVES) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int c = cb + wave + AD_MERGE_WAVES * i;
+            const float* src = part_o + (base + (c < last ? c : last)) * D;
+            a0[i] = src[d0];
+            a1[i] = src[d1];
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) add_chunk(cb + wave + AD_MERGE_WAVES * i, a0[i], a1[i]);
+    }
+    if (lane == 0) s_l[wave] = ll;
+    s_o[wave][lane] = o0;
+    s_o[wave][lane + 64] = o1;
+    __syncthreads();
+    if (wave != 0) return;
+    ll = s_l[0];
+    o0 = s_o[0][lane];
+    o1 = s_o[0][lane + 64];
+#pragma unroll
+    for (int w = 1; w < AD_MERGE_WAVES; ++w) {
+        ll += s_l[w];
+        o0 += s_o[w][lane];
+        o1 += s_o[w][lane + 64];
+    }
+    bf16_t* orow = out + (size_t)s * out_stride + (size_t)h * D;
+    if (lane < D) orow[lane] = f32_to_bf16(o0 / ll);
+    if (lane + 64 < D) orow[lane + 64] = f32_to_bf16(o1 / ll);
+}
+
+// The same for any number of chunks (contexts beyond 64 chunks): the maxima are found in a pass of
+// their own, and wavefront w adds the chunks c0 + w, c0 + w + 4, ...
+__global__ __launch_bounds__(64 * AD_MERGE_WAVES) void attn_decode_merge_long_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, const int* __restrict__ context_lens,
     bf16_t* __restrict__ out, int out_stride, int max_chunks, int H, int D, int window) {
     __shared__ float s_m[AD_MERGE_WAVES], s_l[AD_MERGE_WAVES], s_o[AD_MERGE_WAVES][128];
@@ -410,8 +502,12 @@ static int launch_decode(const void* q, int q_stride, void* out, int out_stride,
         (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, block_tables, table_width,
         context_lens, part_o, part_ml, max_chunks, H, KVH, page_shift, scale_log2, window);
     TM_CHECK_LAUNCH();
-    attn_decode_merge_kernel<<<dim3(S, H), 64 * AD_MERGE_WAVES, 0, stream>>>(
-        part_o, part_ml, context_lens, (bf16_t*)out, out_stride, max_chunks, H, D, window);
+    if (max_chunks <= TM_WAVE)
+        attn_decode_merge_kernel<<<dim3(S, H), 64 * AD_MERGE_WAVES, 0, stream>>>(
+            part_o, part_ml, context_lens, (bf16_t*)out, out_stride, max_chunks, H, D, window);
+    else
+        attn_decode_merge_long_kernel<<<dim3(S, H), 64 * AD_MERGE_WAVES, 0, stream>>>(
+            part_o, part_ml, context_lens, (bf16_t*)out, out_stride, max_chunks, H, D, window);
     TM_CHECK_LAUNCH();
     return TM_OK;
 }
