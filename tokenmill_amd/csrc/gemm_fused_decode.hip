@@ -137,42 +137,58 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void fused_norm_gem
             gb[j].u = in ? *(const u32x4_t*)(wB + k) : u32x4_t{0, 0, 0, 0};
         }
     };
+    // What the epilogue will need from memory is asked for long before it is used, and in an order
+    // that lets the long loads go first in effect: loads come back in the order they were issued, so
+    // the token's position and cache slot (a few bytes from the cache, and the rotary row's address
+    // hangs on the position) are asked for BEFORE the matrix, and can be waited for while the matrix
+    // is still on its way; the bias and the rotary row follow the matrix and are not looked at (not
+    // even widened) until the epilogue.
+    const int tok = r;                                               // the epilogue's token of this lane
+    const bool epi_lane = wave == 0 && tok < M && 4 * g < ROWS;
+    // The positions are read at addresses that are the same in every lane, which makes them scalar
+    // loads: those are counted apart from the vector loads, so waiting for them does not wait for the
+    // matrix. Each lane then picks its token's.
+    int tok_pos = 0;
+    if constexpr (EPI == FD_EPI_QKV) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int pos_i = a.positions[i < M ? i : 0];
+            tok_pos = tok == i ? pos_i : tok_pos;
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
     // matrix loads of the first group go out before the norm is computed
     FFrag fa[KCH], fb[KCH], fa2[PIPE ? KCH : 1], fb2[PIPE ? KCH : 1];
     load_group(fa, fb, ks0, cu.rows_ok);
     if constexpr (PIPE) load_group(fa2, fb2, ks0 + KCH, cu.rows_ok);
+    __builtin_amdgcn_sched_barrier(0);
 
-    // What the epilogue will need from memory is asked for now, long before it is used: its address
-    // depends on a value that has to be loaded first (the token's position), two trips to memory that
-    // must not stand between the norm and the products.
     struct EpilogueInputs {
-        float bias[2][4];
-        float cos[4], sin[4];
-        int slot;
-    };
-    const int tok = r;                                               // the epilogue's token of this lane
-    const bool epi_lane = wave == 0 && tok < M && 4 * g < ROWS;
+        union {
+            f32x4_t f;              // four rows of a strip as loaded: a 32-bit bias, or
+            uint2 h;                // a bfloat16 one (only the kind there is gets loaded and read)
+        } bias[2];
+        f32x4_t cos, sin;
+        int slot;                   // (every lane loads, the lanes without a token from entry 0; what came is
+    };                              // looked at only where it is meant: a load under a test is waited for where the test ends)
+    const int bias_kind = !a.bias ? 0 : (a.bias_f32 ? 2 : 1);       // the same for every lane
     auto epilogue_inputs = [&](const FusedUnit& t) {
-        EpilogueInputs e = {{{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}, {1.f, 1.f, 1.f, 1.f}, {0.f, 0.f, 0.f, 0.f}, -1};
-        if (EPI == FD_EPI_QKV && epi_lane) {
-            if (a.bias) {
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int ia = t.nA + 4 * g + i, ib = t.nB + 4 * g + i;
-                    e.bias[0][i] = a.bias_f32 ? ((const float*)a.bias)[ia] : bf16_to_f32(((const bf16_t*)a.bias)[ia]);
-                    e.bias[1][i] = a.bias_f32 ? ((const float*)a.bias)[ib] : bf16_to_f32(((const bf16_t*)a.bias)[ib]);
-                }
+        EpilogueInputs e;
+        if constexpr (EPI == FD_EPI_QKV) {
+            const int ia = t.nA + 4 * g, ib = t.nB + 4 * g;         // (the bias is 16-byte aligned)
+            if (bias_kind == 2) {
+                e.bias[0].f = *(const f32x4_t*)((const float*)a.bias + ia);
+                e.bias[1].f = *(const f32x4_t*)((const float*)a.bias + ib);
+            } else if (bias_kind == 1) {
+                e.bias[0].h = *(const uint2*)((const bf16_t*)a.bias + ia);
+                e.bias[1].h = *(const uint2*)((const bf16_t*)a.bias + ib);
             }
-            e.slot = a.slots ? a.slots[tok] : -1;
-            if (t.head < a.H + a.KVH) {
-                const size_t at = (size_t)a.positions[tok] * (a.D / 2) + ROWS * t.jt + 4 * g;
-                const f32x4_t cv = *(const f32x4_t*)(a.cos_t + at), sv = *(const f32x4_t*)(a.sin_t + at);
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    e.cos[i] = cv[i];
-                    e.sin[i] = sv[i];
-                }
-            }
+            // value heads have no rotary row: they read that of the first pair and do not use it
+            const int jt = t.head < a.H + a.KVH ? t.jt : 0;
+            const size_t at = (size_t)tok_pos * (a.D / 2) + ROWS * jt + 4 * g;
+            e.cos = *(const f32x4_t*)(a.cos_t + at);
+            e.sin = *(const f32x4_t*)(a.sin_t + at);
+            e.slot = (a.slots ? a.slots : a.positions)[tok < M ? tok : 0];
         }
         return e;
     };
@@ -364,13 +380,23 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void fused_norm_gem
                     }
                 }
             } else {
+                f32x4_t bA = {0.f, 0.f, 0.f, 0.f}, bB = {0.f, 0.f, 0.f, 0.f};
+                if (bias_kind == 2) {
+                    bA = e.bias[0].f;
+                    bB = e.bias[1].f;
+                } else if (bias_kind == 1) {
+                    bA = f32x4_t{__uint_as_float(e.bias[0].h.x << 16), __uint_as_float(e.bias[0].h.x & 0xffff0000u),
+                                 __uint_as_float(e.bias[0].h.y << 16), __uint_as_float(e.bias[0].h.y & 0xffff0000u)};
+                    bB = f32x4_t{__uint_as_float(e.bias[1].h.x << 16), __uint_as_float(e.bias[1].h.x & 0xffff0000u),
+                                 __uint_as_float(e.bias[1].h.y << 16), __uint_as_float(e.bias[1].h.y & 0xffff0000u)};
+                }
                 float xA[4], xB[4];
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    xA[i] = fd_round(accA[i] + e.bias[0][i]);
-                    xB[i] = fd_round(accB[i] + e.bias[1][i]);
+                    xA[i] = fd_round(accA[i] + bA[i]);
+                    xB[i] = fd_round(accB[i] + bB[i]);
                 }
-                const int slot = e.slot;
+                const int slot = a.slots ? e.slot : -1;
                 if (done.head < a.H + a.KVH) {
                     const int half = a.D / 2;
                     const int j0 = ROWS * done.jt + 4 * g;                       // pair index of element 0
@@ -454,6 +480,7 @@ extern "C" int tm_fused_norm_qkv_rope(const float* resid, const void* norm_w, in
         !q_out || ((uintptr_t)q_out % 8) || page <= 0 || (page & (page - 1)) || !(eps > 0.f))
         return TM_ERR_ARG;
     if (slots && (!k_pool || !v_pool)) return TM_ERR_ARG;
+    if (bias && ((uintptr_t)bias % 16)) return TM_ERR_ARG;          // read four rows at a time
     FusedArgs a{};
     a.resid = resid; a.norm_w = norm_w; a.norm_w_f32 = norm_w_dtype == TM_F32; a.eps = eps; a.M = M; a.K = K;
     a.W = (const bf16_t*)W; a.bias = bias; a.bias_f32 = bias_dtype == TM_F32;

@@ -499,7 +499,8 @@ def fused_norm_qkv_rope(resid: torch.Tensor, norm_w: torch.Tensor, eps: float, w
         _need(page & (page - 1) == 0, "fused qkv: the page size must be a power of two")
         _ints(slots, M, "slots")
     if bias is not None:
-        _need(tuple(bias.shape) == (w.shape[0],) and bias.is_contiguous(), "fused qkv: bias [rows]")
+        _need(tuple(bias.shape) == (w.shape[0],) and bias.is_contiguous() and bias.data_ptr() % 16 == 0,
+              "fused qkv: bias [rows], 16-byte aligned")
     _need(eps > 0, "fused qkv: eps must be positive")
     _check(library().tm_fused_norm_qkv_rope(_p(resid), _p(norm_w), code(norm_w.dtype), c_float(eps), c_int(M), c_int(K),
                                             _p(w), _p(bias), c_int(code(bias.dtype) if bias is not None else -1),

@@ -52,8 +52,10 @@ class GQAttention(Mixer):
         rms = x.fusable_rms()
         tables = getattr(self.position, "fusable_tables", lambda: None)()
         page = cache.k.shape[1]
+        bias = self.qkv.bias
         if (rms is None or tables is None or not gemm.fused_decode_ok(x.resid, self.qkv.weight) or page & (page - 1)
-                or step.max_context_len > self.position.max_positions):
+                or step.max_context_len > self.position.max_positions
+                or (bias is not None and bias.data_ptr() % 16)):
             return None
         q = torch.empty((x.num_tokens, self.q_size), dtype=torch.bfloat16, device=x.resid.device)
         write = cache.write
