@@ -85,9 +85,9 @@ void* flush_buffer(int device) {
     return buf;
 }
 
-// Mean time of a few runs of one algorithm on the caller's own operands, each run after the caches
-// were flushed (the result is the same whichever algorithm wrote it last, up to rounding);
-// negative if it fails.
+// Mean time of a few runs of one algorithm on the caller's own operands (the result is the same
+// whichever algorithm wrote it last, up to rounding); with `flush` each run follows a flush of the
+// caches. Negative if it fails.
 float time_algo(hipblasLtHandle_t handle, const Plan& p, const hipblasLtMatmulAlgo_t& algo, const Operands& op,
                 void* flush) {
     const float one = 1.f, zero = 0.f;
@@ -97,18 +97,28 @@ float time_algo(hipblasLtHandle_t handle, const Plan& p, const hipblasLtMatmulAl
         hipEventDestroy(t0);
         return -1.f;
     }
-    constexpr int WARM = 1, TIMED = 4;
+    constexpr int WARM = 2, TIMED = 5;
     float total = 0.f;
     bool ok = true;
-    for (int i = 0; i < WARM + TIMED && ok; ++i) {
-        if (flush) ok = hipMemsetAsync(flush, i, FLUSH_BYTES, op.stream) == hipSuccess;
-        hipEventRecord(t0, op.stream);
-        ok = ok && hipblasLtMatmul(handle, p.desc, &one, op.W, p.w, op.A, p.a, &zero, op.C, p.c, op.C, p.c, &algo,
-                                   op.workspace, op.workspace_bytes, op.stream) == HIPBLAS_STATUS_SUCCESS;
+    if (!flush) {       // operands in cache: the runs follow each other without a gap, one time for all of them
+        for (int i = 0; i < WARM + TIMED && ok; ++i) {
+            if (i == WARM) hipEventRecord(t0, op.stream);
+            ok = hipblasLtMatmul(handle, p.desc, &one, op.W, p.w, op.A, p.a, &zero, op.C, p.c, op.C, p.c, &algo,
+                                 op.workspace, op.workspace_bytes, op.stream) == HIPBLAS_STATUS_SUCCESS;
+        }
         hipEventRecord(t1, op.stream);
-        float ms = 0.f;
-        ok = ok && hipEventSynchronize(t1) == hipSuccess && hipEventElapsedTime(&ms, t0, t1) == hipSuccess;
-        if (i >= WARM) total += ms;
+        ok = ok && hipEventSynchronize(t1) == hipSuccess && hipEventElapsedTime(&total, t0, t1) == hipSuccess;
+    } else {            // each run after a flush, timed alone
+        for (int i = 0; i < WARM + TIMED && ok; ++i) {
+            ok = hipMemsetAsync(flush, i, FLUSH_BYTES, op.stream) == hipSuccess;
+            hipEventRecord(t0, op.stream);
+            ok = ok && hipblasLtMatmul(handle, p.desc, &one, op.W, p.w, op.A, p.a, &zero, op.C, p.c, op.C, p.c, &algo,
+                                       op.workspace, op.workspace_bytes, op.stream) == HIPBLAS_STATUS_SUCCESS;
+            hipEventRecord(t1, op.stream);
+            float ms = 0.f;
+            ok = ok && hipEventSynchronize(t1) == hipSuccess && hipEventElapsedTime(&ms, t0, t1) == hipSuccess;
+            if (i >= WARM) total += ms;
+        }
     }
     hipEventDestroy(t0);
     hipEventDestroy(t1);
