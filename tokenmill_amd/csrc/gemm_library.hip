@@ -97,7 +97,7 @@ float time_algo(hipblasLtHandle_t handle, const Plan& p, const hipblasLtMatmulAl
         hipEventDestroy(t0);
         return -1.f;
     }
-    constexpr int WARM = 2, TIMED = 5;
+    const int WARM = 2, TIMED = flush ? 5 : 20;
     float total = 0.f;
     bool ok = true;
     if (!flush) {       // operands in cache: the runs follow each other without a gap, one time for all of them
