@@ -175,7 +175,9 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void fused_norm_gem
     auto epilogue_inputs = [&](const FusedUnit& t) {
         EpilogueInputs e;
         if constexpr (EPI == FD_EPI_QKV) {
-            const int ia = t.nA + 4 * g, ib = t.nB + 4 * g;         // (the bias is 16-byte aligned)
+            // lanes beyond the strip's rows (4 g >= ROWS) have no epilogue: they read what group 0 reads
+            const int ge = 4 * g < ROWS ? 4 * g : 0;
+            const int ia = t.nA + ge, ib = t.nB + ge;               // (the bias is 16-byte aligned)
             if (bias_kind == 2) {
                 e.bias[0].f = *(const f32x4_t*)((const float*)a.bias + ia);
                 e.bias[1].f = *(const f32x4_t*)((const float*)a.bias + ib);
@@ -185,7 +187,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void fused_norm_gem
             }
             // value heads have no rotary row: they read that of the first pair and do not use it
             const int jt = t.head < a.H + a.KVH ? t.jt : 0;
-            const size_t at = (size_t)tok_pos * (a.D / 2) + ROWS * jt + 4 * g;
+            const size_t at = (size_t)tok_pos * (a.D / 2) + ROWS * jt + (4 * g < ROWS ? 4 * g : 0);
             e.cos = *(const f32x4_t*)(a.cos_t + at);
             e.sin = *(const f32x4_t*)(a.sin_t + at);
             e.slot = (a.slots ? a.slots : a.positions)[tok < M ? tok : 0];
