@@ -451,7 +451,12 @@ def test_gemm_skinny_with_silu_epilogue(ops, M, I, K):
 @pytest.mark.parametrize("H,KVH,D,page", [(14, 2, 64, 16), (6, 1, 32, 16), (5, 5, 128, 32), (16, 1, 64, 16),
                                            (8, 2, 96, 16), (4, 2, 64, 64)])
 @pytest.mark.parametrize("window", [0, 40])
-def test_paged_attention_decode_mfma(ops, H, KVH, D, page, window):
+@pytest.mark.parametrize("one_block", [False, True])
+def test_paged_attention_decode_mfma(ops, monkeypatch, H, KVH, D, page, window, one_block):
+    """one_block: the kernel for many requests (one block walks a request's whole context), which the
+    dispatcher would only take from 192 (request, kv head) pairs on."""
+    if one_block:
+        monkeypatch.setattr(ops, "DECODE_SPLIT_PAIRS", 0)
     dt = torch.bfloat16
     lens = [1, 2, 16, 17, 255, 256, 257, 700, 64, 1000]
     q_lens = [1] * len(lens)
@@ -486,7 +491,7 @@ def test_paged_attention_decode_mfma(ops, H, KVH, D, page, window):
     # block tables wider than any context (the shape a captured graph has), scratch memory full of NaN
     # beyond what the step writes: up to 64 chunks the merge reads ahead of the context length, beyond
     # that another merge kernel runs
-    for max_context in (4096, 20000):
+    for max_context in () if one_block else (4096, 20000):
         width = -(-max_context // page)
         tables = torch.zeros(S, width, dtype=torch.int32)
         tables[:, :case["tables"].shape[1]] = case["tables"]
