@@ -400,6 +400,68 @@ def test_gemm_skinny(ops, M, N, K):
     assert torch.equal(out_s, out32)
 
 
+@pytest.mark.parametrize("rows", [4, 8, 16])
+@pytest.mark.parametrize("N,K", [(896, 4864), (50, 72), (1153, 40), (16, 32)])
+def test_pack_weight_layout(ops, rows, N, K):
+    """The strip order, element by element from its definition; rows and k that do not exist are zeros."""
+    torch.manual_seed(18)
+    w = torch.randn(N, K).to(torch.bfloat16)
+    pw = ops.pack_weight(w.to(DEV), rows)
+    ks, strips = -(-K // 32), -(-N // rows)
+    data = pw.data.cpu().view(strips, ks, 4, rows, 8)
+    assert (pw.n, pw.k, pw.rows, pw.parts) == (N, K, rows, (N,))
+    idx = torch.randint(0, strips * ks * 4 * rows * 8, (2000,))
+    for flat in idx.tolist() + [0, data.numel() - 1]:
+        i = flat % 8
+        r = (flat // 8) % rows
+        g = (flat // (8 * rows)) % 4
+        k_step = (flat // (32 * rows)) % ks
+        s_ = flat // (32 * rows * ks)
+        n, k = s_ * rows + r, 32 * k_step + 8 * g + i
+        want = w[n, k] if n < N and k < K else torch.tensor(0.0, dtype=torch.bfloat16)
+        assert data.reshape(-1)[flat] == want, (flat, n, k)
+    two = ops.pack_weight(torch.cat([w, w]).to(DEV), rows, [N, N])     # two parts: each starts a strip of its own
+    assert torch.equal(two.data.cpu().view(2, -1)[0], pw.data.cpu()) and torch.equal(two.data.cpu().view(2, -1)[1], pw.data.cpu())
+
+
+@pytest.mark.parametrize("M,N,K", [(8, 896, 4864), (16, 896, 896), (1, 307, 120), (8, 1152, 896), (5, 16 * 2048 + 5, 72),
+                                   (3, 3584, 2056), (16, 50, 4864)])
+def test_gemm_skinny_over_a_packed_matrix_gives_the_same_bits(ops, M, N, K):
+    torch.manual_seed(19)
+    dt = torch.bfloat16
+    a = torch.randn(M, K).to(dt).to(DEV)
+    w = (torch.randn(N, K) * 0.1).to(dt).to(DEV)
+    b = torch.randn(N).to(dt).to(DEV)
+    for rows in (4, 8, 16):
+        pw = ops.pack_weight(w, rows)
+        for out_dt in (dt, torch.float32):
+            plain, packed = torch.empty(M, N, dtype=out_dt, device=DEV), torch.full((M, N), 7.0, dtype=out_dt, device=DEV)
+            ops.gemm_skinny(a, w, b, plain)
+            ops.gemm_skinny(a, pw, b, packed)
+            if rows == ops.skinny_strip_rows(N, K):                      # the same strips, the same split of K: the same bits
+                assert torch.equal(plain, packed)
+            else:
+                torch.testing.assert_close(packed.float(), plain.float(), **tol(dt))
+        resid = torch.randn(M, N, device=DEV) * 5
+        acc_plain, acc_packed = resid.clone(), resid.clone()
+        ops.gemm_skinny(a, w, b, None, accum=acc_plain)
+        ops.gemm_skinny(a, pw, b, None, accum=acc_packed)
+        if rows == ops.skinny_strip_rows(N, K):
+            assert torch.equal(acc_plain, acc_packed)
+        else:
+            torch.testing.assert_close(acc_packed, acc_plain, rtol=1.6e-2, atol=1e-2 + 1e-5)
+    if N % 2 == 0:                                                       # the stacked [gate; up] matrix
+        I = N // 2
+        pw = ops.pack_weight(w, 16, [I, I])
+        plain, packed = torch.empty(M, I, dtype=dt, device=DEV), torch.full((M, I), 7.0, dtype=dt, device=DEV)
+        ops.gemm_skinny(a, w, None, plain, silu=True)
+        ops.gemm_skinny(a, pw, None, packed, silu=True)
+        assert torch.equal(plain, packed)
+    with pytest.raises(ops.KernelArgumentError):                         # more rows than the packed kernels take
+        ops.gemm_skinny(torch.zeros(17, K, dtype=dt, device=DEV), ops.pack_weight(w, 16), None,
+                        torch.empty(17, N, dtype=dt, device=DEV))
+
+
 @pytest.mark.parametrize("tune", [0, 6])
 @pytest.mark.parametrize("M,N,K", [(300, 1152, 896), (17, 896, 4864), (2048, 200, 120), (1, 5000, 64), (70, 307, 72)])
 def test_gemm_library(ops, M, N, K, tune):
@@ -621,7 +683,8 @@ def test_fused_norm_qkv_rope(ops, M, K, H, KVH, D, page):
     vp = torch.full((pages, KVH, D, page), 7.0, dtype=dt, device=DEV)
     q_out = torch.empty(M, H * D, dtype=dt, device=DEV)
     r_dev = resid.to(DEV)
-    ops.fused_norm_qkv_rope(r_dev, nw.to(dt).to(DEV), eps, W.to(dt).to(DEV), b.to(dt).to(DEV), q_out, H, KVH, D,
+    Wp = ops.pack_weight(W.to(dt).to(DEV), ops.fused_qkv_strip_rows(H, KVH, D, K))
+    ops.fused_norm_qkv_rope(r_dev, nw.to(dt).to(DEV), eps, Wp, b.to(dt).to(DEV), q_out, H, KVH, D,
                             half[0].to(DEV), half[1].to(DEV), positions.to(DEV), slots.to(DEV), kp, vp)
     assert torch.equal(r_dev.cpu(), resid)                              # the residual is only read
     torch.testing.assert_close(q_out.float().cpu().view(M, H, D), qq, **tol(dt))
@@ -636,8 +699,12 @@ def test_fused_norm_qkv_rope(ops, M, K, H, KVH, D, page):
     assert (kflat[~written] == 7.0).all() and (vflat[~written] == 7.0).all()
     # a norm weight stored in 32-bit
     nw32 = torch.rand(K) + 0.5
-    ops.fused_norm_qkv_rope(r_dev, nw32.to(DEV), eps, W.to(dt).to(DEV), None, q_out, H, KVH, D, half[0].to(DEV),
+    ops.fused_norm_qkv_rope(r_dev, nw32.to(DEV), eps, Wp, None, q_out, H, KVH, D, half[0].to(DEV),
                             half[1].to(DEV), positions.to(DEV), None, None, None)
+    with pytest.raises(ops.KernelArgumentError):                        # a matrix packed for another kernel
+        wrong = ops.pack_weight(W.to(dt).to(DEV), 4)
+        ops.fused_norm_qkv_rope(r_dev, nw32.to(DEV), eps, wrong, None, q_out, H, KVH, D, half[0].to(DEV),
+                                half[1].to(DEV), positions.to(DEV), None, None, None)
     normed = q(resid * torch.rsqrt((resid * resid).mean(-1, keepdim=True) + eps), dt)
     qkv2 = P.linear(q(nw32 * normed, dt), W, None, dt)
     qq2 = P.apply_rope(qkv2[:, :H * D].view(M, H, D), cos, sin, positions.long(), dt)
@@ -655,7 +722,8 @@ def test_fused_norm_gate_up_silu(ops, M, K, I):
     gu = P.linear(h, W, None, dt)
     want = P.silu_mul(gu[:, :I], gu[:, I:], dt)
     out = torch.empty(M, I, dtype=dt, device=DEV)
-    ops.fused_norm_gate_up_silu(resid.to(DEV), nw.to(dt).to(DEV), eps, W.to(dt).to(DEV), out)
+    Wp = ops.pack_weight(W.to(dt).to(DEV), 16, [I, I])
+    ops.fused_norm_gate_up_silu(resid.to(DEV), nw.to(dt).to(DEV), eps, Wp, out)
     torch.testing.assert_close(out.float().cpu(), want, rtol=2e-2, atol=2e-2)
     assert ((out.float().cpu() - want).abs() > 1e-2).float().mean() < 0.01
 

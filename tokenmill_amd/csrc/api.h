@@ -31,6 +31,17 @@ int tm_attn_paged_generic(const void* q, int q_stride, void* out, int out_stride
 int tm_gemm_skinny(const void* A, int lda, const void* W, const void* bias, int bias_dtype, void* C, int ldc, int M,
                    int N, int K, int out_dtype, int silu, float* accum, int ldacc, hipStream_t stream);
 
+// Strip order of a bfloat16 matrix W [N, K] for the decode-step products ("packed", strips of R = 16, 8 or 4
+// rows): with KS = ceil(K / 32) k-steps, packed[((s * KS + ks) * 4 + g) * R + r][i] = W[s * R + r][32 ks + 8 g + i]
+// for i < 8, zero where the row or the k does not exist; ceil(N / R) strips in all. A wavefront's
+// 16-byte loads of one k-step of one strip are then one run of R * 64 bytes. A stacked matrix whose
+// parts meet in an epilogue (gate and up) is packed part by part, each part's strips behind the other's.
+int tm_skinny_strip_rows(int N, int K);
+int tm_fused_qkv_strip_rows(int H, int KVH, int D, int K);
+int tm_gemm_skinny_packed(const void* A, int lda, const void* W, int rows, const void* bias, int bias_dtype, void* C,
+                          int ldc, int M, int N, int K, int out_dtype, int silu, float* accum, int ldacc,
+                          hipStream_t stream);
+
 int tm_attn_decode_mfma(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
                         const void* v_pool, const int* block_tables, int table_width, const int* context_lens,
                         float* part_o, float* part_ml, int max_chunks, int S, int H, int KVH, int D, int page,

@@ -51,7 +51,8 @@ struct FusedArgs {
     int norm_w_f32;
     float eps;
     int M, K;
-    const bf16_t* W;        // [rows, K]
+    const bf16_t* W;        // the matrix in strip order (see tm_pack_layout in api.h), strips of the kernel's ROWS
+    int up_strip0;          // SiLU epilogue: index of the first strip of the up rows
     const void* bias;       // [rows] or null
     int bias_f32;
     // QKV epilogue
@@ -72,6 +73,7 @@ struct FusedArgs {
 // The two strips of ROWS matrix rows a block multiplies together ("unit" u).
 struct FusedUnit {
     int nA, nB;             // first rows of the strips
+    int sA, sB;             // their indices in the packed matrix
     int head, jt;           // QKV: the head and which slice of it
     bool rows_ok;           // this lane's rows exist
 };
@@ -112,10 +114,13 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void fused_norm_gem
                 t.nA = t.head * a.D + 2 * ROWS * t.jt;
                 t.nB = t.nA + ROWS;
             }
+            t.sA = t.nA / ROWS;                                      // D % 32 == 0: every strip starts on a multiple of ROWS
+            t.sB = t.nB / ROWS;
         } else {                                                     // gate rows and the up rows that meet them
             t.nA = ROWS * u;
             t.nB = a.I + ROWS * u;
-            t.rows_ok = r < ROWS && t.nA + r < a.I;
+            t.sA = u;
+            t.sB = a.up_strip0 + u;                                  // (rows beyond I are zeros in the packed matrix)
         }
         return t;
     };
@@ -126,15 +131,20 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void fused_norm_gem
     const int ks1 = ks0 + per < ksteps ? ks0 + per : ksteps;
     int u = blockIdx.x;
     FusedUnit cu = unit_of(u);
-    const bf16_t* wA = a.W + (size_t)(cu.nA + r) * K + 8 * g;
-    const bf16_t* wB = a.W + (size_t)(cu.nB + r) * K + 8 * g;
+    // The matrix comes in strip order: the 16-byte piece of lane (r, g) for k-step ks of strip s lies at
+    // ((s * ksteps + ks) * 4 + g) * ROWS + r pieces, so a wavefront's load is one run of ROWS * 64 bytes
+    // and a strip is one run of memory; rows and k beyond the matrix are zeros there.
+    constexpr int FRAG = 32 * ROWS;                                  // bfloat16 values of a (strip, k-step)
+    const int lane_off = (g * ROWS + (r < ROWS ? r : 0)) * 8;
+    auto strip_pointer = [&](int strip) { return a.W + (size_t)strip * ksteps * FRAG + lane_off; };
+    const bf16_t* wA = strip_pointer(cu.sA);
+    const bf16_t* wB = strip_pointer(cu.sB);
     auto load_group = [&](auto& ga, auto& gb, int base, bool rows_ok) {
 #pragma unroll
         for (int j = 0; j < KCH; ++j) {
-            const int k = (base + j) * 32;
-            const bool in = rows_ok && base + j < ks1 && k + 8 * g < K;
-            ga[j].u = in ? *(const u32x4_t*)(wA + k) : u32x4_t{0, 0, 0, 0};
-            gb[j].u = in ? *(const u32x4_t*)(wB + k) : u32x4_t{0, 0, 0, 0};
+            const bool in = rows_ok && base + j < ks1;
+            ga[j].u = in ? *(const u32x4_t*)(wA + (size_t)(base + j) * FRAG) : u32x4_t{0, 0, 0, 0};
+            gb[j].u = in ? *(const u32x4_t*)(wB + (size_t)(base + j) * FRAG) : u32x4_t{0, 0, 0, 0};
         }
     };
     // What the epilogue will need from memory is asked for long before it is used, and in an order
@@ -345,8 +355,8 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void fused_norm_gem
         const FusedUnit done = cu;
         if (more) {
             cu = unit_of(un);
-            wA = a.W + (size_t)(cu.nA + r) * K + 8 * g;
-            wB = a.W + (size_t)(cu.nB + r) * K + 8 * g;
+            wA = strip_pointer(cu.sA);
+            wB = strip_pointer(cu.sB);
             load_group(fa, fb, ks0, cu.rows_ok);
             if constexpr (PIPE) load_group(fa2, fb2, ks0 + KCH, cu.rows_ok);
             e_next = epilogue_inputs(cu);
@@ -471,8 +481,18 @@ static bool fused_common_ok(int M, int K, const void* resid, const void* W) {
     return M > 0 && M <= 16 && K > 0 && K % 8 == 0 && ((uintptr_t)resid % 16) == 0 && ((uintptr_t)W % 16) == 0;
 }
 
+// Rows of a strip of the packed q|k|v matrix that tm_fused_norm_qkv_rope reads: strips of 16 rows where
+// they give the chip enough blocks, else of 8; a long K runs one block of 8 wavefronts a CU, and more
+// blocks than CUs would mean a second round for a few of them.
+extern "C" int tm_fused_qkv_strip_rows(int H, int KVH, int D, int K) {
+    const int units16 = (H + 2 * KVH) * (D / 32);
+    const bool one_block_a_cu = K >= 2048;
+    return (units16 >= 256 || (one_block_a_cu && units16 >= 128)) ? 16 : 8;
+}
+
 // q_out[M, H*D], K cache, V cache <- rope(norm(resid) Wqkv^T + b).  Needs M <= 16, D % 32 == 0, a
-// rotary table over the whole head, page a power of two.
+// rotary table over the whole head, page a power of two. W: the [(H + 2 KVH) D, K] matrix packed in
+// strips of tm_fused_qkv_strip_rows(H, KVH, D, K) rows.
 extern "C" int tm_fused_norm_qkv_rope(const float* resid, const void* norm_w, int norm_w_dtype, float eps, int M,
                                       int K, const void* W, const void* bias, int bias_dtype, void* q_out, int H,
                                       int KVH, int D, const float* cos_t, const float* sin_t, const int* positions,
@@ -490,15 +510,13 @@ extern "C" int tm_fused_norm_qkv_rope(const float* resid, const void* norm_w, in
     a.positions = positions; a.slots = slots; a.k_pool = (bf16_t*)k_pool; a.v_pool = (bf16_t*)v_pool;
     a.page_shift = 0;
     while ((1 << a.page_shift) < page) ++a.page_shift;
-    // strips of 16 rows where they give the chip enough blocks, else of 8; a long K runs one block of 8
-    // wavefronts a CU, and more blocks than CUs would mean a second round for a few of them
     const int units16 = (H + 2 * KVH) * (D / 32);
-    const bool one_block_a_cu = K >= 2048;
-    if (units16 >= 256 || (one_block_a_cu && units16 >= 128)) return launch_fused<FD_EPI_QKV, 16>(a, units16, units16, stream);
+    if (tm_fused_qkv_strip_rows(H, KVH, D, K) == 16) return launch_fused<FD_EPI_QKV, 16>(a, units16, units16, stream);
     return launch_fused<FD_EPI_QKV, 8>(a, 2 * units16, 2 * units16, stream);
 }
 
-// act[M, I] <- silu(norm(resid) Wg^T) * (norm(resid) Wu^T), W = [Wg; Wu] [2I, K].  Needs M <= 16.
+// act[M, I] <- silu(norm(resid) Wg^T) * (norm(resid) Wu^T).  Needs M <= 16. W: Wg [I, K] and Wu [I, K]
+// each packed in strips of 16 rows, Wu behind Wg.
 extern "C" int tm_fused_norm_gate_up_silu(const float* resid, const void* norm_w, int norm_w_dtype, float eps, int M,
                                           int K, const void* W, void* act_out, int I, hipStream_t stream) {
     if (M == 0) return TM_OK;
@@ -510,6 +528,7 @@ extern "C" int tm_fused_norm_gate_up_silu(const float* resid, const void* norm_w
     // no more blocks than the chip holds at once (two a CU, one for a long K): beyond that a block takes
     // several units and the norm is computed once for all of them
     const int units = (I + 15) / 16;
+    a.up_strip0 = units;
     const int most = K >= 2048 ? 256 : 512;
     return launch_fused<FD_EPI_SILU, 16>(a, units, units < most ? units : most, stream);
 }

@@ -26,11 +26,14 @@ def _skinny_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
             and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
 
 
-def linear(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, out: torch.Tensor) -> torch.Tensor:
-    """out[M, N] = x[M, K] @ w[N, K]^T (+ bias)."""
+def linear(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, out: torch.Tensor, packed=None) -> torch.Tensor:
+    """out[M, N] = x[M, K] @ w[N, K]^T (+ bias). ``packed``: w in strip order, read instead where it serves."""
     M = x.shape[0]
     if M == 0:
         return out
+    if packed is not None and len(packed.parts) == 1 and out.stride(1) == 1 and _packed_ok(x, packed) \
+            and not (out.dtype == torch.float32 and bias is None and w.shape[0] >= 16384):
+        return ops.gemm_skinny(x, packed, bias, out)
     if x.dtype != torch.bfloat16:
         if ops.gemv_f32_ok(x, w, bias, out):                    # a decode step of the 32-bit path
             return ops.gemv_f32(x, w, bias, out)
@@ -51,25 +54,40 @@ def linear(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, out: tor
     return ops.gemm_nt_tiled(x, w, bias, out)
 
 
-def gate_up_silu(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor) -> bool:
-    """out[M, I] = silu(x Wg^T) * (x Wu^T) in one kernel, if a fused kernel takes this shape."""
+def _packed_ok(x: torch.Tensor, packed) -> bool:
+    K = x.shape[1]
+    stride = x.stride(0) if x.shape[0] > 1 else K
+    return (packed is not None and 0 < x.shape[0] <= ops.PACKED_ROWS and x.dtype == torch.bfloat16 and K == packed.k
+            and K % 8 == 0 and stride % 8 == 0 and x.stride(1) == 1 and x.data_ptr() % 16 == 0)
+
+
+def gate_up_silu(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor, packed=None) -> bool:
+    """out[M, I] = silu(x Wg^T) * (x Wu^T) in one kernel, if a fused kernel takes this shape. ``packed``:
+    the same matrix in strip order, read instead where it serves."""
+    if _packed_ok(x, packed) and packed.rows == 16 and len(packed.parts) == 2:
+        ops.gemm_skinny(x, packed, None, out, silu=True)
+        return True
     if x.shape[0] <= SKINNY_ROWS and _skinny_ok(x, w_gate_up):
         ops.gemm_skinny(x, w_gate_up, None, out, silu=True)
         return True
     return False
 
 
-def linear_accumulate(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, accum: torch.Tensor) -> bool:
+def linear_accumulate(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, accum: torch.Tensor,
+                      packed=None) -> bool:
     """accum[M, N] (float32) += round_bf16(x @ w^T + bias) in the product's epilogue, if a kernel does that
-    for this shape."""
+    for this shape. ``packed``: the same matrix in strip order, read instead where it serves."""
+    if _packed_ok(x, packed) and len(packed.parts) == 1:
+        ops.gemm_skinny(x, packed, bias, None, accum=accum)
+        return True
     if 0 < x.shape[0] <= SKINNY_ROWS and _skinny_ok(x, w):
         ops.gemm_skinny(x, w, bias, None, accum=accum)
         return True
     return False
 
 
-def fused_decode_ok(resid: torch.Tensor, w: torch.Tensor) -> bool:
-    """Can the norm-fused decode products take this residual and matrix?"""
+def fused_decode_ok(resid: torch.Tensor, packed) -> bool:
+    """Can the norm-fused decode products take this residual and (packed) matrix?"""
     M, K = resid.shape
-    return (0 < M <= ops.FUSED_DECODE_ROWS and w.dtype == torch.bfloat16 and K % 8 == 0 and ops.fused_lds_fits(M, K)
-            and resid.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
+    return (packed is not None and 0 < M <= ops.FUSED_DECODE_ROWS and K == packed.k and K % 8 == 0
+            and ops.fused_lds_fits(M, K) and resid.data_ptr() % 16 == 0)

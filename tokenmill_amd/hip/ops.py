@@ -312,12 +312,64 @@ def sample_rows(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Te
     return out
 
 
-def gemm_skinny(a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, out: torch.Tensor | None,
-                silu: bool = False, accum: torch.Tensor | None = None) -> torch.Tensor:
+class PackedWeight:
+    """A bfloat16 matrix [N, K] (or several stacked parts of one K) in the strip order the decode-step
+    products read: ``data[((s * KS + ks) * 4 + g) * rows + r, i] = W[s * rows + r, 32 ks + 8 g + i]`` with
+    KS = ceil(K / 32), zero where the row or the k does not exist, so that a wavefront's load of a k-step
+    of a strip is one run of rows * 64 bytes. Each part of ``parts`` (rows per part) starts a strip of its
+    own: the strips of the second part lie behind those of the first."""
+
+    def __init__(self, data: torch.Tensor, n: int, k: int, rows: int, parts: tuple[int, ...]):
+        self.data, self.n, self.k, self.rows, self.parts = data, n, k, rows, parts
+
+
+def pack_weight(w: torch.Tensor, rows: int, parts: list[int] | None = None) -> PackedWeight:
+    """w bfloat16 [N, K] on the GPU -> its strip order in strips of ``rows`` (16, 8 or 4) rows."""
+    _gpu(w)
+    _need(w.dim() == 2 and w.dtype == torch.bfloat16 and rows in (4, 8, 16), "pack_weight: bfloat16 [N, K], strips of 4, 8 or 16 rows")
+    N, K = w.shape
+    parts = [N] if parts is None else list(parts)
+    _need(sum(parts) == N and all(p > 0 for p in parts), "pack_weight: the parts must add up to the matrix's rows")
+    ks = -(-K // 32)
+    out, row0 = [], 0
+    for n in parts:
+        strips = -(-n // rows)
+        padded = torch.zeros((strips * rows, ks * 32), dtype=w.dtype, device=w.device)
+        padded[:n, :K] = w[row0:row0 + n]
+        # [s, r, ks, g, i] -> [s, ks, g, r, i]
+        out.append(padded.view(strips, rows, ks, 4, 8).permute(0, 2, 3, 1, 4).reshape(-1))
+        row0 += n
+    data = torch.cat(out) if len(out) > 1 else out[0].contiguous()
+    return PackedWeight(data, N, K, rows, tuple(parts))
+
+
+def skinny_strip_rows(N: int, K: int) -> int:
+    """Rows of a strip the skinny product wants an [N, K] matrix packed in."""
+    return int(library().tm_skinny_strip_rows(c_int(N), c_int(K)))
+
+
+def fused_qkv_strip_rows(H: int, KVH: int, D: int, K: int) -> int:
+    """Rows of a strip the norm-fused q|k|v product wants its matrix packed in."""
+    return int(library().tm_fused_qkv_strip_rows(c_int(H), c_int(KVH), c_int(D), c_int(K)))
+
+
+def _packed_operand(w: PackedWeight, rows_expected: int | None, who: str) -> None:
+    _need(isinstance(w, PackedWeight) and w.data.is_cuda and w.data.dtype == torch.bfloat16 and w.data.is_contiguous()
+          and w.data.data_ptr() % 16 == 0, f"{who}: the matrix must be a PackedWeight on the GPU")
+    if rows_expected is not None:
+        _need(w.rows == rows_expected, f"{who}: the matrix is packed in strips of {w.rows} rows, the kernel reads {rows_expected}")
+
+
+def gemm_skinny(a: torch.Tensor, w: "torch.Tensor | PackedWeight", bias: torch.Tensor | None,
+                out: torch.Tensor | None, silu: bool = False, accum: torch.Tensor | None = None) -> torch.Tensor:
     """MFMA product for at most 64 rows of bfloat16 activations: out[M, N] = a @ w^T (+ bias), or with
     ``silu`` out[M, N] = silu(a @ w[:N]^T) * (a @ w[N:]^T) for a stacked [gate; up] matrix w [2N, K].
     out is bfloat16 or float32 (float32 not with silu). With ``accum`` (float32 [M, N]) nothing is
-    stored to out: the result, rounded to bfloat16, is added into accum (the residual stream)."""
+    stored to out: the result, rounded to bfloat16, is added into accum (the residual stream).
+    w may be a ``PackedWeight`` (at most 16 rows of a then; with silu packed as two parts of 16-row
+    strips): the same bits, read faster."""
+    if isinstance(w, PackedWeight):
+        return _gemm_skinny_packed(a, w, bias, out, silu, accum)
     _gpu(a, w, bias, out, accum)
     M, K = a.shape
     if accum is not None:
@@ -356,6 +408,39 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, out
                                     _p(None), c_int(0), _stream()), "gemm_skinny")
     return out
 
+
+def _gemm_skinny_packed(a, w: PackedWeight, bias, out, silu: bool, accum) -> torch.Tensor:
+    _gpu(a, bias, out, accum)
+    _packed_operand(w, 16 if silu else None, "gemm_skinny")
+    M, K = a.shape
+    N = w.n // 2 if silu else w.n
+    _need(a.dtype == torch.bfloat16 and a.dim() == 2 and a.stride(1) == 1 and 0 < M <= PACKED_ROWS and K == w.k,
+          f"gemm_skinny: bfloat16 a [M<={PACKED_ROWS}, {w.k}] for a packed matrix")
+    _need(w.parts == ((N, N) if silu else (w.n,)), "gemm_skinny: with silu the matrix is packed as its two halves, else as one part")
+    lda = a.stride(0) if M > 1 else max(K, a.stride(0))
+    _need(K % 8 == 0 and lda % 8 == 0 and a.data_ptr() % 16 == 0,
+          "gemm_skinny: K and the row stride must be multiples of 8 and the activations 16-byte aligned")
+    if bias is not None:
+        _need(not silu and tuple(bias.shape) == (N,) and bias.is_contiguous(), "gemm_skinny: bias must be [N], not with silu")
+    if accum is not None:
+        _need(out is None and not silu and accum.dtype == torch.float32 and tuple(accum.shape) == (M, N)
+              and accum.stride(1) == 1, "gemm_skinny: accum must be float32 [M, N], and excludes out and silu")
+        ldacc = accum.stride(0) if M > 1 else max(N, accum.stride(0))
+        c, ldc, out_code = None, N, BF16
+    else:
+        _need(out is not None and tuple(out.shape) == (M, N) and out.stride(1) == 1
+              and out.dtype in (torch.bfloat16, torch.float32) and not (silu and out.dtype != torch.bfloat16),
+              "gemm_skinny: out [M, N] bfloat16, or float32 without silu")
+        ldacc = 0
+        c, ldc, out_code = out, (out.stride(0) if M > 1 else max(N, out.stride(0))), code(out.dtype)
+    _check(library().tm_gemm_skinny_packed(_p(a), c_int(lda), _p(w.data), c_int(w.rows), _p(bias),
+                                           c_int(code(bias.dtype) if bias is not None else -1), _p(c), c_int(ldc),
+                                           c_int(M), c_int(N), c_int(K), c_int(out_code), c_int(1 if silu else 0),
+                                           _p(accum), c_int(ldacc), _stream()), "gemm_skinny_packed")
+    return accum if accum is not None else out
+
+
+PACKED_ROWS = 16            # most rows of activations the products over packed matrices take
 
 DECODE_CHUNK = 256          # keys per block of the split decode attention
 DECODE_SPLIT_PAIRS = 192    # below this many (request, kv head) pairs the split kernels (with scratch memory) run
@@ -473,19 +558,21 @@ def attn_prefill_f32(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v
 FUSED_DECODE_ROWS = 16      # most tokens the norm-fused decode products take
 
 
-def fused_norm_qkv_rope(resid: torch.Tensor, norm_w: torch.Tensor, eps: float, w: torch.Tensor,
+def fused_norm_qkv_rope(resid: torch.Tensor, norm_w: torch.Tensor, eps: float, w: PackedWeight,
                         bias: torch.Tensor | None, q_out: torch.Tensor, H: int, KVH: int, D: int, cos: torch.Tensor,
                         sin: torch.Tensor, positions: torch.Tensor, slots: torch.Tensor | None,
                         k_pool: torch.Tensor | None, v_pool: torch.Tensor | None) -> torch.Tensor:
     """q_out[M, H*D] and the cache <- rope(rmsnorm(resid) * norm_w @ w^T + bias) for at most 16 tokens.
-    resid float32 [M, K]; w bfloat16 [(H + 2 KVH) D, K]; cos/sin float32 [max_pos, D/2]."""
-    _gpu(resid, norm_w, w, bias, q_out, cos, sin, positions, slots, k_pool, v_pool)
+    resid float32 [M, K]; w the [(H + 2 KVH) D, K] matrix packed in strips of
+    ``fused_qkv_strip_rows(H, KVH, D, K)`` rows; cos/sin float32 [max_pos, D/2]."""
+    _gpu(resid, norm_w, bias, q_out, cos, sin, positions, slots, k_pool, v_pool)
     M, K = resid.shape
     _need(0 < M <= FUSED_DECODE_ROWS, f"fused qkv: at most {FUSED_DECODE_ROWS} tokens, got {M}")
     _need(resid.dtype == torch.float32 and resid.is_contiguous() and resid.data_ptr() % 16 == 0, "fused qkv: resid float32 [M, K]")
-    _need(w.dtype == torch.bfloat16 and w.is_contiguous() and tuple(w.shape) == ((H + 2 * KVH) * D, K) and K % 8 == 0
-          and w.data_ptr() % 16 == 0, "fused qkv: w must be contiguous bfloat16 [(H+2KVH)D, K], K a multiple of 8")
     _need(D % 32 == 0, f"fused qkv: head size {D} must be a multiple of 32")
+    _packed_operand(w, fused_qkv_strip_rows(H, KVH, D, K), "fused qkv")
+    _need((w.n, w.k) == ((H + 2 * KVH) * D, K) and len(w.parts) == 1 and K % 8 == 0,
+          "fused qkv: w must be the packed [(H+2KVH)D, K] matrix, K a multiple of 8")
     _need(tuple(norm_w.shape) == (K,) and norm_w.is_contiguous() and norm_w.data_ptr() % 16 == 0, "fused qkv: norm weight [K]")
     _need(cos.dtype == torch.float32 and sin.dtype == torch.float32 and cos.is_contiguous() and sin.is_contiguous()
           and cos.shape == sin.shape and cos.dim() == 2 and cos.shape[1] * 2 == D,
@@ -499,11 +586,11 @@ def fused_norm_qkv_rope(resid: torch.Tensor, norm_w: torch.Tensor, eps: float, w
         _need(page & (page - 1) == 0, "fused qkv: the page size must be a power of two")
         _ints(slots, M, "slots")
     if bias is not None:
-        _need(tuple(bias.shape) == (w.shape[0],) and bias.is_contiguous() and bias.data_ptr() % 16 == 0,
+        _need(tuple(bias.shape) == (w.n,) and bias.is_contiguous() and bias.data_ptr() % 16 == 0,
               "fused qkv: bias [rows], 16-byte aligned")
     _need(eps > 0, "fused qkv: eps must be positive")
     _check(library().tm_fused_norm_qkv_rope(_p(resid), _p(norm_w), code(norm_w.dtype), c_float(eps), c_int(M), c_int(K),
-                                            _p(w), _p(bias), c_int(code(bias.dtype) if bias is not None else -1),
+                                            _p(w.data), _p(bias), c_int(code(bias.dtype) if bias is not None else -1),
                                             _p(q_out), c_int(H), c_int(KVH), c_int(D), _p(cos), _p(sin), _p(positions),
                                             _p(slots), _p(k_pool if slots is not None else None),
                                             _p(v_pool if slots is not None else None), c_int(page), _stream()),
@@ -511,21 +598,23 @@ def fused_norm_qkv_rope(resid: torch.Tensor, norm_w: torch.Tensor, eps: float, w
     return q_out
 
 
-def fused_norm_gate_up_silu(resid: torch.Tensor, norm_w: torch.Tensor, eps: float, w: torch.Tensor,
+def fused_norm_gate_up_silu(resid: torch.Tensor, norm_w: torch.Tensor, eps: float, w: PackedWeight,
                             out: torch.Tensor) -> torch.Tensor:
-    """out[M, I] <- silu(x Wg^T) * (x Wu^T), x = rmsnorm(resid) * norm_w, w = [Wg; Wu] bfloat16 [2I, K]."""
-    _gpu(resid, norm_w, w, out)
+    """out[M, I] <- silu(x Wg^T) * (x Wu^T), x = rmsnorm(resid) * norm_w, w = [Wg; Wu] [2I, K] packed as
+    its two halves in strips of 16 rows."""
+    _gpu(resid, norm_w, out)
     M, K = resid.shape
     I = out.shape[1]
     _need(0 < M <= FUSED_DECODE_ROWS, f"fused gate-up: at most {FUSED_DECODE_ROWS} tokens, got {M}")
     _need(resid.dtype == torch.float32 and resid.is_contiguous() and resid.data_ptr() % 16 == 0, "fused gate-up: resid float32 [M, K]")
-    _need(w.dtype == torch.bfloat16 and w.is_contiguous() and tuple(w.shape) == (2 * I, K) and K % 8 == 0 and I % 4 == 0
-          and w.data_ptr() % 16 == 0, "fused gate-up: w must be contiguous bfloat16 [2I, K]; K % 8 == 0, I % 4 == 0")
+    _packed_operand(w, 16, "fused gate-up")
+    _need((w.n, w.k) == (2 * I, K) and w.parts == (I, I) and K % 8 == 0 and I % 4 == 0,
+          "fused gate-up: w must be the packed [2I, K] matrix in two parts of I rows; K % 8 == 0, I % 4 == 0")
     _need(tuple(norm_w.shape) == (K,) and norm_w.is_contiguous() and norm_w.data_ptr() % 16 == 0, "fused gate-up: norm weight [K]")
     _need(out.dtype == torch.bfloat16 and out.is_contiguous() and out.shape[0] == M, "fused gate-up: out bfloat16 [M, I]")
     _need(eps > 0, "fused gate-up: eps must be positive")
     _check(library().tm_fused_norm_gate_up_silu(_p(resid), _p(norm_w), code(norm_w.dtype), c_float(eps), c_int(M),
-                                                c_int(K), _p(w), _p(out), c_int(I), _stream()),
+                                                c_int(K), _p(w.data), _p(out), c_int(I), _stream()),
            "fused_norm_gate_up_silu")
     return out
 

@@ -40,6 +40,9 @@ class GQAttention(Mixer):
         self.qkv.load(tensors, prefix)
         self.o.load(tensors, prefix)
         self.position.load(tensors, prefix)
+        if self.head_dim % 32 == 0:
+            self.qkv.pack(lambda: ops.fused_qkv_strip_rows(self.num_heads, self.num_kv_heads, self.head_dim, self.hidden))
+        self.o.pack(lambda: ops.skinny_strip_rows(self.hidden, self.q_size))
 
     def cache_spec(self):
         return KVCacheSpec(self.num_kv_heads, self.head_dim, self.window)
@@ -53,13 +56,13 @@ class GQAttention(Mixer):
         tables = getattr(self.position, "fusable_tables", lambda: None)()
         page = cache.k.shape[1]
         bias = self.qkv.bias
-        if (rms is None or tables is None or not gemm.fused_decode_ok(x.resid, self.qkv.weight) or page & (page - 1)
+        if (rms is None or tables is None or not gemm.fused_decode_ok(x.resid, self.qkv.packed) or page & (page - 1)
                 or step.max_context_len > self.position.max_positions
                 or (bias is not None and bias.data_ptr() % 16)):
             return None
         q = torch.empty((x.num_tokens, self.q_size), dtype=torch.bfloat16, device=x.resid.device)
         write = cache.write
-        ops.fused_norm_qkv_rope(x.resid, rms[0], rms[1], self.qkv.weight, self.qkv.bias, q, self.num_heads,
+        ops.fused_norm_qkv_rope(x.resid, rms[0], rms[1], self.qkv.packed, self.qkv.bias, q, self.num_heads,
                                 self.num_kv_heads, self.head_dim, tables[0], tables[1], step.positions,
                                 step.groups[cache.group].slot_mapping if write else None,
                                 cache.k if write else None, cache.v if write else None)

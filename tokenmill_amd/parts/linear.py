@@ -24,6 +24,7 @@ class Linear(Part):
         self.has_bias = bias
         self.weight: torch.Tensor | None = None
         self.bias: torch.Tensor | None = None
+        self.packed: ops.PackedWeight | None = None     # the matrix again in the order the decode kernels read
 
     def tensor_specs(self, prefix: str) -> dict[str, TensorSpec]:
         specs = {}
@@ -42,6 +43,15 @@ class Linear(Part):
             if self.weight.dtype == torch.float32 and self.bias.dtype != torch.float32:
                 self.bias = self.bias.float()          # a 32-bit product adds a 32-bit bias
 
+    def pack(self, rows, parts: list[int] | None = None) -> None:
+        """Keep a second copy of a bfloat16 matrix in strip order (``ops.pack_weight``) for the products of
+        decode steps, which read it about 15% faster that way; prompt-sized products keep reading the
+        row-major one. ``rows``: rows of a strip, or a function that gives them (asked only if the matrix
+        is packed). A matrix of another type or not on a GPU is left as it is."""
+        w = self.weight
+        if w is not None and w.dtype == torch.bfloat16 and w.is_cuda:
+            self.packed = ops.pack_weight(w, rows() if callable(rows) else rows, parts)
+
     def use_weight(self, weight: torch.Tensor) -> None:
         """Share another part's matrix (a tied output head)."""
         self.weight = weight
@@ -54,14 +64,15 @@ class Linear(Part):
         w = self.weight
         out_dtype = out_dtype or x.dtype
         from tokenmill_amd.hip import gemm
-        if accumulate_into is not None and w.dtype == x.dtype and gemm.linear_accumulate(x, w, self.bias, accumulate_into):
+        if accumulate_into is not None and w.dtype == x.dtype and \
+                gemm.linear_accumulate(x, w, self.bias, accumulate_into, packed=self.packed):
             return None
         if w.dtype != x.dtype:
             # a matrix the checkpoint stores in 32-bit stays 32-bit: widen the activations for it
             x = ops.convert(x.contiguous(), torch.empty(x.shape, dtype=w.dtype, device=x.device))
         inner_dtype = torch.float32 if x.dtype == torch.float32 else out_dtype
         out = torch.empty((x.shape[0], self.out_features), dtype=inner_dtype, device=x.device)
-        gemm.linear(x, w, self.bias, out)
+        gemm.linear(x, w, self.bias, out, packed=self.packed if x.dtype == w.dtype else None)
         if out.dtype != out_dtype:
             out = ops.convert(out, torch.empty(out.shape, dtype=out_dtype, device=out.device))
         return out

@@ -22,6 +22,8 @@ class SwiGLU(FeedForward):
     def load(self, tensors, prefix: str) -> None:
         self.gate_up.load(tensors, prefix)
         self.down.load(tensors, prefix)
+        self.gate_up.pack(16, [self.intermediate, self.intermediate])
+        self.down.pack(lambda: ops.skinny_strip_rows(self.hidden, self.intermediate))
 
     def forward(self, x, step: StepContext | None = None, residual: torch.Tensor | None = None):
         w = self.gate_up.weight
@@ -29,12 +31,13 @@ class SwiGLU(FeedForward):
         if isinstance(x, NormedInput) and x.dtype == torch.bfloat16 and self.gate_up.bias is None and \
                 self.intermediate % 4 == 0:
             rms = x.fusable_rms()
-            if rms is not None and gemm.fused_decode_ok(x.resid, w):      # the kernel that starts at the norm
+            if rms is not None and gemm.fused_decode_ok(x.resid, self.gate_up.packed):   # the kernel that starts at the norm
                 act = torch.empty((x.num_tokens, self.intermediate), dtype=torch.bfloat16, device=x.resid.device)
-                ops.fused_norm_gate_up_silu(x.resid, rms[0], rms[1], w, act)
+                ops.fused_norm_gate_up_silu(x.resid, rms[0], rms[1], self.gate_up.packed, act)
         if act is None:
             x = as_tensor(x)
             act = torch.empty((x.shape[0], self.intermediate), dtype=x.dtype, device=x.device)
-            if not (w.dtype == x.dtype and self.gate_up.bias is None and gemm.gate_up_silu(x, w, act)):
+            if not (w.dtype == x.dtype and self.gate_up.bias is None
+                    and gemm.gate_up_silu(x, w, act, packed=self.gate_up.packed)):
                 ops.silu_mul(self.gate_up.forward(x), act)
         return self.down.forward(act, accumulate_into=residual)
