@@ -728,6 +728,73 @@ def test_fused_norm_gate_up_silu(ops, M, K, I):
     assert ((out.float().cpu() - want).abs() > 1e-2).float().mean() < 0.01
 
 
+@pytest.mark.parametrize("M,K,H,KVH,D,page", [(64, 896, 14, 2, 64, 16), (17, 192, 6, 1, 32, 16), (40, 1024, 4, 4, 128, 32),
+                                               (33, 120, 3, 1, 96, 64), (5, 896, 14, 2, 64, 16)])
+def test_panel_qkv_rope(ops, M, K, H, KVH, D, page):
+    """q|k|v + bias + rotary + cache write for up to 64 tokens from the normed input kept in LDS."""
+    torch.manual_seed(21)
+    dt = torch.bfloat16
+    theta, max_pos, pages = 1e6, 500, 12
+    rows = (H + 2 * KVH) * D
+    x = q(torch.randn(M, K), dt)
+    W, b = q(torch.randn(rows, K) * 0.05, dt), q(torch.randn(rows) * 0.5, dt)
+    positions = torch.randint(0, max_pos, (M,), dtype=torch.int32)
+    slots = torch.randperm(pages * page)[:M].to(torch.int32)
+    slots[1] = -1
+    qkv = P.linear(x, W, b, dt)
+    cos, sin = P.rope_tables(max_pos, D, theta)
+    qq = P.apply_rope(qkv[:, :H * D].view(M, H, D), cos, sin, positions.long(), dt)
+    kk = P.apply_rope(qkv[:, H * D:(H + KVH) * D].view(M, KVH, D), cos, sin, positions.long(), dt)
+    vv = qkv[:, (H + KVH) * D:].view(M, KVH, D)
+    half = cos[:, :D // 2].contiguous(), sin[:, :D // 2].contiguous()
+    kp = torch.full((pages, page, KVH, D), 7.0, dtype=dt, device=DEV)
+    vp = torch.full((pages, KVH, D, page), 7.0, dtype=dt, device=DEV)
+    q_out = torch.empty(M, H * D, dtype=dt, device=DEV)
+    assert ops.panel_fits(M, K)
+    Wp = ops.pack_weight(W.to(dt).to(DEV), ops.fused_qkv_strip_rows(H, KVH, D, K))
+    wide = torch.zeros(M, K + 16, dtype=dt, device=DEV)                 # a strided input
+    wide[:, :K] = x.to(dt).to(DEV)
+    ops.panel_qkv_rope(wide[:, :K], Wp, b.to(dt).to(DEV), q_out, H, KVH, D, half[0].to(DEV), half[1].to(DEV),
+                       positions.to(DEV), slots.to(DEV), kp, vp)
+    torch.testing.assert_close(q_out.float().cpu().view(M, H, D), qq, **tol(dt))
+    kflat = kp.float().cpu().view(-1, KVH, D)
+    vflat = vp.float().cpu().permute(0, 3, 1, 2).reshape(-1, KVH, D)
+    written = torch.zeros(pages * page, dtype=torch.bool)
+    for t in range(M):
+        if slots[t] >= 0:
+            written[slots[t]] = True
+            torch.testing.assert_close(kflat[slots[t]], kk[t], **tol(dt))
+            torch.testing.assert_close(vflat[slots[t]], vv[t], **tol(dt))
+    assert (kflat[~written] == 7.0).all() and (vflat[~written] == 7.0).all()
+    # a token's result does not depend on the other tokens of the call; no bias, no cache write
+    q_all = torch.empty(M, H * D, dtype=dt, device=DEV)
+    ops.panel_qkv_rope(wide[:, :K], Wp, None, q_all, H, KVH, D, half[0].to(DEV), half[1].to(DEV), positions.to(DEV),
+                       None, None, None)
+    q_one = torch.empty(1, H * D, dtype=dt, device=DEV)
+    ops.panel_qkv_rope(wide[M - 1:, :K], Wp, None, q_one, H, KVH, D, half[0].to(DEV), half[1].to(DEV),
+                       positions[M - 1:].to(DEV), None, None, None)
+    assert torch.equal(q_one[0], q_all[M - 1])
+    assert not ops.panel_fits(65, K) and not ops.panel_fits(M, 1032) and not ops.panel_fits(64, 1024)
+
+
+@pytest.mark.parametrize("M,K,I", [(64, 896, 4864), (17, 64, 128), (48, 192, 320), (33, 120, 200), (9, 1024, 100)])
+def test_panel_gate_up_silu(ops, M, K, I):
+    torch.manual_seed(22)
+    dt = torch.bfloat16
+    x, W = q(torch.randn(M, K), dt), q(torch.randn(2 * I, K) * 0.1, dt)
+    gu = P.linear(x, W, None, dt)
+    want = P.silu_mul(gu[:, :I], gu[:, I:], dt)
+    out = torch.empty(M, I, dtype=dt, device=DEV)
+    Wp = ops.pack_weight(W.to(dt).to(DEV), 16, [I, I])
+    xd = x.to(dt).to(DEV)
+    ops.panel_gate_up_silu(xd, Wp, out)
+    torch.testing.assert_close(out.float().cpu(), want, rtol=2e-2, atol=2e-2)
+    assert ((out.float().cpu() - want).abs() > 1e-2).float().mean() < 0.01      # a rounding flip of gate or up now and then
+    one = torch.empty(1, I, dtype=dt, device=DEV)
+    ops.panel_gate_up_silu(xd[M - 1:], Wp, one)
+    assert torch.equal(one[0], out[M - 1])
+
+
 @pytest.mark.parametrize("M,N,K", [(8, 896, 4864), (1, 64, 128), (40, 200, 120), (64, 896, 896)])
 def test_gemm_skinny_adds_into_the_residual(ops, M, N, K):
     torch.manual_seed(15)

@@ -55,6 +55,12 @@ int tm_fused_norm_qkv_rope(const float* resid, const void* norm_w, int norm_w_dt
 int tm_fused_norm_gate_up_silu(const float* resid, const void* norm_w, int norm_w_dtype, float eps, int M, int K,
                                const void* W, void* act_out, int I, hipStream_t stream);
 
+int tm_gemm_panel_fits(int M, int K);
+int tm_panel_qkv_rope(const void* X, int ldx, int M, int K, const void* W, const void* bias, int bias_dtype, void* q_out,
+                      int H, int KVH, int D, const float* cos_t, const float* sin_t, const int* positions,
+                      const int* slots, void* k_pool, void* v_pool, int page, hipStream_t stream);
+int tm_panel_gate_up_silu(const void* X, int ldx, int M, int K, const void* W, void* act_out, int I, hipStream_t stream);
+
 int tm_attn_prefill_mfma(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
                          const void* v_pool, const int* block_tables, int table_width, const int* tiles, int n_tiles,
                          int H, int KVH, int D, int page, float scale, int window, hipStream_t stream);

@@ -15,68 +15,7 @@
 // paths agree up to the order of 32-bit sums.
 #include "common.h"
 #include "api.h"
-
-typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-typedef float f32x4_t __attribute__((ext_vector_type(4)));
-typedef float f32x2_t __attribute__((ext_vector_type(2)));
-typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
-
-union FFrag {
-    u32x4_t u;
-    bf16x8_t b;
-};
-
-__device__ __forceinline__ uint32_t fd_pack(float a, float b) {
-    const bf16x2_t v = __builtin_convertvector(f32x2_t{a, b}, bf16x2_t);
-    return *(const uint32_t*)&v;
-}
-
-__device__ __forceinline__ float fd_round(float a) { return bf16_to_f32(f32_to_bf16(a)); }
-
-#define FD_EPI_QKV 0
-#define FD_EPI_SILU 1
-#define FD_KCH 8            // k-steps of one register group of matrix loads, per wavefront (one group in all)
-#define FD_KCH_PIPE 6       // the same where two groups take turns
-#define FD_XPAD 8           // padding of an LDS row of x, in elements
-#define FD_RC 8             // 4-element vectors of a residual row a thread keeps in registers
-
-// rows of x a block keeps in LDS for M tokens
-__host__ __device__ __forceinline__ int fused_rows(int M) { return M <= 4 ? 4 : (M <= 8 ? 8 : 16); }
-
-struct FusedArgs {
-    // norm + product
-    const float* resid;     // [M, K]
-    const void* norm_w;     // [K]
-    int norm_w_f32;
-    float eps;
-    int M, K;
-    const bf16_t* W;        // the matrix in strip order (see tm_pack_layout in api.h), strips of the kernel's ROWS
-    int up_strip0;          // SiLU epilogue: index of the first strip of the up rows
-    const void* bias;       // [rows] or null
-    int bias_f32;
-    // QKV epilogue
-    bf16_t* q_out;          // [M, H*D]
-    int H, KVH, D;
-    const float* cos_t;     // [max_pos, D/2]
-    const float* sin_t;
-    const int* positions;   // [M]
-    const int* slots;       // [M]; < 0: not stored
-    bf16_t* k_pool;         // [pages, page, KVH, D]
-    bf16_t* v_pool;         // [pages, KVH, D, page]
-    int page_shift;
-    // SiLU epilogue
-    bf16_t* act_out;        // [M, I]
-    int I;
-};
-
-// The two strips of ROWS matrix rows a block multiplies together ("unit" u).
-struct FusedUnit {
-    int nA, nB;             // first rows of the strips
-    int sA, sB;             // their indices in the packed matrix
-    int head, jt;           // QKV: the head and which slice of it
-    bool rows_ok;           // this lane's rows exist
-};
+#include "fused_common.h"
 
 // ROWS: rows of a strip (16 or 8). Short strips leave rows of the MFMA tile empty (their lanes load
 // nothing) and double the number of units, for matrices that would otherwise give fewer blocks
@@ -98,32 +37,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void fused_norm_gem
     const int wave = threadIdx.x / TM_WAVE, lane = threadIdx.x % TM_WAVE;
     const int r = lane % 16, g = lane / 16;
 
-    auto unit_of = [&](int u) {
-        FusedUnit t;
-        t.head = 0;
-        t.jt = 0;
-        t.rows_ok = r < ROWS;
-        if (EPI == FD_EPI_QKV) {
-            const int per_head = a.D / (2 * ROWS);
-            t.head = u / per_head;
-            t.jt = u % per_head;
-            if (t.head < a.H + a.KVH) {                              // the two halves of ROWS rotary pairs
-                t.nA = t.head * a.D + ROWS * t.jt;
-                t.nB = t.nA + a.D / 2;
-            } else {
-                t.nA = t.head * a.D + 2 * ROWS * t.jt;
-                t.nB = t.nA + ROWS;
-            }
-            t.sA = t.nA / ROWS;                                      // D % 32 == 0: every strip starts on a multiple of ROWS
-            t.sB = t.nB / ROWS;
-        } else {                                                     // gate rows and the up rows that meet them
-            t.nA = ROWS * u;
-            t.nB = a.I + ROWS * u;
-            t.sA = u;
-            t.sB = a.up_strip0 + u;                                  // (rows beyond I are zeros in the packed matrix)
-        }
-        return t;
-    };
+    auto unit_of = [&](int u) { return fused_unit_of<EPI, ROWS>(a, u, r); };
 
     const int ksteps = (K + 31) / 32;
     const int per = (ksteps + WAVES - 1) / WAVES;

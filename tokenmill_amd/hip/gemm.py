@@ -1,12 +1,15 @@
 """Which matrix-product kernel a Linear runs.
 
 float32: the LDS-tiled kernel with 32-bit multiply-adds (a true 32-bit product, fixed summation
-order), or up to 16 rows a matrix-vector kernel of the same kind that streams the matrix once. bfloat16: up to 16 rows (decode steps) the MFMA kernels of this library that stream the
-matrix once and carry the layer's epilogue (bias, rotary + cache write, SiLU·up, residual add) or
-start at the norm; above that the library's matrix product (hipBLASLt, called from this package's
-own library with the plan of every shape kept), as the reference's engine uses a library
-for all of its products (reference src/infer/model/layers.py:144,150,163-164, src/infer/model/qwen2.py:51-52);
-measured on an MI355X the library is the faster one from about 32 rows on, and for the wide output
+order), or up to 16 rows a matrix-vector kernel of the same kind that streams the matrix once.
+bfloat16: up to 16 rows (decode steps) the MFMA kernels of this library that stream the matrix once
+(from its packed copy where the Linear keeps one) and carry the layer's epilogue (bias, rotary +
+cache write, SiLU·up, residual add) or start at the norm; from 17 to 48 rows the q|k|v and gate|up
+products keep the normed input in LDS and carry the same epilogues; everything else goes to the
+library's matrix product (hipBLASLt, called from this package's own library with the plan of every
+shape kept), as the reference's engine uses a library for all of its products (reference
+src/infer/model/layers.py:144,150,163-164, src/infer/model/qwen2.py:51-52); measured on an MI355X
+the library is the faster one from about 32 rows on for a plain product, and for the wide output
 head at any row count. Shapes neither takes run the tiled kernel.
 """
 from __future__ import annotations
@@ -16,6 +19,8 @@ import torch
 from tokenmill_amd.hip import ops
 
 SKINNY_ROWS = 16            # most rows the skinny kernels are preferred for
+PANEL_ROWS = 48             # most rows the products that keep the normed input in LDS are preferred for (they
+                            # take 64; measured, the library and the element-wise kernels are as fast from 56 on)
 SKINNY_MAX_ROWS = 64        # most rows they can take
 
 
@@ -70,7 +75,20 @@ def gate_up_silu(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor, pa
     if x.shape[0] <= SKINNY_ROWS and _skinny_ok(x, w_gate_up):
         ops.gemm_skinny(x, w_gate_up, None, out, silu=True)
         return True
+    if panel_ok(x, packed) and packed.rows == 16 and len(packed.parts) == 2 and out.shape[1] % 4 == 0:
+        ops.panel_gate_up_silu(x, packed, out)
+        return True
     return False
+
+
+def panel_ok(x: torch.Tensor, packed) -> bool:
+    """Can the products that keep the normed input in LDS (17 to 64 tokens) take x and this packed matrix?"""
+    if packed is None or x.dim() != 2:
+        return False
+    M, K = x.shape
+    stride = x.stride(0) if M > 1 else K
+    return (ops.PACKED_ROWS < M <= PANEL_ROWS and x.dtype == torch.bfloat16 and K == packed.k and x.stride(1) == 1
+            and stride % 8 == 0 and x.data_ptr() % 16 == 0 and ops.panel_fits(M, K))
 
 
 def linear_accumulate(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, accum: torch.Tensor,

@@ -619,6 +619,74 @@ def fused_norm_gate_up_silu(resid: torch.Tensor, norm_w: torch.Tensor, eps: floa
     return out
 
 
+PANEL_ROWS = 64             # most tokens the products that keep the normed input in LDS take
+
+
+def panel_fits(M: int, K: int) -> bool:
+    """Do the panel products (q|k|v + rotary + cache write, gate|up + SiLU·up for up to 64 tokens behind a
+    norm that ran by itself) take M tokens of width K?"""
+    return bool(library().tm_gemm_panel_fits(c_int(M), c_int(K)))
+
+
+def _panel_input(x: torch.Tensor, who: str) -> int:
+    M, K = x.shape
+    _need(x.dtype == torch.bfloat16 and x.stride(1) == 1 and x.data_ptr() % 16 == 0 and 0 < M <= PANEL_ROWS
+          and panel_fits(M, K), f"{who}: x bfloat16 [M<={PANEL_ROWS}, K] with x and the partial sums fitting a block's LDS")
+    ldx = x.stride(0) if M > 1 else max(K, x.stride(0))
+    _need(ldx % 8 == 0, f"{who}: rows of x must be 16-byte aligned")
+    return ldx
+
+
+def panel_qkv_rope(x: torch.Tensor, w: PackedWeight, bias: torch.Tensor | None, q_out: torch.Tensor, H: int, KVH: int,
+                   D: int, cos: torch.Tensor, sin: torch.Tensor, positions: torch.Tensor, slots: torch.Tensor | None,
+                   k_pool: torch.Tensor | None, v_pool: torch.Tensor | None) -> torch.Tensor:
+    """q_out[M, H*D] and the cache <- rope(x @ w^T + bias) for up to 64 tokens; x bfloat16 [M, K] is the normed
+    input, everything else as for ``fused_norm_qkv_rope``."""
+    _gpu(x, bias, q_out, cos, sin, positions, slots, k_pool, v_pool)
+    M, K = x.shape
+    ldx = _panel_input(x, "panel qkv")
+    _need(D % 32 == 0, f"panel qkv: head size {D} must be a multiple of 32")
+    _packed_operand(w, fused_qkv_strip_rows(H, KVH, D, K), "panel qkv")
+    _need((w.n, w.k) == ((H + 2 * KVH) * D, K) and len(w.parts) == 1, "panel qkv: w must be the packed [(H+2KVH)D, K] matrix")
+    _need(cos.dtype == torch.float32 and sin.dtype == torch.float32 and cos.is_contiguous() and sin.is_contiguous()
+          and cos.shape == sin.shape and cos.dim() == 2 and cos.shape[1] * 2 == D,
+          "panel qkv: cos/sin must be float32 [max_pos, D/2] (rotation over the whole head)")
+    _need(q_out.dtype == torch.bfloat16 and q_out.is_contiguous() and tuple(q_out.shape) == (M, H * D), "panel qkv: q_out [M, H*D]")
+    _ints(positions, M, "positions")
+    page = 16
+    if slots is not None:
+        _need(k_pool is not None and v_pool is not None, "panel qkv: slots need the cache pools")
+        page = _check_pools(k_pool, v_pool, KVH, D, torch.bfloat16, "panel qkv")
+        _need(page & (page - 1) == 0, "panel qkv: the page size must be a power of two")
+        _ints(slots, M, "slots")
+    if bias is not None:
+        _need(tuple(bias.shape) == (w.n,) and bias.is_contiguous() and bias.data_ptr() % 16 == 0,
+              "panel qkv: bias [rows], 16-byte aligned")
+    _check(library().tm_panel_qkv_rope(_p(x), c_int(ldx), c_int(M), c_int(K), _p(w.data), _p(bias),
+                                       c_int(code(bias.dtype) if bias is not None else -1), _p(q_out), c_int(H),
+                                       c_int(KVH), c_int(D), _p(cos), _p(sin), _p(positions), _p(slots),
+                                       _p(k_pool if slots is not None else None),
+                                       _p(v_pool if slots is not None else None), c_int(page), _stream()),
+           "panel_qkv_rope")
+    return q_out
+
+
+def panel_gate_up_silu(x: torch.Tensor, w: PackedWeight, out: torch.Tensor) -> torch.Tensor:
+    """out[M, I] <- silu(x Wg^T) * (x Wu^T) for up to 64 tokens; x bfloat16 [M, K] is the normed input, w as
+    for ``fused_norm_gate_up_silu``."""
+    _gpu(x, out)
+    M, K = x.shape
+    I = out.shape[1]
+    ldx = _panel_input(x, "panel gate-up")
+    _packed_operand(w, 16, "panel gate-up")
+    _need((w.n, w.k) == (2 * I, K) and w.parts == (I, I) and I % 4 == 0,
+          "panel gate-up: w must be the packed [2I, K] matrix in two parts of I rows; I % 4 == 0")
+    _need(out.dtype == torch.bfloat16 and out.is_contiguous() and out.shape[0] == M, "panel gate-up: out bfloat16 [M, I]")
+    _check(library().tm_panel_gate_up_silu(_p(x), c_int(ldx), c_int(M), c_int(K), _p(w.data), _p(out), c_int(I),
+                                           _stream()), "panel_gate_up_silu")
+    return out
+
+
 def fused_lds_fits(M: int, K: int) -> bool:
     """Does the normed input of M tokens (4, 8 or 16 rows of K + 8 bfloat16), beside the partial sums of
     the block's 4 (K < 2048) or 8 wavefronts, fit the 160 KB of LDS a block of the norm-fused products may use?"""

@@ -68,10 +68,29 @@ class GQAttention(Mixer):
                                 cache.k if write else None, cache.v if write else None)
         return q
 
+    def _panel_qkv(self, x: torch.Tensor, step: StepContext, cache: KVCacheView) -> torch.Tensor | None:
+        """The same for 17 to 64 tokens, from the normed input; None if that kernel does not take this step."""
+        tables = getattr(self.position, "fusable_tables", lambda: None)()
+        page = cache.k.shape[1]
+        bias = self.qkv.bias
+        if (tables is None or self.head_dim % 32 or not gemm.panel_ok(x, self.qkv.packed) or page & (page - 1)
+                or step.max_context_len > self.position.max_positions
+                or (bias is not None and bias.data_ptr() % 16)):
+            return None
+        q = torch.empty((x.shape[0], self.q_size), dtype=torch.bfloat16, device=x.device)
+        write = cache.write
+        ops.panel_qkv_rope(x, self.qkv.packed, bias, q, self.num_heads, self.num_kv_heads, self.head_dim, tables[0],
+                           tables[1], step.positions, step.groups[cache.group].slot_mapping if write else None,
+                           cache.k if write else None, cache.v if write else None)
+        return q
+
     def forward(self, x, step: StepContext, cache: KVCacheView, residual: torch.Tensor | None = None):
         q = self._fused_qkv(x, step, cache)
         if q is None:
-            q = self.qkv.forward(as_tensor(x))                             # [T, (H + 2 KVH) D], q first
+            x = as_tensor(x)
+            q = self._panel_qkv(x, step, cache)
+        if q is None:
+            q = self.qkv.forward(x)                                        # [T, (H + 2 KVH) D], q first
             self.position.encode_and_store(q, self.num_heads, self.num_kv_heads, self.head_dim, step, cache)
         out = torch.empty((q.shape[0], self.q_size), dtype=q.dtype, device=q.device)
         attn_kernels.paged_attention(q, out, cache, step, self.num_heads, self.num_kv_heads, self.head_dim,
