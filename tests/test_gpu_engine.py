@@ -107,6 +107,35 @@ def test_same_tokens_under_every_cutting_and_a_starved_pool(model_dirs, plains, 
         assert outs == base
 
 
+def test_steps_of_17_to_48_tokens_take_the_panel_products(model_dirs, plains, monkeypatch):
+    """24 requests decoding together, and prompt steps of 20 to 40 tokens: the q|k|v and gate|up products
+    that keep the normed input in LDS run (counted), and every token is the plain implementation's."""
+    from tokenmill_amd import SamplingParams
+    from tokenmill_amd.hip import ops
+    calls = {"qkv": 0, "gate_up": 0}
+    real_qkv, real_gu = ops.panel_qkv_rope, ops.panel_gate_up_silu
+
+    def counted_qkv(*a, **k):
+        calls["qkv"] += 1
+        return real_qkv(*a, **k)
+
+    def counted_gu(*a, **k):
+        calls["gate_up"] += 1
+        return real_gu(*a, **k)
+
+    monkeypatch.setattr(ops, "panel_qkv_rope", counted_qkv)
+    monkeypatch.setattr(ops, "panel_gate_up_silu", counted_gu)
+    eng = make_engine(model_dirs["B"], "bfloat16", max_num_batched_tokens=40)
+    prompts = [random_ids(1 + (7 * i) % 19, 384, 300 + i) for i in range(24)]
+    outs = eng.generate(prompts, SamplingParams(max_tokens=10, ignore_eos=True))
+    for p, o in zip(prompts, outs):
+        assert len(o) == 10
+        verify(plains["B"], p, o, torch.bfloat16)
+    layers = 3
+    assert calls["qkv"] >= 9 * layers and calls["gate_up"] == calls["qkv"]       # the decode steps of 24 tokens at least
+    assert eng.cache.num_free_pages == eng.cache.num_pages
+
+
 def test_stop_rules_abort_and_rejections(model_dirs):
     from tokenmill_amd import RequestRejected, SamplingParams
     eng = make_engine(model_dirs["A"], "float32", max_model_len=40)
