@@ -711,7 +711,8 @@ def test_fused_norm_qkv_rope(ops, M, K, H, KVH, D, page):
     torch.testing.assert_close(q_out.float().cpu().view(M, H, D), qq2, **tol(dt))
 
 
-@pytest.mark.parametrize("M,K,I", [(8, 896, 4864), (1, 64, 128), (16, 192, 320), (3, 120, 200)])
+@pytest.mark.parametrize("M,K,I", [(8, 896, 4864), (1, 64, 128), (16, 192, 320), (3, 120, 200),
+                                   (8, 2048, 5000), (5, 256, 8300)])      # the last two: more units than blocks
 def test_fused_norm_gate_up_silu(ops, M, K, I):
     torch.manual_seed(14)
     dt = torch.bfloat16
