@@ -136,6 +136,22 @@ def test_steps_of_17_to_48_tokens_take_the_panel_products(model_dirs, plains, mo
     assert eng.cache.num_free_pages == eng.cache.num_pages
 
 
+def test_without_the_packed_copy_of_the_matrices(model_dirs, plains):
+    """`pack_weights=False` keeps one copy of each matrix: the decode steps then take the kernels that
+    read it row-major, and the tokens are still the plain implementation's."""
+    from tokenmill_amd import SamplingParams
+    eng = make_engine(model_dirs["B"], "bfloat16", pack_weights=False)
+    layer = eng.model.layers[0]
+    assert layer.mixer.qkv.packed is None and layer.ffn.down.packed is None
+    packed = make_engine(model_dirs["B"], "bfloat16")
+    assert packed.model.layers[0].mixer.qkv.packed is not None and packed.model.layers[0].ffn.gate_up.packed.parts == (320, 320)
+    prompts = [random_ids(n, 384, 400 + i) for i, n in enumerate((3, 20, 33))]
+    sp = SamplingParams(max_tokens=12, ignore_eos=True)
+    for e in (eng, packed):
+        for p, o in zip(prompts, e.generate(prompts, sp)):
+            verify(plains["B"], p, o, torch.bfloat16)
+
+
 def test_stop_rules_abort_and_rejections(model_dirs):
     from tokenmill_amd import RequestRejected, SamplingParams
     eng = make_engine(model_dirs["A"], "float32", max_model_len=40)

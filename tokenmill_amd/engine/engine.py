@@ -58,7 +58,8 @@ class LLMEngine:
         if model is None:
             self.device = resolve_device(cfg.device)
             self.dtype = resolve_dtype(cfg.dtype)
-            model = load_model(cfg.model, self.dtype, self.device, max_positions=cfg.max_model_len)
+            model = load_model(cfg.model, self.dtype, self.device, max_positions=cfg.max_model_len,
+                               pack_weights=cfg.pack_weights)
         else:
             self.device, self.dtype = model.device, model.dtype
         self.model = model

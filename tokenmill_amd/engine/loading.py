@@ -25,17 +25,30 @@ def resolve_device(name: str) -> torch.device:
     return torch.device("cuda:0" if name == "auto" else name)
 
 
-def load_model(model_dir: str | Path, dtype: torch.dtype, device: torch.device, max_positions: int | None = None):
-    """The model that config.json names, with its weights on ``device``."""
+def _load(model, tensors, dtype, device, pack_weights: bool) -> None:
+    from tokenmill_amd.parts.linear import Linear
+    before = Linear.keep_packed_copy
+    Linear.keep_packed_copy = pack_weights
+    try:
+        model.load(tensors, dtype, device)
+    finally:
+        Linear.keep_packed_copy = before
+
+
+def load_model(model_dir: str | Path, dtype: torch.dtype, device: torch.device, max_positions: int | None = None,
+               pack_weights: bool = True):
+    """The model that config.json names, with its weights on ``device``. ``pack_weights``: keep a second
+    copy of each layer matrix in the order the decode-step kernels read it."""
     arch, cfg = load_config(model_dir)
     model = arch.build_model(cfg, max_positions)
     tensors = read_checkpoint(model_dir, model.tensor_specs(), dtype, device, model.ignorable)
-    model.load(tensors, dtype, device)
+    _load(model, tensors, dtype, device, pack_weights)
     return model
 
 
 def load_random_model(config: dict, seed: int, dtype: torch.dtype, device: torch.device,
-                      max_positions: int | None = None, std: float = 0.02, norm_std: float = 0.0):
+                      max_positions: int | None = None, std: float = 0.02, norm_std: float = 0.0,
+                      pack_weights: bool = True):
     """The model that ``config`` (config.json contents) names, with random weights drawn on the
     device: the random-weights mode without the trip through a file, for large shapes."""
     from tokenmill_amd.config.registry import architecture_name, get_architecture
@@ -57,5 +70,5 @@ def load_random_model(config: dict, seed: int, dtype: torch.dtype, device: torch
         else:
             t = torch.randn(spec.shape, generator=g, dtype=torch.float32, device=device) * std
         tensors[name] = t if spec.kind == "int" else t.to(storage_dtype(torch.bfloat16, spec.kind, dtype))
-    model.load(tensors, dtype, device)
+    _load(model, tensors, dtype, device, pack_weights)
     return model

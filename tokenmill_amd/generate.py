@@ -61,7 +61,7 @@ def main(argv=None) -> int:
         path = Path(args.random)
         config = json.loads((path / "config.json" if path.is_dir() else path).read_text())
         model = load_random_model(config, args.weights_seed, resolve_dtype(cfg.dtype), resolve_device(cfg.device),
-                                  max_positions=cfg.max_model_len)
+                                  max_positions=cfg.max_model_len, pack_weights=cfg.pack_weights)
     engine = LLMEngine(cfg, model=model)
     if args.prompt_ids is not None:
         prompts = [[int(t) for t in part.split(",") if t.strip()] for part in args.prompt_ids.split(";") if part.strip()]

@@ -14,6 +14,10 @@ from tokenmill_amd.weights.loader import TensorSpec
 
 
 class Linear(Part):
+    # Whether `pack` keeps the second, packed copy. The loaders set it from the engine's options before a
+    # model takes its tensors (twice the layer matrices in memory against faster decode steps).
+    keep_packed_copy = True
+
     def __init__(self, in_features: int, out_features: list[int] | int, names: list[str] | str,
                  bias: bool = False):
         self.in_features = in_features
@@ -49,7 +53,7 @@ class Linear(Part):
         row-major one. ``rows``: rows of a strip, or a function that gives them (asked only if the matrix
         is packed). A matrix of another type or not on a GPU is left as it is."""
         w = self.weight
-        if w is not None and w.dtype == torch.bfloat16 and w.is_cuda:
+        if Linear.keep_packed_copy and w is not None and w.dtype == torch.bfloat16 and w.is_cuda:
             self.packed = ops.pack_weight(w, rows() if callable(rows) else rows, parts)
 
     def use_weight(self, weight: torch.Tensor) -> None:
