@@ -16,7 +16,8 @@
 //                  in ascending chunk order.
 //
 //   Which keys meet in which partial and in which order partials are added depends on positions
-//   only, so what a request gets does not depend on which other requests are in the batch.
+//   only, so within either way what a request gets does not depend on which other requests are in
+//   the batch (which way runs depends on how many there are: the two differ by rounding).
 //
 //   Operand layouts need no LDS: keys K[page][slot][kvh][d] give the A operand of S^T = K Q^T
 //   (16 keys x 32 d per instruction), values V[page][kvh][d][slot] give the A operand of
