@@ -174,7 +174,7 @@ def main() -> int:
                    "tied": bool(shape.get("tie_word_embeddings", False)),
                    "global_batch": args.batch, "seq_len": prompt_len, "context": context,
                    "max_model_len": max_model_len, "block_size": BLOCK_SIZE, "parallelism": "single GPU",
-                   "hip_graphs": not args.no_graphs, "tune_gemm": not args.no_tune},
+                   "hip_graphs": not args.no_graphs, "tune_gemm": not args.no_tune, "packed_weights": True},
         "prefill": {"value": round(prompt_len / prefill_s, 1), "tokens": prompt_len, "ms": round(prefill_s * 1e3, 3),
                     "frac": round(flops / prefill_s / PEAK_FLOPS[args.dtype], 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
