@@ -147,8 +147,10 @@ def test_gemm_tiled(ops, dt, M, N, K):
     assert torch.equal(one[0], out32[M - 1])
 
 
-def paged_case(dt, lens, q_lens, H, KVH, D, page, seed, spike=None):
-    """Random requests laid out in shuffled pages. Returns device operands and the CPU truth."""
+def paged_case(dt, lens, q_lens, H, KVH, D, page, seed, spike=None, ramp=None):
+    """Random requests laid out in shuffled pages. Returns device operands and the CPU truth.
+    ramp: a request whose scores rise steadily with the key's position (about 5 units of log2 per 32
+    keys), so that the running maximum of a flash-style kernel keeps moving."""
     g = torch.Generator().manual_seed(seed)
     S = len(lens)
     n_pages = sum(-(-n // page) for n in lens) + 3
@@ -169,6 +171,9 @@ def paged_case(dt, lens, q_lens, H, KVH, D, page, seed, spike=None):
             k[far, :, 0] = 12.0
             qq[n - 1] *= 0.0
             qq[n - 1, :, 0] = 12.0
+        if ramp is not None and ramp == s:
+            k[:, :, 1] = (torch.arange(n, dtype=torch.float32)[:, None] * (0.15 * (64 / D) ** 0.5)).to(dt)
+            qq[:, :, 1] = 6.0
         for i in range(-(-n // page)):
             tables[s, i] = perm[used]
             lo, hi = i * page, min(n, (i + 1) * page)
@@ -583,7 +588,7 @@ def test_paged_attention_prefill_mfma(ops, H, KVH, D, page, window):
     dt = torch.bfloat16
     lens = [2, 37, 130, 64, 5, 300, 33, 200]
     q_lens = [2, 37, 2, 64, 3, 45, 17, 200]      # whole prompts and portions that start and end mid-page
-    case = paged_case(dt, lens, q_lens, H, KVH, D, page, seed=12, spike=(5, 3) if not window else None)
+    case = paged_case(dt, lens, q_lens, H, KVH, D, page, seed=12, spike=(5, 3) if not window else None, ramp=7)
     if window:
         for s, (n, ql) in enumerate(zip(lens, q_lens)):
             for i in range(max(0, n - ql - window + 1) // page):

@@ -18,6 +18,8 @@
 #include "common.h"
 #include "api.h"
 
+#define PF_SLACK 8.f        // how far (log2 units) a score may exceed the running reference before it moves
+
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
@@ -169,8 +171,15 @@ __device__ __forceinline__ void attend_block(KVBlock<D>& blk, HeadState<D, HPW>&
         float bm = fmaxf(fmaxf(fmaxf(sc[hh][0][0], sc[hh][0][1]), fmaxf(sc[hh][0][2], sc[hh][0][3])),
                          fmaxf(fmaxf(sc[hh][1][0], sc[hh][1][1]), fmaxf(sc[hh][1][2], sc[hh][1][3])));
         bm = column_max(bm) * scale_log2;                        // scale > 0: the maximum commutes with it
-        if (__any(bm > st.m[hh])) {                              // some column's maximum grew: rescale
-            const float m_new = fmaxf(st.m[hh], bm);
+        // The running reference m of a column moves only when the block's maximum exceeds it by more
+        // than PF_SLACK (in units of log2): until then the weights are exp2(s - m) <= 2^PF_SLACK instead of
+        // <= 1, which changes nothing but their common scale (it cancels against the sum), and the
+        // rescaling of the accumulators, the expensive part of a block on the vector unit, becomes rare.
+        // Each column decides for itself and one that stays multiplies by exactly 1, so a query's result
+        // does not depend on the other queries of its tile.
+        const bool grow = bm > st.m[hh] + PF_SLACK;              // (true for a column that has seen no key: m = -inf)
+        if (__any(grow)) {
+            const float m_new = grow ? bm : st.m[hh];
             const float corr = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(st.m[hh] - m_new);
             st.m[hh] = m_new;
             st.l[hh] *= corr;
