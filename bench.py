@@ -2,7 +2,7 @@
 weights, synthetic token ids, on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype bfloat16|float32] [--layers L]
-                    [--config CONFIG.json]     (another shape of the architecture; the default is the 0.5B shape)
+                    [--config CONFIG.json|NAME] (another shape of the architecture; the default is the 0.5B shape)
 
 A "step" is one decode step of the engine (scheduling, metadata upload, the forward pass and greedy
 sampling) with a batch of 8 requests, each holding a 2,048-token prompt. One JSON line is printed.
@@ -18,11 +18,8 @@ from pathlib import Path
 
 sys.path.insert(0, str(Path(__file__).resolve().parent))
 
-# the headline configuration: the Qwen2.5-0.5B shape
-SHAPE = {"architectures": ["Qwen2ForCausalLM"], "num_hidden_layers": 24, "hidden_size": 896,
-         "num_attention_heads": 14, "num_key_value_heads": 2, "intermediate_size": 4864, "vocab_size": 151936,
-         "rope_theta": 1e6, "rms_norm_eps": 1e-6, "tie_word_embeddings": True, "max_position_embeddings": 32768,
-         "use_sliding_window": False}
+# the headline configuration: the shipped Qwen2.5-0.5B shape (tokenmill_amd/config/shapes/qwen2.5-0.5b.json)
+HEADLINE_SHAPE = "qwen2.5-0.5b"
 MAX_MODEL_LEN = 4096
 PROMPT_LEN = 2048
 BLOCK_SIZE = 16
@@ -65,7 +62,7 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (named in config)")
     ap.add_argument("--prompt-len", type=int, default=PROMPT_LEN,
                     help="tokens of every prompt: the prefill's length and the context the decode steps start from")
-    ap.add_argument("--config", default=None, help="a config.json: run its shape instead of the 0.5B shape")
+    ap.add_argument("--config", default=None, help="a config.json or a shipped shape's name (7b, 32b): run it instead of the 0.5B shape")
     ap.add_argument("--no-graphs", action="store_true", help="launch decode steps kernel by kernel")
     ap.add_argument("--no-tune", action="store_true", help="keep the library's first choice of matrix-product algorithm")
     ap.add_argument("--skip-points", action="store_true", help="only the headline batch and the prefill")
@@ -86,9 +83,11 @@ def main() -> int:
     torch.cuda.set_device(0)
     device = torch.device("cuda:0")
     dtype = {"bfloat16": torch.bfloat16, "float32": torch.float32}[args.dtype]
-    shape, shape_name = dict(SHAPE), "Qwen2.5-0.5B shape"
+    from tokenmill_amd.config.shapes import read_shape
+
+    shape, shape_name = read_shape(HEADLINE_SHAPE), "Qwen2.5-0.5B shape"
     if args.config:
-        shape, shape_name = json.loads(Path(args.config).read_text()), Path(args.config).stem
+        shape, shape_name = read_shape(args.config), Path(args.config).stem
     layers_full = shape["num_hidden_layers"]
     if args.layers:
         shape["num_hidden_layers"] = args.layers

@@ -163,3 +163,19 @@ def test_a_tensor_stored_in_32_bit_stays_so_and_integer_tables_become_int32(tmp_
     assert {t[k].dtype for k in "abc"} == {torch.float32} and t["t"].dtype == torch.int32
     with pytest.raises(WeightsError, match="integer"):
         read_checkpoint(tmp_path, dict(specs, a=TensorSpec((4, 4), kind="int")), torch.bfloat16, "cpu")
+
+
+def test_shipped_shapes_read_by_name_alias_or_path(tmp_path):
+    from tokenmill_amd.config.shapes import read_shape, shape_names
+
+    assert {"qwen2.5-0.5b", "qwen2.5-7b", "qwen2.5-32b", "tiny-a", "tiny-b"} <= set(shape_names())
+    for name in shape_names():
+        raw = read_shape(name)
+        cfg = get_architecture(raw["architectures"][0]).config_from_dict(raw, None)
+        assert cfg.num_attention_heads % cfg.num_key_value_heads == 0
+    assert read_shape("7B") == read_shape("qwen2.5-7b")
+    assert read_shape("0.5b")["hidden_size"] == 896 and read_shape("0.5b")["tie_word_embeddings"] is True
+    (tmp_path / "config.json").write_text(json.dumps(qwen2_config(**TINY_B)))
+    assert read_shape(str(tmp_path)) == read_shape(str(tmp_path / "config.json")) == qwen2_config(**TINY_B)
+    with pytest.raises(FileNotFoundError, match="shipped shapes"):
+        read_shape("no-such-shape")

@@ -221,9 +221,9 @@ def test_command_line(model_dirs, plains):
 
 def test_command_line_random_weights(model_dirs):
     """--random CONFIG: weights drawn on the device from --weights-seed; the same seed gives the same tokens,
-    another seed another model."""
-    def run(seed):
-        r = subprocess.run([sys.executable, "-m", "tokenmill_amd.generate", "--random", str(model_dirs["B"]),
+    another seed another model. A shipped shape's name stands for its config.json."""
+    def run(seed, source=None):
+        r = subprocess.run([sys.executable, "-m", "tokenmill_amd.generate", "--random", source or str(model_dirs["B"]),
                             "--weights-seed", str(seed), "--prompt-lens", "9,4", "--max-tokens", "8", "--ignore-eos",
                             "--num-blocks", "16", "--max-model-len", "64", "--block-size", "8"],
                            capture_output=True, text=True, cwd=ROOT, timeout=300)
@@ -233,6 +233,8 @@ def test_command_line_random_weights(model_dirs):
     assert [len(o) for o in first] == [8, 8]
     assert first == again
     assert first != other
+    named = run(3, "tiny-a")
+    assert [len(o) for o in named] == [8, 8] and all(0 <= t < 256 for o in named for t in o)
 
 
 @pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])

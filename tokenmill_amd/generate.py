@@ -6,8 +6,8 @@ engine flags, plus where the prompts come from and how to sample.
     python -m tokenmill_amd.generate --model DIR --prompt-lens 5,17,33 --prompt-seed 0 --temperature 0.8
     python -m tokenmill_amd.generate --random CONFIG.json --weights-seed 1 --prompt-lens 64 --max-tokens 32
 
-``--random`` takes a config.json (or a folder holding one) and draws the weights on the device
-from ``--weights-seed`` instead of reading a checkpoint.
+``--random`` takes a config.json (or a folder holding one) or the name of a shipped shape (0.5b, 7b, 32b,
+tiny-a, tiny-b) and draws the weights on the device from ``--weights-seed`` instead of reading a checkpoint.
 
 Token ids in, token ids out (one JSON line per prompt).
 """
@@ -25,7 +25,8 @@ def main(argv=None) -> int:
     parser = argparse.ArgumentParser(description="tokenmill_amd: continuous-batching generation on one MI355X")
     add_engine_args(parser)
     parser.add_argument("--random", default=None, metavar="CONFIG",
-                        help="a config.json (or its folder): run it with random weights instead of --model")
+                        help="a config.json (or its folder), or the name of a shipped shape (tiny-a, tiny-b, 0.5b, 7b, 32b): "
+                             "run it with random weights instead of --model")
     parser.add_argument("--weights-seed", type=int, default=0, help="seed of the random weights")
     parser.add_argument("--prompt-ids", default=None, help='prompts as token ids: "1,2,3;4,5"')
     parser.add_argument("--prompt-lens", default=None, help="lengths of uniform-random prompts: 5,17,33")
@@ -54,12 +55,10 @@ def main(argv=None) -> int:
     cfg = engine_config_from_args(args)
     model = None
     if args.random:
-        from pathlib import Path
-
+        from tokenmill_amd.config.shapes import read_shape
         from tokenmill_amd.engine.loading import load_random_model, resolve_device, resolve_dtype
 
-        path = Path(args.random)
-        config = json.loads((path / "config.json" if path.is_dir() else path).read_text())
+        config = read_shape(args.random)
         model = load_random_model(config, args.weights_seed, resolve_dtype(cfg.dtype), resolve_device(cfg.device),
                                   max_positions=cfg.max_model_len, pack_weights=cfg.pack_weights)
     engine = LLMEngine(cfg, model=model)

@@ -68,14 +68,17 @@ def write_random_model(config: dict, out_dir, seed: int, std: float = 0.02, norm
 
 def main(argv=None) -> None:
     p = argparse.ArgumentParser(description="write a model folder with random weights")
-    p.add_argument("--config", required=True, help="a config.json of a registered architecture")
+    p.add_argument("--config", required=True,
+                   help="a config.json of a registered architecture, or a shipped shape's name (tiny-a, 0.5b, 7b, ...)")
     p.add_argument("--out", required=True)
     p.add_argument("--seed", type=int, default=0)
     p.add_argument("--std", type=float, default=0.02)
     p.add_argument("--norm-std", type=float, default=0.0, help="norm weights are 1 + N(0, this)")
     p.add_argument("--storage", default="bfloat16", choices=["bfloat16", "float32"])
     a = p.parse_args(argv)
-    write_random_model(json.loads(Path(a.config).read_text()), a.out, a.seed, a.std, a.norm_std, a.storage)
+    from tokenmill_amd.config.shapes import read_shape
+
+    write_random_model(read_shape(a.config), a.out, a.seed, a.std, a.norm_std, a.storage)
     print(f"wrote {a.out}")
 
 
