@@ -467,25 +467,31 @@ def test_gemm_skinny_over_a_packed_matrix_gives_the_same_bits(ops, M, N, K):
                         torch.empty(17, N, dtype=dt, device=DEV))
 
 
-@pytest.mark.parametrize("tune", [0, 6])
+@pytest.mark.parametrize("tune,after", [(0, 3), (6, 1), (6, 3)])
 @pytest.mark.parametrize("M,N,K", [(300, 1152, 896), (17, 896, 4864), (2048, 200, 120), (1, 5000, 64), (70, 307, 72)])
-def test_gemm_library(ops, M, N, K, tune):
+def test_gemm_library(ops, M, N, K, tune, after):
     """The library product behind the cached plan: with and without bias, bfloat16 and float32 out,
-    a strided input, the same bits on the second call (the kept plan), with and without timing the
-    candidates first. A shape the library refuses comes back as False and `linear` takes another kernel."""
+    a strided input, the same bits on the second call (the kept plan); untimed, with the candidates
+    timed at the first call, and timed when the shape comes the third time (every call before and
+    after gives the product). A shape the library refuses comes back as False and `linear` takes
+    another kernel."""
     from tokenmill_amd.hip import gemm
     torch.manual_seed(12)
     dt = torch.bfloat16
     a, w, b = q(torch.randn(M, K), dt), q(torch.randn(N, K) * 0.1, dt), q(torch.randn(N), dt)
     want = a @ w.t()
     da, dw, db = a.to(dt).to(DEV), w.to(dt).to(DEV), b.to(dt).to(DEV)
-    ops.gemm_library_tune(tune)
+    ops.gemm_library_tune(tune, after)
     try:
         out = torch.full((M, N), 7.0, dtype=dt, device=DEV)
         if ops.gemm_library(da, dw, db, out):
             torch.testing.assert_close(out.float().cpu(), q(want + b, dt), **tol(dt))
             again = torch.empty_like(out)
             assert ops.gemm_library(da, dw, db, again) and torch.equal(again, out)
+            for _ in range(after):                          # past the call that times the candidates
+                later = torch.full((M, N), 7.0, dtype=dt, device=DEV)
+                assert ops.gemm_library(da, dw, db, later)
+                torch.testing.assert_close(later.float().cpu(), q(want + b, dt), **tol(dt))
         out32 = torch.full((M, N), 7.0, dtype=torch.float32, device=DEV)
         if ops.gemm_library(da, dw, None, out32):
             torch.testing.assert_close(out32.cpu(), want, rtol=1e-4, atol=1e-4 * K ** 0.5)

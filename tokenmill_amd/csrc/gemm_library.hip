@@ -12,6 +12,8 @@
 // of that result, i.e. per output feature, and is added to the 32-bit sum before rounding.
 #include <hipblaslt/hipblaslt.h>
 
+#include <cstdio>
+#include <cstdlib>
 #include <mutex>
 #include <unordered_map>
 
@@ -43,6 +45,14 @@ struct Plan {
     hipblasLtMatmulAlgo_t algo;
     size_t workspace = 0;
     bool ok = false;
+    int calls = 0;          // eager calls of this shape with the matrix of its first call so far
+    const void* first_w = nullptr;
+    bool timed = false;     // its candidates have been timed (or timing was tried)
+    // The candidates the heuristic gave when the plan was made, kept until they are timed. They are
+    // asked for once: a second, longer query for a product the library has already answered a short
+    // one for gave the same first choice followed by far slower candidates than the one long query.
+    hipblasLtMatmulHeuristicResult_t* found = nullptr;
+    int n_found = 0;
 };
 
 struct Library {
@@ -56,9 +66,13 @@ Library& lib() {
     return *l;
 }
 
-// How many of the heuristic's candidates the first call of a shape times before it keeps the
-// fastest (0 or 1: keep the heuristic's first choice untimed).
+// How many of the heuristic's candidates are timed for a shape before the fastest is kept (0 or 1:
+// keep the heuristic's first choice untimed), and at which call of a shape that happens. Steps of a
+// serving run come in hundreds of different numbers of rows, most of them once: timing costs tens
+// of milliseconds per shape, so only a shape that comes back is timed (or one whose caller says
+// that it will be replayed, by asking for the first call).
 int g_tune_candidates = 0;
+int g_tune_after = 3;
 
 struct Operands {
     const void *A, *W, *bias;
@@ -125,8 +139,25 @@ float time_algo(hipblasLtHandle_t handle, const Plan& p, const hipblasLtMatmulAl
     return ok ? total / TIMED : -1.f;
 }
 
-bool make_plan(hipblasLtHandle_t handle, const PlanKey& k, const Operands& op, Plan& p) {
-    const size_t workspace_bytes = op.workspace_bytes;
+constexpr int MAX_CANDIDATES = 32;
+
+// The library's candidates for a plan's product, best first by its own heuristic.
+int candidates(hipblasLtHandle_t handle, const Plan& p, size_t workspace_bytes, int want,
+               hipblasLtMatmulHeuristicResult_t (&found)[MAX_CANDIDATES]) {
+    hipblasLtMatmulPreference_t pref = nullptr;
+    if (hipblasLtMatmulPreferenceCreate(&pref) != HIPBLAS_STATUS_SUCCESS) return 0;
+    const uint64_t max_ws = workspace_bytes;
+    hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &max_ws, sizeof(max_ws));
+    if (want > MAX_CANDIDATES) want = MAX_CANDIDATES;
+    int n_found = 0;
+    const hipblasStatus_t st =
+        hipblasLtMatmulAlgoGetHeuristic(handle, p.desc, p.w, p.a, p.c, p.c, pref, want, found, &n_found);
+    hipblasLtMatmulPreferenceDestroy(pref);
+    return st == HIPBLAS_STATUS_SUCCESS ? n_found : 0;
+}
+
+// Descriptors, layouts and the heuristic's first valid choice: no run, no wait.
+bool make_plan(hipblasLtHandle_t handle, const PlanKey& k, size_t workspace_bytes, Plan& p) {
     const hipDataType in_t = HIP_R_16BF, out_t = k.out_f32 ? HIP_R_32F : HIP_R_16BF;
     if (hipblasLtMatmulDescCreate(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F) != HIPBLAS_STATUS_SUCCESS) return false;
     const hipblasOperation_t tr = HIPBLAS_OP_T, no = HIPBLAS_OP_N;
@@ -142,69 +173,83 @@ bool make_plan(hipblasLtHandle_t handle, const PlanKey& k, const Operands& op, P
         hipblasLtMatrixLayoutCreate(&p.a, in_t, k.K, k.M, k.lda) != HIPBLAS_STATUS_SUCCESS ||
         hipblasLtMatrixLayoutCreate(&p.c, out_t, k.N, k.M, k.ldc) != HIPBLAS_STATUS_SUCCESS)
         return false;
-    hipblasLtMatmulPreference_t pref = nullptr;
-    if (hipblasLtMatmulPreferenceCreate(&pref) != HIPBLAS_STATUS_SUCCESS) return false;
-    const uint64_t max_ws = workspace_bytes;
-    hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &max_ws, sizeof(max_ws));
-    constexpr int MAX_CANDIDATES = 32;
+    hipblasLtMatmulHeuristicResult_t found[MAX_CANDIDATES];
+    const int n_found = candidates(handle, p, workspace_bytes, g_tune_candidates > 1 ? g_tune_candidates : 1, found);
+    for (int i = 0; i < n_found && !p.ok; ++i)
+        if (found[i].state == HIPBLAS_STATUS_SUCCESS) {
+            p.algo = found[i].algo;
+            p.workspace = found[i].workspaceSize;
+            p.ok = true;
+        }
+    if (p.ok && n_found > 1) {
+        p.found = new hipblasLtMatmulHeuristicResult_t[n_found];
+        for (int i = 0; i < n_found; ++i) p.found[i] = found[i];
+        p.n_found = n_found;
+    }
+    return p.ok;
+}
+
+// Times up to g_tune_candidates of the library's candidates on the caller's own operands and keeps
+// the fastest. Needs the stream to run now: never called while it is being captured into a graph.
+void time_plan(hipblasLtHandle_t handle, const PlanKey& k, const Operands& op, Plan& p) {
     hipblasLtMatmulHeuristicResult_t found[MAX_CANDIDATES];
     int n_found = 0;
-    // timing needs the stream to run now: never while it is being captured into a graph
-    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-    hipStreamIsCapturing(op.stream, &capturing);
-    int want = g_tune_candidates < 1 || capturing != hipStreamCaptureStatusNone ? 1 : g_tune_candidates;
-    if (want > MAX_CANDIDATES) want = MAX_CANDIDATES;
-    const hipblasStatus_t st =
-        hipblasLtMatmulAlgoGetHeuristic(handle, p.desc, p.w, p.a, p.c, p.c, pref, want, found, &n_found);
-    hipblasLtMatmulPreferenceDestroy(pref);
-    if (st != HIPBLAS_STATUS_SUCCESS || n_found < 1) return false;
-    int best = -1;
-    if (want > 1) {
-        if (k.bias_dtype != TM_NONE)
-            hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &op.bias, sizeof(op.bias));
-        // The heuristic's first choice stays unless another candidate beats it clearly (timings of a
-        // few runs scatter by some percent).
-        // Flushed where the matrix is the larger part of what the product reads and writes (few
-        // rows: the matrix comes from HBM in a real step); with many rows the activations, which the
-        // kernel before has just written, are the larger part, and those are in cache in a step too.
-        const size_t out_size = k.out_f32 ? 4 : 2;
-        const bool cold = (size_t)k.N * k.K * 2 > (size_t)k.M * k.K * 2 + (size_t)k.M * k.N * out_size;
-        void* flush = cold ? flush_buffer(k.device) : nullptr;
-        float best_ms = 0.f, first_ms = -1.f;
-        int first = -1;
-        for (int i = 0; i < n_found; ++i) {
-            if (found[i].state != HIPBLAS_STATUS_SUCCESS || found[i].workspaceSize > workspace_bytes) continue;
-            const float ms = time_algo(handle, p, found[i].algo, op, flush);
-            if (ms < 0.f) continue;
-            if (first < 0) {
-                first = i;
-                first_ms = ms;
-            }
-            if (best < 0 || ms < best_ms) {
-                best = i;
-                best_ms = ms;
-            }
+    if (p.found) {
+        n_found = p.n_found < g_tune_candidates ? p.n_found : g_tune_candidates;
+        for (int i = 0; i < n_found; ++i) found[i] = p.found[i];
+        delete[] p.found;
+        p.found = nullptr;
+        p.n_found = 0;
+    } else {                                // the plan was made before timing was switched on
+        n_found = candidates(handle, p, op.workspace_bytes, g_tune_candidates, found);
+    }
+    if (n_found < 2) return;
+    if (k.bias_dtype != TM_NONE)
+        hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &op.bias, sizeof(op.bias));
+    // The heuristic's first choice stays unless another candidate beats it clearly (timings of a
+    // few runs scatter by some percent).
+    // Flushed where the matrix is the larger part of what the product reads and writes (few
+    // rows: the matrix comes from HBM in a real step); with many rows the activations, which the
+    // kernel before has just written, are the larger part, and those are in cache in a step too.
+    const size_t out_size = k.out_f32 ? 4 : 2;
+    const bool cold = (size_t)k.N * k.K * 2 > (size_t)k.M * k.K * 2 + (size_t)k.M * k.N * out_size;
+    void* flush = cold ? flush_buffer(k.device) : nullptr;
+    float best_ms = 0.f, first_ms = -1.f;
+    int best = -1, first = -1;
+    for (int i = 0; i < n_found; ++i) {
+        if (found[i].state != HIPBLAS_STATUS_SUCCESS || found[i].workspaceSize > op.workspace_bytes) continue;
+        const float ms = time_algo(handle, p, found[i].algo, op, flush);
+        if (getenv("TOKENMILL_TUNE_LOG")) fprintf(stderr, " %.4f", ms);
+        if (ms < 0.f) continue;
+        if (first < 0) {
+            first = i;
+            first_ms = ms;
         }
-        if (first >= 0 && best_ms > 0.93f * first_ms) best = first;
+        if (best < 0 || ms < best_ms) {
+            best = i;
+            best_ms = ms;
+        }
     }
-    if (best < 0) {                         // untimed, or nothing could be timed: the heuristic's first valid choice
-        for (int i = 0; i < n_found && best < 0; ++i)
-            if (found[i].state == HIPBLAS_STATUS_SUCCESS) best = i;
-        if (best < 0) return false;
-    }
+    if (first >= 0 && best_ms > 0.93f * first_ms) best = first;
+    if (getenv("TOKENMILL_TUNE_LOG"))
+        fprintf(stderr, "[tokenmill_amd] timed M=%d N=%d K=%d %s: %d candidates, first %.4f ms, best %.4f ms, kept #%d\n",
+                k.M, k.N, k.K, cold ? "cold" : "warm", n_found, first_ms, best_ms, best);
+    if (best < 0) return;                   // nothing could be timed: the plan stays as it is
     p.algo = found[best].algo;
     p.workspace = found[best].workspaceSize;
-    p.ok = true;
-    return true;
 }
 
 }  // namespace
 
-// The first call of every shape from now on times up to n of the library's candidates on that
-// call's operands and keeps the fastest; 0 keeps the library's first choice (the default).
-extern "C" int tm_gemm_library_tune(int n) {
+// From now on a shape's candidates (up to n of them) are timed on its own operands when it is
+// called the `after`-th time with the same matrix outside a graph capture, and the fastest is kept; n = 0 keeps the
+// library's first choice (the default). after = 1 times a shape at its first call: for a caller
+// that is about to capture the step into a graph and replay it.
+extern "C" int tm_gemm_library_tune(int n, int after) {
+    if (n < 0 || n > MAX_CANDIDATES || after < 1) return TM_ERR_ARG;
     std::lock_guard<std::mutex> guard(lib().lock);
-    g_tune_candidates = n < 0 ? 0 : n;
+    g_tune_candidates = n;
+    g_tune_after = after;
     return TM_OK;
 }
 
@@ -236,11 +281,23 @@ extern "C" int tm_gemm_library(const void* A, int lda, const void* W, int ldw, c
         auto it = l.plans.find(key);
         if (it == l.plans.end()) {
             Plan made;
-            const Operands op{A, W, bias, C, workspace, workspace_bytes, stream};
-            make_plan(handle, key, op, made);                        // a failed plan is kept too: asked once
+            make_plan(handle, key, workspace_bytes, made);           // a failed plan is kept too: asked once
             it = l.plans.emplace(key, made).first;
         }
-        plan = it->second;
+        Plan& kept = it->second;
+        if (kept.ok && !kept.timed && g_tune_candidates > 1) {
+            hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+            hipStreamIsCapturing(stream, &capturing);
+            // calls with the matrix of the first call are counted: every layer of a step brings the
+            // shape once with its own matrix, and a step is not a shape that came back
+            if (!kept.first_w) kept.first_w = W;
+            if (capturing == hipStreamCaptureStatusNone && W == kept.first_w && ++kept.calls >= g_tune_after) {
+                kept.timed = true;
+                const Operands op{A, W, bias, C, workspace, workspace_bytes, stream};
+                time_plan(handle, key, op, kept);
+            }
+        }
+        plan = kept;
     }
     if (!plan.ok || plan.workspace > workspace_bytes) return TM_ERR_UNSUPPORTED;
     if (bias_dtype != TM_NONE)          // the descriptor is shared by every call of this shape: calls on one device are serial

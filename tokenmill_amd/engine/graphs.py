@@ -153,7 +153,8 @@ class DecodeGraphs:
         torch.cuda.synchronize()
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):                       # a first run outside the graph: lazy set-up happens here
+        # a first run outside the graph: lazy set-up happens here, and the library's products are timed now
+        with torch.cuda.stream(side), ops.gemm_library_tune_at_once():
             runner.model.forward(step, runner.pools.views)
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
@@ -211,7 +212,8 @@ class PortionGraphs:
             torch.cuda.synchronize()
             side = torch.cuda.Stream()
             side.wait_stream(torch.cuda.current_stream())
-            with torch.cuda.stream(side):                   # a first run outside the graph: lazy set-up happens here
+            # a first run outside the graph: lazy set-up happens here, and the library's products are timed now
+            with torch.cuda.stream(side), ops.gemm_library_tune_at_once():
                 runner.model.forward(step, runner.pools.views)
             torch.cuda.current_stream().wait_stream(side)
             torch.cuda.synchronize()

@@ -7,6 +7,7 @@ BEFORE anything is launched; a kernel never sees a size it was not written for. 
 """
 from __future__ import annotations
 
+import contextlib
 import ctypes
 from ctypes import c_float, c_int, c_longlong, c_void_p
 
@@ -189,11 +190,32 @@ def library_workspace(device: torch.device) -> torch.Tensor:
     return ws
 
 
-def gemm_library_tune(candidates: int) -> None:
-    """From now on the first call of every new shape times up to ``candidates`` of the library's
-    algorithms on its own operands and keeps the fastest (0: the library's first choice, untimed)."""
-    _need(0 <= candidates <= 32, "gemm_library_tune: 0 to 32 candidates")
-    _check(library().tm_gemm_library_tune(c_int(candidates)), "gemm_library_tune")
+TUNE_AFTER_CALLS = 3        # a shape's candidates are timed when it is called this often (most shapes of a serving run come once)
+_tune = {"candidates": 0, "after": TUNE_AFTER_CALLS}
+
+
+def gemm_library_tune(candidates: int, after: int = TUNE_AFTER_CALLS) -> None:
+    """From now on a shape that is called the ``after``-th time with the same matrix (outside a graph capture) has up to
+    ``candidates`` of the library's algorithms timed on its own operands, and the fastest is kept
+    (0: the library's first choice, untimed)."""
+    _need(0 <= candidates <= 32 and after >= 1, "gemm_library_tune: 0 to 32 candidates, after >= 1 calls")
+    _check(library().tm_gemm_library_tune(c_int(candidates), c_int(after)), "gemm_library_tune")
+    _tune["candidates"], _tune["after"] = candidates, after
+
+
+@contextlib.contextmanager
+def gemm_library_tune_at_once():
+    """Inside, a shape is timed at its first call (if timing is on at all): for the run before a
+    graph capture, whose shapes are about to be replayed many times."""
+    candidates, after = _tune["candidates"], _tune["after"]
+    if candidates < 2:
+        yield
+        return
+    gemm_library_tune(candidates, 1)
+    try:
+        yield
+    finally:
+        gemm_library_tune(candidates, after)
 
 
 def gemm_library(a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, out: torch.Tensor) -> bool:
