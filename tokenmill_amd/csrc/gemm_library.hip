@@ -71,6 +71,7 @@ Library& lib() {
 // serving run come in hundreds of different numbers of rows, most of them once: timing costs tens
 // of milliseconds per shape, so only a shape that comes back is timed (or one whose caller says
 // that it will be replayed, by asking for the first call).
+// With TOKENMILL_TUNE_LOG set in the environment every timing is printed to stderr.
 int g_tune_candidates = 0;
 int g_tune_after = 3;
 
