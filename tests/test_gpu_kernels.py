@@ -508,6 +508,23 @@ def test_gemm_library(ops, M, N, K, tune, after):
         ops.gemm_library_tune(0)
 
 
+def test_gemm_library_takes_a_candidate_whose_workspace_fits(ops):
+    """At 8,192 rows of the gate|up product the library's first choice asks for more workspace than it is
+    given: the plan takes the first candidate that fits instead of refusing the shape (a refused shape
+    runs 64 rows at a time through the skinny kernel, ten times slower)."""
+    torch.manual_seed(13)
+    dt = torch.bfloat16
+    M, N, K = 8192, 9728, 896
+    da = torch.randn(M, K, device=DEV).to(dt)
+    dw = (torch.randn(N, K, device=DEV) * 0.1).to(dt)
+    out = torch.full((M, N), 7.0, dtype=dt, device=DEV)
+    ops.gemm_library_tune(0)
+    assert ops.gemm_library(da, dw, None, out)
+    rows = torch.arange(0, M, 257)
+    want = da[rows].float().cpu() @ dw.float().cpu().t()
+    torch.testing.assert_close(out[rows].float().cpu(), q(want, dt), **tol(dt))
+
+
 @pytest.mark.parametrize("M,I,K", [(1, 128, 64), (8, 4864, 896), (40, 200, 120), (64, 320, 192)])
 def test_gemm_skinny_with_silu_epilogue(ops, M, I, K):
     torch.manual_seed(10)

@@ -93,14 +93,20 @@ __device__ __forceinline__ void load_kv_block(KVBlock<D>& blk, int2 pages, int s
     }
 }
 
+// max(a, b, c) in the nesting the compiler turns into one three-operand maximum. A two-operand
+// maximum of values whose origin it cannot see (matrix-unit results, lane swaps) costs it an extra
+// instruction per operand (it first makes signalling NaNs quiet); the three-operand form does not,
+// so the reductions below are chains of these, started from a constant.
+__device__ __forceinline__ float max3(float a, float b, float c) { return fmaxf(fmaxf(a, b), c); }
+
 // maximum over the four lanes (r, 0..3) that hold one query column
 __device__ __forceinline__ float column_max(float v) {
     const uint32_t u = __float_as_uint(v);
     const auto a = __builtin_amdgcn_permlane32_swap(u, u, false, false);     // lanes l and l ^ 32
-    const float m32 = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+    const float m32 = max3(-INFINITY, __uint_as_float(a[0]), __uint_as_float(a[1]));
     const uint32_t w = __float_as_uint(m32);
     const auto b = __builtin_amdgcn_permlane16_swap(w, w, false, false);     // lanes l and l ^ 16
-    return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+    return max3(-INFINITY, __uint_as_float(b[0]), __uint_as_float(b[1]));
 }
 
 // Running softmax state of the query heads a wavefront works on.
@@ -168,8 +174,10 @@ __device__ __forceinline__ void attend_block(KVBlock<D>& blk, HeadState<D, HPW>&
                     if (kj > tv.my_pos || kj < tv.my_lo) sc[hh][t][i] = -INFINITY;
                 }
         }
-        float bm = fmaxf(fmaxf(fmaxf(sc[hh][0][0], sc[hh][0][1]), fmaxf(sc[hh][0][2], sc[hh][0][3])),
-                         fmaxf(fmaxf(sc[hh][1][0], sc[hh][1][1]), fmaxf(sc[hh][1][2], sc[hh][1][3])));
+        float bm = max3(-INFINITY, sc[hh][0][0], sc[hh][0][1]);
+        bm = max3(bm, sc[hh][0][2], sc[hh][0][3]);
+        bm = max3(bm, sc[hh][1][0], sc[hh][1][1]);
+        bm = max3(bm, sc[hh][1][2], sc[hh][1][3]);
         bm = column_max(bm) * scale_log2;                        // scale > 0: the maximum commutes with it
         // The running reference m of a column moves only when the block's maximum exceeds it by more
         // than PF_SLACK (in units of log2): until then the weights are exp2(s - m) <= 2^PF_SLACK instead of

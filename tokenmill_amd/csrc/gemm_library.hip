@@ -174,15 +174,20 @@ bool make_plan(hipblasLtHandle_t handle, const PlanKey& k, size_t workspace_byte
         hipblasLtMatrixLayoutCreate(&p.a, in_t, k.K, k.M, k.lda) != HIPBLAS_STATUS_SUCCESS ||
         hipblasLtMatrixLayoutCreate(&p.c, out_t, k.N, k.M, k.ldc) != HIPBLAS_STATUS_SUCCESS)
         return false;
+    // Several candidates also when none will be timed: the heuristic's first choice can ask for more
+    // workspace than the preference allows (a split of K with one partial result per split, seen at
+    // 8,192 and 16,384 rows), and the first that fits is taken.
+    constexpr int UNTIMED_CANDIDATES = 8;
     hipblasLtMatmulHeuristicResult_t found[MAX_CANDIDATES];
-    const int n_found = candidates(handle, p, workspace_bytes, g_tune_candidates > 1 ? g_tune_candidates : 1, found);
+    const int n_found = candidates(handle, p, workspace_bytes,
+                                   g_tune_candidates > UNTIMED_CANDIDATES ? g_tune_candidates : UNTIMED_CANDIDATES, found);
     for (int i = 0; i < n_found && !p.ok; ++i)
-        if (found[i].state == HIPBLAS_STATUS_SUCCESS) {
+        if (found[i].state == HIPBLAS_STATUS_SUCCESS && found[i].workspaceSize <= workspace_bytes) {
             p.algo = found[i].algo;
             p.workspace = found[i].workspaceSize;
             p.ok = true;
         }
-    if (p.ok && n_found > 1) {
+    if (p.ok && n_found > 1 && g_tune_candidates > 1) {
         p.found = new hipblasLtMatmulHeuristicResult_t[n_found];
         for (int i = 0; i < n_found; ++i) p.found[i] = found[i];
         p.n_found = n_found;
