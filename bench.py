@@ -2,6 +2,7 @@
 weights, synthetic token ids, on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype bfloat16|float32] [--layers L]
+                    [--part offline [--requests 300 --offline-prompt 512 --offline-gen 128 --chunked]]
                     [--config CONFIG.json|NAME] (another shape of the architecture; the default is the 0.5B shape)
 
 A "step" is one decode step of the engine (scheduling, metadata upload, the forward pass and greedy
@@ -66,8 +67,14 @@ def main() -> int:
     ap.add_argument("--no-graphs", action="store_true", help="launch decode steps kernel by kernel")
     ap.add_argument("--no-tune", action="store_true", help="keep the library's first choice of matrix-product algorithm")
     ap.add_argument("--skip-points", action="store_true", help="only the headline batch and the prefill")
-    ap.add_argument("--part", default="all", choices=["all", "decode", "prefill"],
-                    help="run only the decode steps or only the prefill (for profiling one of them)")
+    ap.add_argument("--part", default="all", choices=["all", "decode", "prefill", "offline"],
+                    help="run only the decode steps or only the prefill (for profiling one of them), or an offline "
+                         "run: --requests prompts of --offline-prompt tokens submitted at once, --offline-gen tokens each")
+    ap.add_argument("--requests", type=int, default=300)
+    ap.add_argument("--offline-prompt", type=int, default=512)
+    ap.add_argument("--offline-gen", type=int, default=128)
+    ap.add_argument("--offline-seqs", type=int, default=128, help="requests running at a time in the offline run")
+    ap.add_argument("--chunked", action="store_true", help="offline run: portions of prompts beside decoding requests")
     args = ap.parse_args()
     prompt_len = args.prompt_len
     max_model_len = max(MAX_MODEL_LEN, prompt_len + args.steps + args.warmup + 128)
@@ -141,6 +148,36 @@ def main() -> int:
             assert outs and outs[0].finished
         return statistics.median(times[1:])              # the first run warms up
 
+    def time_offline():
+        """All requests at once, as the reference's offline runs do (reference bench/results/results.md:11-18:
+        300 requests of 512 prompt and 128 generated tokens); a short run first warms up and captures graphs."""
+        per_seq = -(-(args.offline_prompt + args.offline_gen + 1) // BLOCK_SIZE)
+        cfg = EngineConfig(dtype=args.dtype, block_size=BLOCK_SIZE, num_blocks=args.offline_seqs * per_seq + 64,
+                           max_model_len=max_model_len, max_num_seqs=args.offline_seqs, max_num_batched_tokens=2048,
+                           enable_chunked_prefill=args.chunked, hip_graphs=not args.no_graphs,
+                           tune_gemm=not args.no_tune)
+        eng = LLMEngine(cfg, model=model)
+        sp = SamplingParams(max_tokens=args.offline_gen, ignore_eos=True)
+
+        def run(n):
+            reqs = [torch.randint(0, shape["vocab_size"], (args.offline_prompt,), generator=gen).tolist() for _ in range(n)]
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            outs = eng.generate(reqs, sp)
+            torch.cuda.synchronize()
+            assert all(len(o) == args.offline_gen for o in outs)
+            return time.perf_counter() - t0
+        run(min(args.requests, 2 * args.offline_seqs))
+        return run(args.requests)
+
+    if args.part == "offline":
+        t = time_offline()
+        gen_tokens = args.requests * args.offline_gen
+        print(json.dumps({"offline": {"requests": args.requests, "prompt": args.offline_prompt, "gen": args.offline_gen,
+                                      "running": args.offline_seqs, "chunked": args.chunked, "s": round(t, 3),
+                                      "gen_tok_s": round(gen_tokens / t, 1),
+                                      "tok_s": round((gen_tokens + args.requests * args.offline_prompt) / t, 1)}}))
+        return 0
     if args.part == "prefill":
         prefill_s = time_prefill()
         print(json.dumps({"prefill": {"value": round(prompt_len / prefill_s, 1), "tokens": prompt_len,
