@@ -19,7 +19,6 @@ fixed size, taken with its first pages and returned with them.
 from __future__ import annotations
 
 import enum
-import math
 from dataclasses import dataclass, field
 
 from tokenmill_amd.cache.allocator import OutOfPages, PageAllocator, SlotAllocator
@@ -53,6 +52,7 @@ class CacheManager:
             raise ValueError("page_size must be at least 1")
         self.page_size = page_size
         self.windows = list(group_windows)
+        self.any_window = any(w is not None for w in self.windows)
         counts = [num_pages] * len(self.windows) if isinstance(num_pages, int) else list(num_pages)
         if len(counts) != len(self.windows):
             raise ValueError("one page count per group")
@@ -68,7 +68,7 @@ class CacheManager:
         return len(self.allocators)
 
     def pages_for(self, num_tokens: int) -> int:
-        return math.ceil(num_tokens / self.page_size)
+        return -(-num_tokens // self.page_size)
 
     @property
     def num_free_pages(self) -> int:
@@ -119,18 +119,32 @@ class CacheManager:
 
     def append(self, rc: RequestCache, length: int) -> None:
         """Grow every table to hold ``length`` tokens; all or nothing."""
-        need = self.pages_for(length)
-        if not self.can_append(rc, length):
+        if not self.try_append(rc, length):
             raise OutOfPages(f"{rc.request_id}: cannot grow to {length} tokens")
-        for t, a in zip(rc.tables, self.allocators):
+
+    def try_append(self, rc: RequestCache, length: int) -> bool:
+        """``append`` if there is room, all or nothing; False (nothing changed) if there is not."""
+        need = -(-length // self.page_size)
+        tables, allocators = rc.tables, self.allocators
+        short = False
+        for t, a in zip(tables, allocators):
             if len(t) < need:
-                t.extend(a.allocate(need - len(t)))
+                if a.num_free < need - len(t):
+                    return False
+                short = True
+        if short:
+            for t, a in zip(tables, allocators):
+                if len(t) < need:
+                    t.extend(a.allocate(need - len(t)))
+        return True
 
     def release_behind_window(self, rc: RequestCache, num_computed: int) -> int:
         """Give back, in windowed groups, the pages that no later token can see: with
         ``num_computed`` tokens cached, the next query sits at position >= num_computed and sees
         keys from num_computed - W + 1 on. Returns the number of pages given back."""
         given = 0
+        if not self.any_window:
+            return given
         for g, window in enumerate(self.windows):
             if window is None:
                 continue

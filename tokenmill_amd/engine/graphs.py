@@ -100,8 +100,8 @@ class DecodeGraphs:
         n = len(entries)
         ids = np.zeros(B, dtype=np.int64)
         pos = np.zeros(B, dtype=np.int64)
-        for i, e in enumerate(entries):
-            ids[i], pos[i] = e.tokens[0], e.start
+        ids[:n] = [e.tokens[0] for e in entries]
+        pos[:n] = [e.start for e in entries]
         if ids.min() < 0 or ids.max() >= runner.vocab:
             raise ValueError("a token id is outside the vocabulary")
         if pos.max() >= self.max_positions:
@@ -113,14 +113,14 @@ class DecodeGraphs:
         host[bk.ctx[0]:bk.ctx[1]] = ctx
         state = host[bk.state[0]:bk.state[1]]
         state[:] = 0
-        for i, e in enumerate(entries):
-            state[i] = e.cache.state_slot
+        state[:n] = [e.cache.state_slot for e in entries]
         for g in range(len(runner.pools.groups)):
             slots = host[bk.g_slot[g][0]:bk.g_slot[g][1]]
             tabs = host[bk.g_tab[g][0]:bk.g_tab[g][1]].reshape(B, W)
             slots[:] = -1
             windowed = runner.pools.groups[g].window is not None
             rows = bk.rows_held[g]
+            new_slots = []
             for i, e in enumerate(entries):
                 table = e.cache.tables[g]
                 need = e.start // page + 1
@@ -133,7 +133,8 @@ class DecodeGraphs:
                     row = np.asarray(table[have:need], dtype=np.int64)
                     tabs[i, have:need] = np.where(row == RELEASED, 0, row)
                 rows[i] = (e.cache, need)
-                slots[i] = table[need - 1] * page + e.start % page
+                new_slots.append(table[need - 1] * page + e.start % page)
+            slots[:n] = new_slots
             for i in range(n, B):
                 rows[i] = None
         bk.dev.copy_(bk.pinned, non_blocking=True)

@@ -160,19 +160,22 @@ class Scheduler:
         ``partial`` (chunked mode) requests still inside their prompt are set aside into it instead
         of decoding; until they are visited they can be preempted like any other."""
         queue = sorted(candidates, key=lambda s: s.admit_order)
-        while queue:
-            seq = queue.pop(0)
+        try_append, decode_seqs = self.cache.try_append, out.decode_seqs
+        i = 0                                               # queue[i:] are the requests not yet visited
+        while i < len(queue):
+            seq = queue[i]
+            i += 1
             if partial is not None and seq.num_new_tokens > 1:
                 partial.append(seq)
                 continue
-            while not self.cache.can_append(seq.cache, seq.length):
-                victim = queue.pop() if queue else seq
+            length = seq.length
+            while not try_append(seq.cache, length):
+                victim = queue.pop() if i < len(queue) else seq
                 self._preempt(victim, out)
                 if victim is seq:
                     break
             else:
-                self.cache.append(seq.cache, seq.length)
-                out.decode_seqs.append(seq)
+                decode_seqs.append(seq)
 
     def _schedule_chunked(self, out: SchedulerOutput) -> None:
         budget = self.cfg.max_num_batched_tokens
