@@ -355,6 +355,63 @@ def test_sample_rows_against_the_plain_sampler(ops):
     assert sum(g == w for g, w in zip(got, want)) >= 62
 
 
+def test_sample_rows_wide_vocabulary_against_the_plain_sampler(ops):
+    """A vocabulary of several chunks (no power of two, a short last chunk): every stage of the
+    sampler works over (row, chunk) blocks. Rows with and without each filter in one call, and the same
+    rows alone or with the filters' launches left out give the same tokens."""
+    torch.manual_seed(18)
+    V = 4 * 4096 + 3731
+    R = 40
+    logits = torch.randn(R, V) * 2.5
+    logits[5, 17000:17040] += 6.0                                     # a nucleus inside the last chunks
+    cases = [(0.8, -1, 1.0), (1.0, 20, 1.0), (0.7, -1, 0.9), (1.3, 50, 0.8), (0.0, -1, 1.0), (0.9, 1, 1.0),
+             (1.0, V + 5, 0.999), (0.5, 3, 0.5), (1.5, 3000, 1.0), (2.0, -1, 0.97)]
+    temps, ks, ps, us, want, margins = [], [], [], [], [], []
+    for r in range(R):
+        t, k, p = cases[r % len(cases)]
+        temps.append(t), ks.append(k), ps.append(p)
+        us.append(P.uniform_from_counter(7, r))
+        tok, margin = P.sample_token(logits[r], t, k, p, 7, r)
+        want.append(tok), margins.append(margin)
+    got = sample(ops, logits, temps, ks, ps, us)
+    for r in range(R):
+        assert got[r] == want[r] or margins[r] < 1e-4, f"row {r} {cases[r % len(cases)]}: {got[r]} != {want[r]}"
+    assert sum(g == w for g, w in zip(got, want)) >= R - 2
+    # a row's token does not depend on the rows beside it
+    for r in (2, 3, 7, 8, 19):
+        assert sample(ops, logits[r:r + 1], temps[r:r + 1], ks[r:r + 1], ps[r:r + 1], us[r:r + 1]) == [got[r]]
+    # rows that use no filter: the same with the filters' launches left out
+    plain_rows = [r for r in range(R) if r % len(cases) in (0, 4, 5)]
+    out = torch.empty(len(plain_rows), dtype=torch.int32, device=DEV)
+    f = lambda x: torch.tensor(x, dtype=torch.float32, device=DEV)    # noqa: E731
+    ops.sample_rows(logits[plain_rows].to(DEV), f([temps[r] for r in plain_rows]),
+                    torch.tensor([ks[r] for r in plain_rows], dtype=torch.int32, device=DEV),
+                    f([ps[r] for r in plain_rows]), f([us[r] for r in plain_rows]), out,
+                    uses_top_k=False, uses_top_p=False)
+    assert out.cpu().tolist() == [got[r] for r in plain_rows]
+
+
+def test_sample_rows_keeps_ties_at_the_kth_value_in_vocabulary_order(ops):
+    """Five entries share the k-th largest value, spread over three chunks; top_k = 4 keeps the two larger
+    entries and the first two of the ties, whatever u is; with top_p on top the nucleus is cut inside them."""
+    V = 3 * 4096 + 100
+    row = torch.full((V,), -4.0)
+    row[9000], row[300] = 3.0, 2.5
+    ties = [120, 4095, 4096, 8200, 12300]
+    row[ties] = 1.0
+    n = 256
+    draws = [(i + 0.5) / n for i in range(n)]
+    got = sample(ops, row.repeat(n, 1), [1.0] * n, [4] * n, [1.0] * n, draws)
+    assert set(got) == {9000, 300, 120, 4095}
+    want = torch.softmax(torch.tensor([1.0, 2.5, 1.0, 3.0]), -1)      # tokens 120, 300, 4095, 9000 in vocabulary order
+    for tok, w in zip((120, 300, 4095, 9000), want.tolist()):
+        assert abs(got.count(tok) / n - w) < 1.5 / n + 1e-3
+    got = sample(ops, row.repeat(n, 1), [1.0] * n, [6] * n, [1.0] * n, draws)
+    assert set(got) == {9000, 300, 120, 4095, 4096, 8200}
+    got = sample(ops, row.repeat(n, 1), [1.0] * n, [4] * n, [0.6] * n, draws)    # 3.0 and 2.5 hold 0.84 of the mass
+    assert set(got) == {9000, 300}
+
+
 def test_sample_rows_filters_on_the_references_vectors(ops):
     """reference tests/test_sampling.py:16-31: what top-k and top-p keep."""
     draws = [i / 64 + 1 / 128 for i in range(64)]

@@ -79,7 +79,9 @@ int tm_attn_prefill_f32(const void* q, int q_stride, void* out, int out_stride, 
 int tm_argmax_work_chunks(int V);
 int tm_argmax_rows(const float* logits, int R, int V, int* out, float* work_v, int* work_i, hipStream_t stream);
 
+size_t tm_sample_work_bytes(int R, int V);
 int tm_sample_rows(const float* logits, int R, int V, const float* temperature, const int* top_k,
-                   const float* top_p, const float* u, int* out, hipStream_t stream);
+                   const float* top_p, const float* u, int* out, void* work, size_t work_bytes, int stages,
+                   hipStream_t stream);
 
 }  // extern "C"

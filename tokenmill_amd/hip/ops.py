@@ -318,10 +318,15 @@ def argmax_rows(logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     return out
 
 
+_sample_work: dict[int, torch.Tensor] = {}
+
+
 def sample_rows(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
-                u: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+                u: torch.Tensor, out: torch.Tensor, uses_top_k: bool = True, uses_top_p: bool = True) -> torch.Tensor:
     """One token per row: argmax where temperature <= 1e-5 or top_k == 1, else the inverse CDF at
-    u of softmax(logits / temperature) after the top-k / top-p filters, in vocabulary order."""
+    u of softmax(logits / temperature) after the top-k / top-p filters, in vocabulary order.
+    ``uses_top_k`` / ``uses_top_p``: False if the caller knows that no row asks for that filter (its
+    launches are then left out; a row that asks for none skips their work either way)."""
     _gpu(logits, temperature, top_k, top_p, u, out)
     R, V = logits.shape
     _need(logits.dtype == torch.float32 and logits.is_contiguous(), "sample: logits must be contiguous float32 [R, V]")
@@ -329,8 +334,16 @@ def sample_rows(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Te
         _need(t.dtype == torch.float32 and t.is_contiguous() and t.numel() == R, f"sample: {name} must be float32 [R]")
     _ints(top_k, R, "top_k")
     _ints(out, R, "out")
-    _check(library().tm_sample_rows(_p(logits), c_int(R), c_int(V), _p(temperature), _p(top_k), _p(top_p), _p(u),
-                                    _p(out), _stream()), "sample_rows")
+    _need(V <= 1 << 20, f"sample: at most 2^20 logits a row, got {V}")
+    lib = library()
+    lib.tm_sample_work_bytes.restype = ctypes.c_size_t
+    need = lib.tm_sample_work_bytes(c_int(R), c_int(V))
+    work = _sample_work.get(logits.device.index)
+    if work is None or work.numel() < need:            # kept and grown: one sampling call at a time per device
+        work = _sample_work[logits.device.index] = torch.empty(need, dtype=torch.uint8, device=logits.device)
+    _check(lib.tm_sample_rows(_p(logits), c_int(R), c_int(V), _p(temperature), _p(top_k), _p(top_p), _p(u), _p(out),
+                              _p(work), ctypes.c_size_t(work.numel()), c_int((1 if uses_top_k else 0) | (2 if uses_top_p else 0)),
+                              _stream()), "sample_rows")
     return out
 
 

@@ -74,5 +74,8 @@ class Sampler:
         ks = torch.tensor([p.top_k for p in params], dtype=torch.int32).view(torch.float32)
         host[3] = ks                                              # int32 bits travel in the same copy
         dev = host.to(logits.device, non_blocking=True)
-        ops.sample_rows(logits, dev[0], dev[3].view(torch.int32), dev[1], dev[2], out)
+        vocab = logits.shape[1]
+        ops.sample_rows(logits, dev[0], dev[3].view(torch.int32), dev[1], dev[2], out,
+                        uses_top_k=any(not p.greedy and 0 < p.top_k < vocab for p in params),
+                        uses_top_p=any(not p.greedy and p.top_p < 1.0 for p in params))
         return out.tolist()
