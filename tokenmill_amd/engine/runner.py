@@ -125,7 +125,8 @@ class ModelRunner:
         first_row = [0] * S
         q_lens, starts = [], []
         cu[0] = 0
-        for s, i in enumerate(order):
+        n_portions = sum(1 for e in entries if len(e.tokens) > 1)
+        for s, i in enumerate(order[:n_portions]):
             e = entries[i]
             n = len(e.tokens)
             toks = np.asarray(e.tokens, dtype=np.int64)
@@ -159,6 +160,43 @@ class ModelRunner:
             q_lens.append(n)
             starts.append(e.start)
             row0 += n
+        # single tokens: the same rows, written with a few bulk assignments instead of a dozen array
+        # operations each (a mixed step may hold a hundred of them)
+        singles = [entries[i] for i in order[n_portions:]]
+        if singles:
+            n1 = len(singles)
+            s0 = n_portions
+            toks = np.asarray([e.tokens[0] for e in singles], dtype=np.int64)
+            if toks.min() < 0 or toks.max() >= self.vocab:
+                raise StepError(f"a token id is outside the vocabulary of {self.vocab}")
+            p1 = [e.start for e in singles]
+            ids[row0:row0 + n1] = toks
+            pos[row0:row0 + n1] = p1
+            seq_of[row0:row0 + n1] = np.arange(s0, s0 + n1)
+            cu[s0 + 1:s0 + n1 + 1] = np.arange(row0 + 1, row0 + n1 + 1)
+            ctx_lens[s0:s0 + n1] = [p + 1 for p in p1]
+            slots_state[s0:s0 + n1] = [e.cache.state_slot for e in singles]
+            for g in range(n_groups):
+                tabs = g_tab[g][0][s0 * W:(s0 + n1) * W].reshape(n1, W)
+                windowed = self.pools.groups[g].window is not None
+                new_slots = []
+                for j, (e, p) in enumerate(zip(singles, p1)):
+                    table = e.cache.tables[g]
+                    last = p // page
+                    if table[last] == RELEASED:
+                        raise StepError(f"{e.cache.request_id}: a token would be written to a page already given back")
+                    new_slots.append(table[last] * page + p % page)
+                    row = tabs[j]
+                    row[:last + 1] = table[:last + 1]
+                    row[last + 1:] = 0                                        # padding: never read
+                    if windowed:
+                        row[row == RELEASED] = 0                              # never read: below the window
+                g_slot[g][0][row0:row0 + n1] = new_slots
+            for j, i in enumerate(order[n_portions:]):
+                first_row[i] = row0 + j
+            q_lens.extend([1] * n1)
+            starts.extend(p1)
+            row0 += n1
         if n_tiles > 1:
             # the tiles that see the most keys first: the long ones start early and the short ones fill
             # the end of the launch (a tile's result does not depend on where in the table it stands)
