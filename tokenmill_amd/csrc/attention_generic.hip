@@ -21,6 +21,8 @@
 #define AG_WAVES 4
 #define AG_SPLIT_WAVES 8
 #define AG_MAXD 256
+#define AG_KCHUNK 16        // floats of every key staged at a time
+#define AG_KSTRIDE 20       // floats between two keys of the staged tile (rows 16 bytes aligned, no bank conflicts)
 
 // four consecutive elements as 32-bit floats
 __device__ __forceinline__ void ag_load4(const float* p, float (&v)[4]) {
@@ -41,13 +43,19 @@ __device__ __forceinline__ void ag_load4(const bf16_t* p, float (&v)[4]) {
 //                are merged through LDS in wavefront order (steps with few tokens, where the pairs
 //                alone would leave most of the chip idle). Which keys a wavefront takes depends on
 //                the token's own position and window only.
-template <typename T, bool SPLIT>
+// DMAX > 0 (head sizes up to 128): the weights meet the values with a lane still holding its own key, so
+//                that a load of one d reads runs of consecutive keys; every lane keeps partial sums for
+//                all d over its keys and the lanes are added once, at the end. DMAX = 0: a lane holds
+//                d = lane, lane + 64, ... and the keys of a group are visited one after the other.
+template <typename T, bool SPLIT, int DMAX>
 __global__ __launch_bounds__((SPLIT ? AG_SPLIT_WAVES : AG_WAVES) * TM_WAVE) void attn_paged_generic_kernel(
     const T* __restrict__ q, int q_stride, T* __restrict__ out, int out_stride,
     const T* __restrict__ k_pool, const T* __restrict__ v_pool, const int* __restrict__ block_tables,
     int table_width, const int* __restrict__ seq_of_token, const int* __restrict__ positions, int T_tokens,
     int H, int KVH, int D, int page, float scale, int window) {
     constexpr int WAVES = SPLIT ? AG_SPLIT_WAVES : AG_WAVES;
+    constexpr bool STAGED = DMAX > 0 && sizeof(T) == 4;         // 32-bit keys through LDS (see the key loop)
+    __shared__ __align__(16) float k_tile[STAGED ? WAVES : 1][STAGED ? TM_WAVE * AG_KSTRIDE : 4];
     __shared__ float q_s[SPLIT ? 1 : AG_WAVES][AG_MAXD];
     __shared__ float s_m[SPLIT ? AG_SPLIT_WAVES : 1], s_l[SPLIT ? AG_SPLIT_WAVES : 1];
     __shared__ float s_acc[SPLIT ? AG_SPLIT_WAVES : 1][SPLIT ? AG_MAXD : 1];
@@ -75,6 +83,9 @@ __global__ __launch_bounds__((SPLIT ? AG_SPLIT_WAVES : AG_WAVES) * TM_WAVE) void
     float acc[AG_MAXD / TM_WAVE];
 #pragma unroll
     for (int i = 0; i < AG_MAXD / TM_WAVE; ++i) acc[i] = 0.f;
+    float part[DMAX > 0 ? DMAX : 1];            // DMAX > 0: this lane's sums over its own keys, every d
+#pragma unroll
+    for (int d = 0; d < (DMAX > 0 ? DMAX : 1); ++d) part[d] = 0.f;
 
     const int first = SPLIT ? lo + wave * TM_WAVE : lo;
     const int stride = SPLIT ? WAVES * TM_WAVE : TM_WAVE;
@@ -83,7 +94,43 @@ __global__ __launch_bounds__((SPLIT ? AG_SPLIT_WAVES : AG_WAVES) * TM_WAVE) void
         const bool valid = j <= p;
         long long row = 0;
         float sc = -INFINITY;
-        if (valid) {
+        if constexpr (STAGED) {
+            // The group's key rows come through LDS, 16 floats of every key at a time: a load takes 64
+            // bytes of each of 16 keys (whole runs of memory), where a lane reading its own key's row
+            // 16 bytes at a time touches 64 cache lines a load and keeps coming back to them.
+            // A lane beyond the newest key stands for the newest key (finite values, score masked).
+            const int jc = valid ? j : p;
+            row = (long long)table[jc / page] * page + (jc % page);
+            long long row_of[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) row_of[c] = __shfl(row, 16 * c + lane / 4, TM_WAVE);
+            float* tile = k_tile[wave];
+            float dot = 0.f;
+            for (int dc = 0; dc < D; dc += AG_KCHUNK) {
+                const int dp = dc + 4 * (lane % 4);
+                // no test around the loads (a tested load is waited for by itself): beyond D they read
+                // the row's first floats again, which the products below never use
+                float4 piece[4];
+#pragma unroll
+                for (int c = 0; c < 4; ++c)
+                    piece[c] = *(const float4*)(k_pool + ((size_t)row_of[c] * KVH + kvh) * D + (dp < D ? dp : 0));
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int c = 0; c < 4; ++c)
+                    *(float4*)(tile + (16 * c + lane / 4) * AG_KSTRIDE + 4 * (lane % 4)) = piece[c];
+#pragma unroll
+                for (int dd = 0; dd < AG_KCHUNK; dd += 4) {
+                    const float4 kv = *(const float4*)(tile + lane * AG_KSTRIDE + dd);
+                    if (dc + dd < D) {
+                        dot = fmaf(qs[dc + dd + 0], kv.x, dot);
+                        dot = fmaf(qs[dc + dd + 1], kv.y, dot);
+                        dot = fmaf(qs[dc + dd + 2], kv.z, dot);
+                        dot = fmaf(qs[dc + dd + 3], kv.w, dot);
+                    }
+                }
+            }
+            if (valid) sc = dot * scale;
+        } else if (valid) {
             row = (long long)table[j / page] * page + (j % page);
             const T* kr = k_pool + ((size_t)row * KVH + kvh) * D;
             float dot = 0.f;
@@ -103,6 +150,24 @@ __global__ __launch_bounds__((SPLIT ? AG_SPLIT_WAVES : AG_WAVES) * TM_WAVE) void
         l = l * corr + wave_sum(pr);
         m = m_new;
         const float pr_v = Elem<T>::round(pr);          // weights are stored-type values when they meet v
+        if constexpr (DMAX > 0) {
+            // a lane beyond the newest key reads the newest key's values (finite) with weight 0
+            const long long rv = (valid || STAGED) ? row : (long long)table[p / page] * page + (p % page);
+            const T* vr = v_pool + ((size_t)(rv / page) * KVH + kvh) * D * page + (rv % page);
+            // every load without a test, all of a group in flight at once: beyond D a lane reads d = 0
+            // again and the sum it feeds is never looked at
+#pragma unroll
+            for (int d0 = 0; d0 < DMAX; d0 += 64) {     // 64 loads in flight at a time
+                float vals[64];
+#pragma unroll
+                for (int d = 0; d < 64; ++d) vals[d] = Elem<T>::load(vr + (size_t)(d0 + d < D ? d0 + d : 0) * page);
+                __builtin_amdgcn_sched_barrier(0);      // (else the compiler asks for them one by one, to save registers)
+#pragma unroll
+                for (int d = 0; d < 64; ++d) part[d0 + d] = fmaf(pr_v, vals[d], part[d0 + d] * corr);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            continue;
+        }
 #pragma unroll
         for (int i = 0; i < AG_MAXD / TM_WAVE; ++i) acc[i] *= corr;
         const int n = (p - j0 + 1) < TM_WAVE ? (p - j0 + 1) : TM_WAVE;
@@ -114,6 +179,15 @@ __global__ __launch_bounds__((SPLIT ? AG_SPLIT_WAVES : AG_WAVES) * TM_WAVE) void
             for (int i = 0; i < AG_MAXD / TM_WAVE; ++i) {
                 const int d = lane + i * TM_WAVE;
                 if (d < D) acc[i] = fmaf(pj, Elem<T>::load(vr + (size_t)d * page), acc[i]);
+            }
+        }
+    }
+    if constexpr (DMAX > 0) {                   // the lanes' sums added, lane d % 64 keeps d
+#pragma unroll
+        for (int d = 0; d < DMAX; ++d) {
+            if (d < D) {
+                const float total = wave_sum(part[d]);
+                if (lane == d % TM_WAVE) acc[d / TM_WAVE] = total;
             }
         }
     }
@@ -152,21 +226,35 @@ __global__ __launch_bounds__((SPLIT ? AG_SPLIT_WAVES : AG_WAVES) * TM_WAVE) void
     }
 }
 
+template <typename T, int DMAX>
+static void launch_generic_d(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
+                             const void* v_pool, const int* block_tables, int table_width, const int* seq_of_token,
+                             const int* positions, int T_tokens, int H, int KVH, int D, int page, float scale,
+                             int window, hipStream_t stream) {
+    const long long pairs = (long long)T_tokens * H;
+    if (pairs < 1024)           // too few (token, head) pairs to fill the chip: the wavefronts of a block split the keys
+        attn_paged_generic_kernel<T, true, DMAX><<<(unsigned)pairs, AG_SPLIT_WAVES * TM_WAVE, 0, stream>>>(
+            (const T*)q, q_stride, (T*)out, out_stride, (const T*)k_pool, (const T*)v_pool, block_tables,
+            table_width, seq_of_token, positions, T_tokens, H, KVH, D, page, scale, window);
+    else
+        attn_paged_generic_kernel<T, false, DMAX><<<(unsigned)((pairs + AG_WAVES - 1) / AG_WAVES),
+                                                    AG_WAVES * TM_WAVE, 0, stream>>>(
+            (const T*)q, q_stride, (T*)out, out_stride, (const T*)k_pool, (const T*)v_pool, block_tables,
+            table_width, seq_of_token, positions, T_tokens, H, KVH, D, page, scale, window);
+}
+
 template <typename T>
 static void launch_generic(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
                            const void* v_pool, const int* block_tables, int table_width, const int* seq_of_token,
                            const int* positions, int T_tokens, int H, int KVH, int D, int page, float scale,
                            int window, hipStream_t stream) {
-    const long long pairs = (long long)T_tokens * H;
-    if (pairs < 1024)           // too few (token, head) pairs to fill the chip: the wavefronts of a block split the keys
-        attn_paged_generic_kernel<T, true><<<(unsigned)pairs, AG_SPLIT_WAVES * TM_WAVE, 0, stream>>>(
-            (const T*)q, q_stride, (T*)out, out_stride, (const T*)k_pool, (const T*)v_pool, block_tables,
-            table_width, seq_of_token, positions, T_tokens, H, KVH, D, page, scale, window);
-    else
-        attn_paged_generic_kernel<T, false><<<(unsigned)((pairs + AG_WAVES - 1) / AG_WAVES), AG_WAVES * TM_WAVE, 0,
-                                              stream>>>(
-            (const T*)q, q_stride, (T*)out, out_stride, (const T*)k_pool, (const T*)v_pool, block_tables,
-            table_width, seq_of_token, positions, T_tokens, H, KVH, D, page, scale, window);
+#define TM_GENERIC(DMAX)                                                                                       \
+    launch_generic_d<T, DMAX>(q, q_stride, out, out_stride, k_pool, v_pool, block_tables, table_width,         \
+                              seq_of_token, positions, T_tokens, H, KVH, D, page, scale, window, stream)
+    if (D <= 64) TM_GENERIC(64);
+    else if (D <= 128) TM_GENERIC(128);
+    else TM_GENERIC(0);
+#undef TM_GENERIC
 }
 
 extern "C" int tm_attn_paged_generic(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
