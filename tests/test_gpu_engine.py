@@ -267,12 +267,12 @@ def test_decode_steps_replayed_from_hip_graphs(model_dirs, plains, dtype_name):
 @pytest.mark.parametrize("portion", [16, 48])
 @pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
 def test_prompt_portions_replayed_from_hip_graphs(model_dirs, plains, dtype_name, portion):
-    """Long prompts cut into portions of 16 tokens (this library's own products) or 48 (the library
-    products, which then are nodes of the graph), one request at a time: the second portion of a
-    length captures a graph, the later ones (of this prompt and of the next prompts, at other
-    positions and on other pages) replay it, with eager steps (the last, shorter portion; the decode
-    steps of other sizes) and synchronisations in between. Every replay must give what the eager
-    engine gives, and what the plain implementation gives."""
+    """Long prompts cut into portions of 16 tokens (run as 32 rows, half of them padding: this library's
+    own products) or 48 (run as 64 rows: the library products, which then are nodes of the graph), one
+    request at a time: the second portion of a size captures a graph, the later ones (of this prompt and
+    of the next prompts, at other positions and on other pages; the last, shorter portions too, which
+    run with the same number of rows) replay it, with eager steps and synchronisations in between.
+    Every replay must give what the eager engine gives, and what the plain implementation gives."""
     from tokenmill_amd import SamplingParams
     lengths = [100, 77, 33, 120] if portion == 16 else [200, 150, 97, 240]
     prompts = [random_ids(n, 384, 190 + i) for i, n in enumerate(lengths)]
@@ -284,7 +284,32 @@ def test_prompt_portions_replayed_from_hip_graphs(model_dirs, plains, dtype_name
         outs[graphs] = [eng.generate([p], sp)[0] for p in prompts]
         if graphs:
             pg = eng.runner.portion_graphs
-            assert pg.replays >= (15 if portion == 16 else 8) and (portion, False) in pg.portions
+            assert pg.replays >= (15 if portion == 16 else 8) and (pg.padded_rows(portion), False) in pg.portions
+        assert eng.cache.num_free_pages == eng.cache.num_pages
+    for p, o in zip(prompts, outs[True]):
+        verify(plains["B"], p, o, DTYPES[dtype_name])
+    assert outs[True] == outs[False]
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_prompts_of_similar_lengths_replay_one_graph(model_dirs, plains, dtype_name):
+    """Whole prompts of many different lengths, one request at a time: a step runs with its rows padded to
+    a few sizes, so lengths 17..32 share one graph and 33..64 another (padding rows carry token 0 without
+    a cache slot, and repeated attention tiles fill the tile table). Tokens as from the eager engine and
+    the plain implementation; a prompt of one token (a decode step) and the cache pages are untouched by
+    the padding."""
+    from tokenmill_amd import SamplingParams
+    lengths = [19, 31, 17, 32, 40, 33, 64, 61, 1, 2, 47, 90, 5, 96, 70]
+    prompts = [random_ids(n, 384, 500 + i) for i, n in enumerate(lengths)]
+    sp = SamplingParams(max_tokens=4, ignore_eos=True)
+    outs = {}
+    for graphs in (False, True):
+        eng = make_engine(model_dirs["B"], dtype_name, block_size=8, hip_graphs=graphs, max_num_seqs=2,
+                          max_num_batched_tokens=128, max_model_len=128)
+        outs[graphs] = [eng.generate([p], sp)[0] for p in prompts]
+        if graphs:
+            pg = eng.runner.portion_graphs
+            assert set(pg.portions) == {(32, True), (64, True), (96, True)} and pg.replays >= 9
         assert eng.cache.num_free_pages == eng.cache.num_pages
     for p, o in zip(prompts, outs[True]):
         verify(plains["B"], p, o, DTYPES[dtype_name])

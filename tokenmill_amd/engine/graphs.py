@@ -174,11 +174,12 @@ class _Portion:
 
 class PortionGraphs:
     """Graphs for steps of exactly one entry with several tokens (a prompt or a portion of one) that
-    wants no logits or those of its last token. A shape (tokens, wants logits) is captured when it
-    comes the second time; the most recently used ``max_graphs`` shapes are kept (each holds the
-    activations of a step of its size)."""
+    wants no logits or those of its last token. The step runs with its rows padded to a few sizes
+    (``padded_rows``); a shape (rows, wants logits) is captured when it comes the second time; the
+    most recently used ``max_graphs`` shapes are kept (each holds the activations of a step of its
+    size)."""
 
-    def __init__(self, runner, max_graphs: int = 4):
+    def __init__(self, runner, max_graphs: int = 16):
         self.runner = runner
         ops.library_workspace(runner.device)
         self.W = -(-runner.max_positions // runner.page_size)
@@ -186,6 +187,14 @@ class PortionGraphs:
         self.seen: dict[tuple, int] = {}
         self.portions: dict[tuple, _Portion] = {}          # insertion order = least recently used first
         self.replays = 0
+
+    @staticmethod
+    def padded_rows(n: int) -> int:
+        """Rows a portion of n tokens runs with: the next multiple of 32 (64 above 512 tokens, 128
+        above 1,024, 256 above 2,048), so that prompts of similar lengths replay one graph; at most
+        an eighth of the rows is padding beyond the first steps."""
+        step = 32 if n <= 512 else (64 if n <= 1024 else (128 if n <= 2048 else 256))
+        return -(-n // step) * step
 
     def can_run(self, entries) -> bool:
         if len(entries) != 1 or self.runner.pools.states:
@@ -199,17 +208,18 @@ class PortionGraphs:
         caller then runs the step kernel by kernel)."""
         runner = self.runner
         e = entries[0]
-        key = (len(e.tokens), bool(e.want))
+        T = self.padded_rows(len(e.tokens))
+        key = (T, bool(e.want))
         slot = self.portions.pop(key, None)
         if slot is None:
             self.seen[key] = self.seen.get(key, 0) + 1
             if self.seen[key] < 2:
                 return None
             slot = _Portion()
-            T, n_groups = len(e.tokens), len(runner.pools.groups)
-            n_ints = 3 * T + 2 + 2 + 1 + n_groups * (T + self.W) + 4 * (-(-T // 16))
+            n_groups = len(runner.pools.groups)
+            n_ints = 3 * T + 2 + 2 + 1 + n_groups * (T + self.W) + 4 * (T // 16)
             slot.dev = torch.zeros(n_ints, dtype=torch.int32, device=runner.device)
-            step, _ = runner.prepare(entries, into=slot.dev, table_width=self.W)
+            step, _ = runner.prepare(entries, into=slot.dev, table_width=self.W, pad_rows_to=T)
             torch.cuda.synchronize()
             side = torch.cuda.Stream()
             side.wait_stream(torch.cuda.current_stream())
@@ -225,7 +235,7 @@ class PortionGraphs:
             while len(self.portions) >= self.max_graphs:    # the least recently used shape gives its memory back
                 self.portions.pop(next(iter(self.portions)))
         else:
-            runner.prepare(entries, into=slot.dev, table_width=self.W)
+            runner.prepare(entries, into=slot.dev, table_width=self.W, pad_rows_to=T)
         self.portions[key] = slot
         slot.graph.replay()
         self.replays += 1

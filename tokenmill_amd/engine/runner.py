@@ -59,12 +59,17 @@ class ModelRunner:
         return self._pinned.numpy()
 
     def prepare(self, entries: list[StepEntry], into: torch.Tensor | None = None,
-                table_width: int | None = None) -> tuple[StepContext, list[int]]:
+                table_width: int | None = None, pad_rows_to: int | None = None) -> tuple[StepContext, list[int]]:
         """Flatten the entries into device metadata. Returns the context and, for each wanted logit
         in the caller's order (entries in the given order, ``want`` in its order), its row in the
         step's logits. ``into``: a device int32 buffer to hold the metadata (a captured graph reads
         it at a fixed address; steps of the same shape lay it out the same way); ``table_width``:
-        pad the block tables to this width instead of the widest of the step."""
+        pad the block tables to this width instead of the widest of the step; ``pad_rows_to`` (a
+        multiple of 16): rows behind the entries' tokens up to this many, so that steps of similar
+        sizes launch the same grids. A padding row is token 0 at position 0 with no cache slot (its
+        keys are not stored) and belongs to no attention tile; every kernel treats rows apart, so
+        what such a row holds reaches no other row. The tile table is filled up to one tile per 16
+        rows with repeats of a real tile, which compute the same rows again."""
         if not entries:
             raise StepError("a step needs at least one entry")
         page = self.page_size
@@ -72,7 +77,12 @@ class ModelRunner:
         # prompt portions first, single tokens last (the order the attention kernels split on)
         order = sorted(range(len(entries)), key=lambda i: len(entries[i].tokens) == 1)
         S = len(entries)
-        T = sum(len(e.tokens) for e in entries)
+        T_real = sum(len(e.tokens) for e in entries)
+        T = T_real
+        if pad_rows_to is not None:
+            if pad_rows_to < T_real or pad_rows_to % 16:
+                raise StepError(f"{T_real} rows cannot be padded to {pad_rows_to}")
+            T = pad_rows_to
         R = sum(len(e.want) for e in entries)
         widths = []
         for e in entries:
@@ -95,7 +105,8 @@ class ModelRunner:
             if table_width < W:
                 raise StepError(f"block tables of {W} pages do not fit the width {table_width}")
             W = table_width
-        n_tiles = sum(-(-len(e.tokens) // 16) for e in entries if len(e.tokens) > 1)
+        n_tiles_real = sum(-(-len(e.tokens) // 16) for e in entries if len(e.tokens) > 1)
+        n_tiles = max(n_tiles_real, T // 16) if (pad_rows_to is not None and n_tiles_real) else n_tiles_real
         n_ints = 3 * T + (S + 1) + 2 * S + max(R, 1) + n_groups * (T + S * W) + 4 * n_tiles
         buf = self._staging(n_ints)
         off = 0
@@ -197,6 +208,15 @@ class ModelRunner:
             q_lens.extend([1] * n1)
             starts.extend(p1)
             row0 += n1
+        if T > T_real:                                                        # padding rows
+            ids[T_real:] = 0
+            pos[T_real:] = 0
+            seq_of[T_real:] = 0
+            for g in range(n_groups):
+                g_slot[g][0][T_real:] = -1
+        if n_tiles > n_tiles_real:                                            # repeats of the last real tile
+            t = tiles.reshape(n_tiles, 4)
+            t[n_tiles_real:] = t[n_tiles_real - 1]
         if n_tiles > 1:
             # the tiles that see the most keys first: the long ones start early and the short ones fill
             # the end of the launch (a tile's result does not depend on where in the table it stands)
