@@ -283,8 +283,8 @@ def test_prompt_portions_replayed_from_hip_graphs(model_dirs, plains, dtype_name
                           max_num_batched_tokens=portion, enable_chunked_prefill=True, max_model_len=256)
         outs[graphs] = [eng.generate([p], sp)[0] for p in prompts]
         if graphs:
-            pg = eng.runner.portion_graphs
-            assert pg.replays >= (15 if portion == 16 else 8) and (pg.padded_rows(portion), False) in pg.portions
+            sg = eng.runner.step_graphs
+            assert sg.replays >= (15 if portion == 16 else 8) and (sg.padded_rows(portion), 1, 0, 0) in sg.captured
         assert eng.cache.num_free_pages == eng.cache.num_pages
     for p, o in zip(prompts, outs[True]):
         verify(plains["B"], p, o, DTYPES[dtype_name])
@@ -308,8 +308,33 @@ def test_prompts_of_similar_lengths_replay_one_graph(model_dirs, plains, dtype_n
                           max_num_batched_tokens=128, max_model_len=128)
         outs[graphs] = [eng.generate([p], sp)[0] for p in prompts]
         if graphs:
-            pg = eng.runner.portion_graphs
-            assert set(pg.portions) == {(32, True), (64, True), (96, True)} and pg.replays >= 9
+            sg = eng.runner.step_graphs
+            assert set(sg.captured) == {(32, 1, 0, 1), (64, 1, 0, 1), (96, 1, 0, 1)} and sg.replays >= 9
+        assert eng.cache.num_free_pages == eng.cache.num_pages
+    for p, o in zip(prompts, outs[True]):
+        verify(plains["B"], p, o, DTYPES[dtype_name])
+    assert outs[True] == outs[False]
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_mixed_steps_replayed_from_hip_graphs(model_dirs, plains, dtype_name):
+    """Many requests at once with a small token budget: most steps hold portions of several prompts beside
+    the decoded tokens of the running requests, in numbers that change from step to step. Such steps are
+    laid out in a padded shape (rows, portions, single tokens and logit rows rounded up) and replayed from
+    a few graphs; requests come and go, pages are handed out again. Tokens as from the eager engine and as
+    the plain implementation gives them."""
+    from tokenmill_amd import SamplingParams
+    lengths = [1 + (11 * i) % 37 for i in range(40)]
+    prompts = [random_ids(n, 384, 700 + i) for i, n in enumerate(lengths)]
+    params = [SamplingParams(max_tokens=3 + i % 9, ignore_eos=True) for i in range(len(prompts))]
+    outs = {}
+    for graphs in (False, True):
+        eng = make_engine(model_dirs["B"], dtype_name, block_size=8, num_blocks=40, hip_graphs=graphs, max_num_seqs=6,
+                          max_num_batched_tokens=24, enable_chunked_prefill=True, max_model_len=96)
+        outs[graphs] = eng.generate(prompts, params)
+        if graphs:
+            sg = eng.runner.step_graphs
+            assert sg.replays >= 20 and any(k[2] > 0 for k in sg.captured) and any(k[1] > 1 for k in sg.captured)
         assert eng.cache.num_free_pages == eng.cache.num_pages
     for p, o in zip(prompts, outs[True]):
         verify(plains["B"], p, o, DTYPES[dtype_name])

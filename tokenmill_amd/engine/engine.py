@@ -73,9 +73,9 @@ class LLMEngine:
         self.cache = CacheManager(self.pools.windows, pages, cfg.block_size, cfg.max_num_seqs, cfg.watermark)
         self.runner = ModelRunner(model, self.pools, max_positions=cfg.max_model_len)
         if cfg.hip_graphs:
-            from tokenmill_amd.engine.graphs import DecodeGraphs, PortionGraphs
+            from tokenmill_amd.engine.graphs import DecodeGraphs, StepGraphs
             self.runner.graphs = DecodeGraphs(self.runner, cfg)
-            self.runner.portion_graphs = PortionGraphs(self.runner)
+            self.runner.step_graphs = StepGraphs(self.runner)
         self.scheduler = Scheduler(cfg, self.cache)
         self.sampler = Sampler(self.device)
         self.seqs: dict[str, Sequence] = {}

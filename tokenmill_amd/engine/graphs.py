@@ -10,9 +10,10 @@ profile of where an eager decode step's time goes, bench/results/profile/decode_
 Padding rows carry token 0 at position 0, a context of one key, and cache slot -1, which the cache
 write skips; their logits are never looked at. The graphs hold no memset node.
 
-A step that is one portion of one prompt launches the same kernels with the same grids as any other
-portion of that length (its positions, pages and tiles are data), so a long prompt cut into equal
-portions, or prompts of one length arriving one after the other, replay one graph: ``PortionGraphs``.
+A step that holds prompt portions, alone or beside single tokens, launches the same kernels with the
+same grids as any other step of its padded shape (positions, pages and tiles are data), so the equal
+portions of a long prompt, prompts of similar lengths arriving one after the other, and the mixed
+steps of a serving run replay a handful of graphs: ``StepGraphs``.
 """
 from __future__ import annotations
 
@@ -165,61 +166,84 @@ class DecodeGraphs:
         bk.graph = graph
 
 
-class _Portion:
+class _Captured:
     def __init__(self):
         self.dev: torch.Tensor | None = None
         self.graph: torch.cuda.CUDAGraph | None = None
         self.logits: torch.Tensor | None = None
 
 
-class PortionGraphs:
-    """Graphs for steps of exactly one entry with several tokens (a prompt or a portion of one) that
-    wants no logits or those of its last token. The step runs with its rows padded to a few sizes
-    (``padded_rows``); a shape (rows, wants logits) is captured when it comes the second time; the
-    most recently used ``max_graphs`` shapes are kept (each holds the activations of a step of its
-    size)."""
+def _next_power_of_two(n: int) -> int:
+    return 1 << (n - 1).bit_length() if n > 0 else 0
 
-    def __init__(self, runner, max_graphs: int = 16):
+
+class StepGraphs:
+    """Graphs for steps that hold prompt portions (whole prompts or parts of them), alone or beside
+    single decoded tokens, where every entry wants at most one row of logits. The step is laid out
+    in a padded shape (``padded_shape``): the portions' rows up to a few sizes, the numbers of
+    portions, single tokens and logit rows up to powers of two, so that steps of similar sizes launch
+    the same grids. A shape is captured when it comes the second time (the fourth, for a step of
+    several entries); the most recently used
+    ``max_graphs`` shapes are kept (each holds the activations of a step of its size)."""
+
+    def __init__(self, runner, max_graphs: int = 16, max_singles: int = 256):
         self.runner = runner
         ops.library_workspace(runner.device)
         self.W = -(-runner.max_positions // runner.page_size)
-        self.max_graphs = max_graphs
+        self.max_graphs, self.max_singles = max_graphs, max_singles
+        self.max_mixed_rows = 1024
         self.seen: dict[tuple, int] = {}
-        self.portions: dict[tuple, _Portion] = {}          # insertion order = least recently used first
+        self.captured: dict[tuple, _Captured] = {}         # insertion order = least recently used first
         self.replays = 0
 
     @staticmethod
     def padded_rows(n: int) -> int:
-        """Rows a portion of n tokens runs with: the next multiple of 32 (64 above 512 tokens, 128
-        above 1,024, 256 above 2,048), so that prompts of similar lengths replay one graph; at most
-        an eighth of the rows is padding beyond the first steps."""
+        """Rows that portions of n tokens in all run with: the next multiple of 32 (64 above 512
+        tokens, 128 above 1,024, 256 above 2,048); at most an eighth of the rows is padding beyond
+        the first steps."""
         step = 32 if n <= 512 else (64 if n <= 1024 else (128 if n <= 2048 else 256))
         return -(-n // step) * step
 
+    @classmethod
+    def padded_shape(cls, entries) -> tuple[int, int, int, int]:
+        """(rows of the portions, portions, single tokens, logit rows) the step is laid out with."""
+        rows = sum(len(e.tokens) for e in entries if len(e.tokens) > 1)
+        portions = sum(1 for e in entries if len(e.tokens) > 1)
+        wanted = sum(len(e.want) for e in entries)
+        return (cls.padded_rows(rows), _next_power_of_two(portions), _next_power_of_two(len(entries) - portions),
+                _next_power_of_two(wanted))
+
     def can_run(self, entries) -> bool:
-        if len(entries) != 1 or self.runner.pools.states:
+        if self.runner.pools.states:
             return False
-        e = entries[0]
-        return len(e.tokens) > 1 and list(e.want) in ([], [len(e.tokens) - 1])
+        portions = sum(1 for e in entries if len(e.tokens) > 1)
+        if portions == 0 or len(entries) - portions > self.max_singles or any(len(e.want) > 1 for e in entries):
+            return False
+        if portions == 1 and len(entries) == 1:
+            return True                                     # few shapes: every size pays
+        # Steps of several entries come in many shapes. A replay saves host time, which only shows while
+        # the step's kernels take less time than launching them one by one (about 4 ms): beyond that many
+        # rows a capture and the padding cost more than the replays give back.
+        rows = sum(len(e.tokens) for e in entries)
+        return rows <= self.max_mixed_rows
 
     @torch.inference_mode()
     def run(self, entries) -> torch.Tensor | None:
-        """The step's logits ([1, vocab] or [0, vocab]), or None if this shape has no graph yet (the
-        caller then runs the step kernel by kernel)."""
+        """The step's logits [wanted, vocab] in the entries' order, or None if this shape has no graph
+        yet (the caller then runs the step kernel by kernel)."""
         runner = self.runner
-        e = entries[0]
-        T = self.padded_rows(len(e.tokens))
-        key = (T, bool(e.want))
-        slot = self.portions.pop(key, None)
+        key = self.padded_shape(entries)
+        wanted = sum(len(e.want) for e in entries)
+        slot = self.captured.pop(key, None)
         if slot is None:
             self.seen[key] = self.seen.get(key, 0) + 1
-            if self.seen[key] < 2:
+            # a capture costs about as much as ten replays save: a shape of several entries (there are
+            # many of them) has to come back a few times first
+            if self.seen[key] < (2 if len(entries) == 1 else 4):
                 return None
-            slot = _Portion()
-            n_groups = len(runner.pools.groups)
-            n_ints = 3 * T + 2 + 2 + 1 + n_groups * (T + self.W) + 4 * (T // 16)
-            slot.dev = torch.zeros(n_ints, dtype=torch.int32, device=runner.device)
-            step, _ = runner.prepare(entries, into=slot.dev, table_width=self.W, pad_rows_to=T)
+            slot = _Captured()
+            slot.dev = torch.zeros(runner.metadata_ints(key, self.W), dtype=torch.int32, device=runner.device)
+            step, _ = runner.prepare(entries, into=slot.dev, table_width=self.W, shape=key)
             torch.cuda.synchronize()
             side = torch.cuda.Stream()
             side.wait_stream(torch.cuda.current_stream())
@@ -232,11 +256,11 @@ class PortionGraphs:
             with torch.cuda.graph(graph):
                 slot.logits = runner.model.forward(step, runner.pools.views)
             slot.graph = graph
-            while len(self.portions) >= self.max_graphs:    # the least recently used shape gives its memory back
-                self.portions.pop(next(iter(self.portions)))
+            while len(self.captured) >= self.max_graphs:   # the least recently used shape gives its memory back
+                self.captured.pop(next(iter(self.captured)))
         else:
-            runner.prepare(entries, into=slot.dev, table_width=self.W, pad_rows_to=T)
-        self.portions[key] = slot
+            runner.prepare(entries, into=slot.dev, table_width=self.W, shape=key)
+        self.captured[key] = slot
         slot.graph.replay()
         self.replays += 1
-        return slot.logits
+        return slot.logits[:wanted]

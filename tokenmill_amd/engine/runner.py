@@ -46,7 +46,7 @@ class ModelRunner:
         self._copied = torch.cuda.Event()
         self._copy_pending = False
         self.graphs = None                        # DecodeGraphs when the engine runs with --hip-graphs
-        self.portion_graphs = None                # PortionGraphs likewise
+        self.step_graphs = None                # StepGraphs likewise
 
     # ------------------------------------------------------------------------------------------------
 
@@ -59,31 +59,38 @@ class ModelRunner:
         return self._pinned.numpy()
 
     def prepare(self, entries: list[StepEntry], into: torch.Tensor | None = None,
-                table_width: int | None = None, pad_rows_to: int | None = None) -> tuple[StepContext, list[int]]:
+                table_width: int | None = None, shape: tuple[int, int, int, int] | None = None
+                ) -> tuple[StepContext, list[int]]:
         """Flatten the entries into device metadata. Returns the context and, for each wanted logit
         in the caller's order (entries in the given order, ``want`` in its order), its row in the
         step's logits. ``into``: a device int32 buffer to hold the metadata (a captured graph reads
         it at a fixed address; steps of the same shape lay it out the same way); ``table_width``:
-        pad the block tables to this width instead of the widest of the step; ``pad_rows_to`` (a
-        multiple of 16): rows behind the entries' tokens up to this many, so that steps of similar
-        sizes launch the same grids. A padding row is token 0 at position 0 with no cache slot (its
-        keys are not stored) and belongs to no attention tile; every kernel treats rows apart, so
-        what such a row holds reaches no other row. The tile table is filled up to one tile per 16
-        rows with repeats of a real tile, which compute the same rows again."""
+        pad the block tables to this width instead of the widest of the step; ``shape`` = (rows of the
+        prompt portions, portions, single tokens, logit rows): lay the step out with this many of each,
+        so that steps of similar sizes launch the same grids (see ``padded_shape``). What is added:
+        rows behind the portions' tokens and single tokens behind the real ones, each token 0 at
+        position 0 with no cache slot (its keys are not stored) and, for a single token, a context of
+        one key in page 0; portions without tokens; repeats of the first logit row; repeats of a real
+        attention tile (which compute the same rows again). Every kernel treats rows apart, so what a
+        padding row holds reaches no other row. The contexts the launches are sized for are then the
+        longest the model allows."""
         if not entries:
             raise StepError("a step needs at least one entry")
         page = self.page_size
         n_groups = len(self.pools.groups)
         # prompt portions first, single tokens last (the order the attention kernels split on)
         order = sorted(range(len(entries)), key=lambda i: len(entries[i].tokens) == 1)
-        S = len(entries)
-        T_real = sum(len(e.tokens) for e in entries)
-        T = T_real
-        if pad_rows_to is not None:
-            if pad_rows_to < T_real or pad_rows_to % 16:
-                raise StepError(f"{T_real} rows cannot be padded to {pad_rows_to}")
-            T = pad_rows_to
-        R = sum(len(e.want) for e in entries)
+        n_portions = sum(1 for e in entries if len(e.tokens) > 1)
+        n_singles = len(entries) - n_portions
+        Tp_real = sum(len(e.tokens) for e in entries if len(e.tokens) > 1)
+        R_real = sum(len(e.want) for e in entries)
+        Tp, P, ND, R = Tp_real, n_portions, n_singles, R_real
+        if shape is not None:
+            Tp, P, ND, R = shape
+            if Tp < Tp_real or Tp % 16 or P < n_portions or ND < n_singles or R < R_real:
+                raise StepError(f"a step of {(Tp_real, n_portions, n_singles, R_real)} does not fit the shape {shape}")
+        S = P + ND
+        T = Tp + ND
         widths = []
         for e in entries:
             if not e.tokens:
@@ -106,7 +113,7 @@ class ModelRunner:
                 raise StepError(f"block tables of {W} pages do not fit the width {table_width}")
             W = table_width
         n_tiles_real = sum(-(-len(e.tokens) // 16) for e in entries if len(e.tokens) > 1)
-        n_tiles = max(n_tiles_real, T // 16) if (pad_rows_to is not None and n_tiles_real) else n_tiles_real
+        n_tiles = self.padded_tiles(Tp, P) if (shape is not None and n_tiles_real) else n_tiles_real
         n_ints = 3 * T + (S + 1) + 2 * S + max(R, 1) + n_groups * (T + S * W) + 4 * n_tiles
         buf = self._staging(n_ints)
         off = 0
@@ -131,12 +138,21 @@ class ModelRunner:
             g_tab.append(take(S * W))
 
         tiles, tiles_s = take(4 * n_tiles)
+        if shape is not None:                               # what no entry fills is padding
+            ids[:] = 0
+            pos[:] = 0
+            seq_of[:] = 0
+            ctx_lens[:] = 1
+            slots_state[:] = 0
+            rows[:] = 0
+            for g in range(n_groups):
+                g_slot[g][0][:] = -1
+                g_tab[g][0][:] = 0
         tile_i = 0
         row0 = 0
         first_row = [0] * S
         q_lens, starts = [], []
         cu[0] = 0
-        n_portions = sum(1 for e in entries if len(e.tokens) > 1)
         for s, i in enumerate(order[:n_portions]):
             e = entries[i]
             n = len(e.tokens)
@@ -173,10 +189,13 @@ class ModelRunner:
             row0 += n
         # single tokens: the same rows, written with a few bulk assignments instead of a dozen array
         # operations each (a mixed step may hold a hundred of them)
+        cu[n_portions + 1:P + 1] = Tp_real                  # portions without tokens
+        row0 = Tp                                           # the single tokens stand behind the portions' rows
         singles = [entries[i] for i in order[n_portions:]]
+        cu[P + 1:] = np.arange(Tp + 1, Tp + ND + 1)
         if singles:
             n1 = len(singles)
-            s0 = n_portions
+            s0 = P
             toks = np.asarray([e.tokens[0] for e in singles], dtype=np.int64)
             if toks.min() < 0 or toks.max() >= self.vocab:
                 raise StepError(f"a token id is outside the vocabulary of {self.vocab}")
@@ -208,12 +227,6 @@ class ModelRunner:
             q_lens.extend([1] * n1)
             starts.extend(p1)
             row0 += n1
-        if T > T_real:                                                        # padding rows
-            ids[T_real:] = 0
-            pos[T_real:] = 0
-            seq_of[T_real:] = 0
-            for g in range(n_groups):
-                g_slot[g][0][T_real:] = -1
         if n_tiles > n_tiles_real:                                            # repeats of the last real tile
             t = tiles.reshape(n_tiles, 4)
             t[n_tiles_real:] = t[n_tiles_real - 1]
@@ -227,8 +240,10 @@ class ModelRunner:
             for w in e.want:
                 rows[r] = first_row[i] + w
                 r += 1
-        if R == 0:
+        if R_real == 0:
             rows[0] = 0
+        elif R > R_real:
+            rows[R_real:R] = rows[0]
 
         if into is None:
             dev = self._pinned[:off].to(self.device, non_blocking=True)
@@ -249,11 +264,24 @@ class ModelRunner:
             num_tokens=T, num_seqs=S, token_ids=d(ids_s), positions=d(pos_s), seq_of_token=d(seq_s),
             cu_q_lens=d(cu_s), context_lens=d(ctx_s), state_slots=d(st_s), logit_rows=d(rows_s)[:R], groups=groups,
             q_lens=q_lens, start_positions=starts, max_q_len=max(q_lens),
-            max_context_len=max(s0 + n for s0, n in zip(starts, q_lens)), num_logit_rows=R,
-            num_decode=sum(1 for n in q_lens if n == 1),
-            max_decode_context=max([s0 + 1 for s0, n in zip(starts, q_lens) if n == 1], default=0),
+            max_context_len=self.max_positions if shape is not None else max(s0 + n for s0, n in zip(starts, q_lens)),
+            num_logit_rows=R, num_decode=ND,
+            max_decode_context=(self.max_positions if ND else 0) if shape is not None else
+            max([s0 + 1 for s0, n in zip(starts, q_lens) if n == 1], default=0),
             prefill_tiles=d(tiles_s).view(n_tiles, 4))
-        return ctx, list(range(R))
+        return ctx, list(range(R_real))
+
+    @staticmethod
+    def padded_tiles(portion_rows: int, portions: int) -> int:
+        """Tiles of 16 tokens that any ``portions`` portions filling ``portion_rows`` rows can need."""
+        return portion_rows // 16 + portions
+
+    def metadata_ints(self, shape: tuple[int, int, int, int], table_width: int) -> int:
+        """Size of the metadata buffer ``prepare`` fills for a step of this shape."""
+        Tp, P, ND, R = shape
+        S, T = P + ND, Tp + ND
+        return (3 * T + (S + 1) + 2 * S + max(R, 1) + len(self.pools.groups) * (T + S * table_width)
+                + 4 * self.padded_tiles(Tp, P))
 
     @torch.inference_mode()
     def step(self, entries: list[StepEntry]) -> torch.Tensor:
@@ -265,8 +293,8 @@ class ModelRunner:
                 e.cache.fresh = False
         if self.graphs is not None and self.graphs.can_run(entries):
             return self.graphs.run(entries)
-        if self.portion_graphs is not None and self.portion_graphs.can_run(entries):
-            logits = self.portion_graphs.run(entries)
+        if self.step_graphs is not None and self.step_graphs.can_run(entries):
+            logits = self.step_graphs.run(entries)
             if logits is not None:
                 return logits
         ctx, _ = self.prepare(entries)
