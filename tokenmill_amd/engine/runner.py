@@ -273,8 +273,10 @@ class ModelRunner:
 
     @staticmethod
     def padded_tiles(portion_rows: int, portions: int) -> int:
-        """Tiles of 16 tokens that any ``portions`` portions filling ``portion_rows`` rows can need."""
-        return portion_rows // 16 + portions
+        """Tiles of 16 tokens that any ``portions`` portions (or fewer) with at most ``portion_rows`` (a multiple
+        of 16) tokens in all can need: every portion but one may add a tile that is not full. One portion
+        needs no more tiles than its rows: a 2,048-token prompt stays at 128 tiles, a block for every CU."""
+        return portion_rows // 16 + max(portions - 1, 0)
 
     def metadata_ints(self, shape: tuple[int, int, int, int], table_width: int) -> int:
         """Size of the metadata buffer ``prepare`` fills for a step of this shape."""
