@@ -434,6 +434,20 @@ def test_window_groups_a_layer_twice_and_a_shared_cache(tmp_path, dtype_name):
             assert_logits_close(row, want, dt, f"toy window model, {name}, {rid} position {p}")
         session.manager.check_invariants()
         assert not session.manager.live and all(a.num_free == session.num_pages for a in session.manager.allocators)
+    # through the engine: decode steps and mixed steps replayed from graphs give the eager engine's tokens,
+    # with pages of the windowed group handed back under way
+    from tokenmill_amd import EngineConfig, LLMEngine, SamplingParams
+    prompts = [random_ids(n, 150, 450 + i) for i, n in enumerate([40, 3, 27, 55, 18, 33] * 4)]
+    outs = {}
+    for graphs in (False, True):
+        eng = LLMEngine(EngineConfig(model=str(d), dtype=dtype_name, block_size=8, num_blocks=64, max_model_len=128,
+                                     max_num_seqs=4, max_num_batched_tokens=24, enable_chunked_prefill=True,
+                                     watermark=0.0, hip_graphs=graphs))
+        outs[graphs] = eng.generate(prompts, SamplingParams(max_tokens=24, ignore_eos=True))
+        if graphs:
+            assert eng.runner.graphs.replays > 0 and eng.runner.step_graphs.replays > 0
+        assert eng.cache.num_free_pages == eng.cache.num_pages
+    assert outs[True] == outs[False]
 
 
 # ----------------------------------------------------------------------------------------------- routed experts, another position encoding
