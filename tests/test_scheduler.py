@@ -293,3 +293,28 @@ def test_every_page_is_back_after_random_traffic():
         cache.check_invariants()
         steps += 1
     assert not sched.has_unfinished() and cache.num_free_pages == 12 and sched.num_preemptions > 0
+
+
+def test_padded_step_shapes_hold_every_step_they_stand_for():
+    """The shapes that steps are laid out in for graph replay: rows, portions, single tokens and logit rows
+    only grow, the rows by at most an eighth beyond the smallest steps, and the tile bound of a shape covers
+    every set of portions that fits it (every portion but one may leave a tile part empty)."""
+    import random
+    from types import SimpleNamespace
+
+    from tokenmill_amd.engine.graphs import StepGraphs
+    from tokenmill_amd.engine.runner import ModelRunner
+
+    rng = random.Random(0)
+    for _ in range(20000):
+        portions = [rng.choice([2, 3, 15, 16, 17, 18, 31, 32, 33, rng.randint(2, 300)]) for _ in range(rng.randint(1, 12))]
+        singles = rng.randint(0, 40)
+        entries = [SimpleNamespace(tokens=[0] * n, want=[n - 1] if rng.random() < 0.5 else []) for n in portions]
+        entries += [SimpleNamespace(tokens=[0], want=[0]) for _ in range(singles)]
+        rows, P, ND, R = StepGraphs.padded_shape(entries)
+        total = sum(portions)
+        assert rows >= total and rows % 32 == 0 and (rows - total < 32 or rows <= total * 1.125)
+        assert P >= len(portions) and ND >= singles and R >= sum(len(e.want) for e in entries)
+        assert P < 2 * len(portions) and (ND < 2 * singles or singles == 0)
+        assert sum(-(-n // 16) for n in portions) <= ModelRunner.padded_tiles(rows, P)
+    assert ModelRunner.padded_tiles(2048, 1) == 128
