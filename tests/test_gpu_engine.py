@@ -339,3 +339,34 @@ def test_mixed_steps_replayed_from_hip_graphs(model_dirs, plains, dtype_name):
     for p, o in zip(prompts, outs[True]):
         verify(plains["B"], p, o, DTYPES[dtype_name])
     assert outs[True] == outs[False]
+
+
+def test_steps_run_kernel_by_kernel_when_a_capture_fails(model_dirs, plains, monkeypatch):
+    """A capture that fails (out of memory for a graph's activations, in the field; forced from the host here)
+    leaves its steps to the eager path: same tokens, the shape is not tried again, other shapes still replay."""
+    from tokenmill_amd import SamplingParams
+    from tokenmill_amd.engine import graphs as G
+    prompts = [random_ids(n, 384, 800 + i) for i, n in enumerate([20, 19, 35, 18, 5, 40, 22])]
+    sp = SamplingParams(max_tokens=6, ignore_eos=True)
+    want = [make_engine(model_dirs["B"], "float32", block_size=8, max_num_seqs=2, max_model_len=96).generate([p], sp)[0]
+            for p in prompts]
+    decode_capture, step_capture = G.DecodeGraphs._capture, G.StepGraphs._capture
+
+    def failing_decode(self, bk):
+        if bk.B == 1:
+            raise RuntimeError("out of memory (forced)")
+        return decode_capture(self, bk)
+
+    def failing_step(self, entries, key):
+        if key[0] == 32:
+            raise RuntimeError("out of memory (forced)")
+        return step_capture(self, entries, key)
+
+    monkeypatch.setattr(G.DecodeGraphs, "_capture", failing_decode)
+    monkeypatch.setattr(G.StepGraphs, "_capture", failing_step)
+    eng = make_engine(model_dirs["B"], "float32", block_size=8, hip_graphs=True, max_num_seqs=2, max_model_len=96)
+    got = [eng.generate([p], sp)[0] for p in prompts]
+    assert got == want
+    assert eng.runner.graphs.failed == {1} and eng.runner.graphs.replays == 0
+    assert eng.runner.step_graphs.failed == {(32, 1, 0, 1)} and (64, 1, 0, 1) in eng.runner.step_graphs.captured
+    assert eng.cache.num_free_pages == eng.cache.num_pages

@@ -17,12 +17,16 @@ steps of a serving run replay a handful of graphs: ``StepGraphs``.
 """
 from __future__ import annotations
 
+import logging
+
 import numpy as np
 import torch
 
 from tokenmill_amd.cache.manager import RELEASED
 from tokenmill_amd.hip import ops
 from tokenmill_amd.parts.base import GroupStep, StepContext
+
+log = logging.getLogger(__name__)
 
 
 class _Bucket:
@@ -77,6 +81,7 @@ class DecodeGraphs:
         top = min(cfg.max_num_seqs, max_batch)
         self.sizes = [b for b in (1, 2, 4, 8, 16, 32, 64, 128, 256) if b < top] + [top]
         self.buckets: dict[int, _Bucket] = {}
+        self.failed: set[int] = set()                       # bucket sizes whose capture failed: those steps run eagerly
         self.replays = 0
         self._copied = torch.cuda.Event()
 
@@ -91,8 +96,11 @@ class DecodeGraphs:
         return self.buckets[B]
 
     @torch.inference_mode()
-    def run(self, entries) -> torch.Tensor:
-        """Float32 logits [wanted, vocab], entries in the given order (each wants place 0 or nothing)."""
+    def run(self, entries) -> torch.Tensor | None:
+        """Float32 logits [wanted, vocab], entries in the given order (each wants place 0 or nothing); None
+        if the graph of this batch size could not be captured (the caller then runs the step kernel by
+        kernel, as the reference does when it runs out of memory for graphs: reference
+        src/infer/engine/cuda_graphs.py:88-110)."""
         runner = self.runner
         bk = self._bucket(len(entries))
         B, W, page = bk.B, bk.W, self.page
@@ -141,7 +149,15 @@ class DecodeGraphs:
         bk.dev.copy_(bk.pinned, non_blocking=True)
         self._copied.record()
         if bk.graph is None:
-            self._capture(bk)
+            if bk.B in self.failed:
+                return None
+            try:
+                self._capture(bk)
+            except RuntimeError as e:                       # out of memory for the graph's activations, mostly
+                self.failed.add(bk.B)
+                bk.graph = None
+                log.warning("no graph for decode steps of %d requests (%s); they run kernel by kernel", bk.B, e)
+                return None
         bk.graph.replay()
         self.replays += 1
         wanted = [i for i, e in enumerate(entries) if e.want]
@@ -194,6 +210,7 @@ class StepGraphs:
         self.max_mixed_rows = 1024
         self.seen: dict[tuple, int] = {}
         self.captured: dict[tuple, _Captured] = {}         # insertion order = least recently used first
+        self.failed: set[tuple] = set()                     # shapes whose capture failed: those steps run eagerly
         self.replays = 0
 
     @staticmethod
@@ -239,23 +256,14 @@ class StepGraphs:
             self.seen[key] = self.seen.get(key, 0) + 1
             # a capture costs about as much as ten replays save: a shape of several entries (there are
             # many of them) has to come back a few times first
-            if self.seen[key] < (2 if len(entries) == 1 else 4):
+            if self.seen[key] < (2 if len(entries) == 1 else 4) or key in self.failed:
                 return None
-            slot = _Captured()
-            slot.dev = torch.zeros(runner.metadata_ints(key, self.W), dtype=torch.int32, device=runner.device)
-            step, _ = runner.prepare(entries, into=slot.dev, table_width=self.W, shape=key)
-            torch.cuda.synchronize()
-            side = torch.cuda.Stream()
-            side.wait_stream(torch.cuda.current_stream())
-            # a first run outside the graph: lazy set-up happens here, and the library's products are timed now
-            with torch.cuda.stream(side), ops.gemm_library_tune_at_once():
-                runner.model.forward(step, runner.pools.views)
-            torch.cuda.current_stream().wait_stream(side)
-            torch.cuda.synchronize()
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                slot.logits = runner.model.forward(step, runner.pools.views)
-            slot.graph = graph
+            try:
+                slot = self._capture(entries, key)
+            except RuntimeError as e:
+                self.failed.add(key)
+                log.warning("no graph for steps of shape %s (%s); they run kernel by kernel", key, e)
+                return None
             while len(self.captured) >= self.max_graphs:   # the least recently used shape gives its memory back
                 self.captured.pop(next(iter(self.captured)))
         else:
@@ -264,3 +272,25 @@ class StepGraphs:
         slot.graph.replay()
         self.replays += 1
         return slot.logits[:wanted]
+
+    @torch.inference_mode()
+    def _capture(self, entries, key) -> _Captured:
+        """A first run of the step outside the graph, then the capture; the step's metadata lie in the
+        buffer the graph reads."""
+        runner = self.runner
+        slot = _Captured()
+        slot.dev = torch.zeros(runner.metadata_ints(key, self.W), dtype=torch.int32, device=runner.device)
+        step, _ = runner.prepare(entries, into=slot.dev, table_width=self.W, shape=key)
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        # a first run outside the graph: lazy set-up happens here, and the library's products are timed now
+        with torch.cuda.stream(side), ops.gemm_library_tune_at_once():
+            runner.model.forward(step, runner.pools.views)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            slot.logits = runner.model.forward(step, runner.pools.views)
+        slot.graph = graph
+        return slot

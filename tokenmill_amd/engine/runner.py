@@ -294,7 +294,9 @@ class ModelRunner:
                 self.pools.reset_state_slot(e.cache.state_slot)
                 e.cache.fresh = False
         if self.graphs is not None and self.graphs.can_run(entries):
-            return self.graphs.run(entries)
+            logits = self.graphs.run(entries)
+            if logits is not None:
+                return logits
         if self.step_graphs is not None and self.step_graphs.can_run(entries):
             logits = self.step_graphs.run(entries)
             if logits is not None:
