@@ -35,7 +35,8 @@ def main(argv=None) -> int:
     parser.add_argument("--temperature", type=float, default=0.0)
     parser.add_argument("--top-k", type=int, default=-1)
     parser.add_argument("--top-p", type=float, default=1.0)
-    parser.add_argument("--sample-seed", type=int, default=None)
+    parser.add_argument("--sample-seed", type=int, default=None,
+                        help="seed of the sampling streams: prompt i uses seed + i (default: drawn from --seed)")
     parser.add_argument("--ignore-eos", action="store_true")
     parser.add_argument("--log-level", default="warning")
     args = parser.parse_args(argv)
@@ -68,8 +69,11 @@ def main(argv=None) -> int:
         g = torch.Generator().manual_seed(args.prompt_seed)
         vocab = engine.runner.vocab
         prompts = [torch.randint(0, vocab, (int(n),), generator=g).tolist() for n in args.prompt_lens.split(",")]
-    params = SamplingParams(max_tokens=args.max_tokens, temperature=args.temperature, top_k=args.top_k,
-                            top_p=args.top_p, seed=args.sample_seed, ignore_eos=args.ignore_eos)
+    # prompt i draws from the stream of seed + i (one seed for all would give every prompt the same draws);
+    # without a seed the engine draws one per request from its own generator (--seed)
+    params = [SamplingParams(max_tokens=args.max_tokens, temperature=args.temperature, top_k=args.top_k,
+                             top_p=args.top_p, seed=None if args.sample_seed is None else args.sample_seed + i,
+                             ignore_eos=args.ignore_eos) for i in range(len(prompts))]
     outputs = engine.generate(prompts, params)
     for i, (p, o) in enumerate(zip(prompts, outputs)):
         print(json.dumps({"prompt": i, "prompt_tokens": len(p), "output_ids": o}))
