@@ -79,7 +79,9 @@ class DecodeGraphs:
         self.max_positions = runner.max_positions
         self.W = -(-runner.max_positions // self.page)
         top = min(cfg.max_num_seqs, max_batch)
-        self.sizes = [b for b in (1, 2, 4, 8, 16, 32, 64, 128, 256) if b < top] + [top]
+        # batch sizes a step is padded to: powers of two and the sizes in between from 16 on (48 keeps 33 to 48
+        # requests on the products that hold the input in LDS, which 64 rows leave)
+        self.sizes = [b for b in (1, 2, 4, 8, 16, 24, 32, 48, 64, 96, 128, 192, 256) if b < top] + [top]
         self.buckets: dict[int, _Bucket] = {}
         self.failed: set[int] = set()                       # bucket sizes whose capture failed: those steps run eagerly
         self.replays = 0
