@@ -117,7 +117,7 @@ def main() -> int:
         sp = SamplingParams(max_tokens=steps + warmup + 8, ignore_eos=True)
         for i, p in enumerate(prompts(batch)):
             eng.add_request(f"d{i}", p, sp)
-        while eng.scheduler.waiting or any(s.num_new_tokens > 1 for s in eng.scheduler.running):
+        while eng.scheduler.queue or any(r.pending > 1 for r in eng.scheduler.live):
             eng.step()                                   # prefills (one prompt a step: budget = 2,048 tokens)
         for _ in range(warmup):
             eng.step()
@@ -129,7 +129,7 @@ def main() -> int:
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         context = prompt_len + warmup + steps // 2
-        for s in list(eng.seqs):
+        for s in list(eng.requests):
             eng.abort_request(s)
         del eng
         return dt / steps, context

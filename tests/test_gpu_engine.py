@@ -54,8 +54,8 @@ def test_greedy_generation_whole_prompts(model_dirs, plains, dtype_name):
     assert [len(o) for o in outs] == [16, 16, 16]
     flips = sum(verify(plains["A"], p, o, DTYPES[dtype_name]) for p, o in zip(prompts, outs))
     assert flips == 0 or dtype_name == "bfloat16"
-    assert not eng.scheduler.running and eng.cache.num_free_pages == eng.cache.num_pages
-    assert eng.stats["prefill_steps"] == 1 and eng.stats["decode_steps"] == 15
+    assert not eng.scheduler.live and eng.cache.num_free_pages == eng.cache.num_pages
+    assert eng.stats["prompt_steps"] == 1 and eng.stats["decode_steps"] == 15 and eng.stats["tokens_out"] == 48
 
 
 @pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
@@ -97,8 +97,8 @@ def test_same_tokens_under_every_cutting_and_a_starved_pool(model_dirs, plains, 
     starved = make_engine(model_dirs["C"], dtype_name, block_size=4, kv_cache_mb=None, num_blocks=40,
                           enable_chunked_prefill=chunked, max_num_batched_tokens=12 if chunked else 512)
     outs = starved.generate(prompts, sp)
-    assert starved.scheduler.num_preemptions > 0
-    assert starved.cache.num_free_pages == starved.cache.num_pages and not starved.scheduler.running
+    assert starved.scheduler.evictions > 0
+    assert starved.cache.num_free_pages == starved.cache.num_pages and not starved.scheduler.live
     starved.cache.check_invariants()
     for p, o in zip(prompts, outs):
         assert len(o) == 24
@@ -161,7 +161,7 @@ def test_stop_rules_abort_and_rejections(model_dirs):
     s = eng.add_request("long", random_ids(35, 256, 71), SamplingParams(max_tokens=100, ignore_eos=True))
     while eng.has_unfinished():
         eng.step()
-    assert s.finish_reason == "length" and s.length == 40
+    assert s.why_done == "length" and s.n_tokens == 40
     # an end-of-sequence token stops with "stop" and stays in the output
     eng.eos_ids = {free_run[4]}
     stopped = eng.generate([prompt], SamplingParams(max_tokens=12))[0]
@@ -255,7 +255,7 @@ def test_decode_steps_replayed_from_hip_graphs(model_dirs, plains, dtype_name):
         seqs += [eng.add_request(f"r{i + 4}", p, sp) for i, (p, sp) in enumerate(zip(prompts[4:], params[4:]))]
         while eng.has_unfinished():
             eng.step()
-        outs[graphs] = [s.output_ids for s in seqs]
+        outs[graphs] = [s.generated for s in seqs]
         if graphs:
             assert eng.runner.graphs.replays > 20 and len(eng.runner.graphs.buckets) >= 3
         assert eng.cache.num_free_pages == eng.cache.num_pages

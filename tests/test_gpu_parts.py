@@ -166,6 +166,7 @@ def test_attention_part_whole_then_portions_then_tokens(dt, H, KVH, D, window):
     attn = GQAttention(hidden, H, KVH, D, D ** -0.5, rope, window=window, names=("q_proj", "k_proj", "v_proj", "o_proj"))
     t = attention_tensors(hidden, H, KVH, D, dt)
     attn.load({k: v.to(dt).to(DEV) for k, v in t.items()}, "a.")
+    attn.prepare(pack_weights=True)
     x = q(torch.randn(L, hidden), dt)
     cfg = {"heads": H, "kv_heads": KVH, "head_dim": D}
     cos, sin = P.rope_tables(L, D, theta)
@@ -207,6 +208,7 @@ def test_feed_forward_part(dt):
          "m.down_proj.weight": q(torch.randn(hidden, inter) * 0.2, dt)}
     assert set(ffn.tensor_specs("m.")) == set(t)
     ffn.load({k: v.to(dt).to(DEV) for k, v in t.items()}, "m.")
+    ffn.prepare(pack_weights=True)
     for M in (4, 90):
         x = q(torch.randn(M, hidden), dt)
         got = ffn.forward(x.to(dt).to(DEV)).float().cpu()
@@ -546,6 +548,10 @@ def build_toy_routed_model(cfg: ToyRoutedConfig, max_positions=None):
         def load(self, tensors, prefix):
             for part, p in self._parts(prefix):
                 part.load(tensors, p)
+
+        def prepare(self, pack_weights):
+            for expert in self.experts:
+                expert.prepare(pack_weights)
 
         def forward(self, x, step, residual=None):
             x = as_tensor(x)

@@ -1,55 +1,39 @@
-"""The continuous-batching engine: add_request / step / abort_request / generate (reference
-src/infer/engine/engine.py:87-281). Every step re-plans the batch, so new requests join at the
-next step and finished ones leave at once. Token ids in, token ids out.
+"""The generation loop. Token ids in, token ids out.
+
+``LLMEngine`` has the reference's five calls (``add_request``, ``step``, ``abort_request``,
+``has_unfinished``, ``generate``; reference src/infer/engine/engine.py:87-281). One ``step`` is: the
+scheduler plans a batch (which is already the list of entries the step function takes), the step
+function returns the logits at the rows that end a request's known tokens, the sampler turns them
+into one token each, and the requests are advanced: a request joins at the next plan after it was
+added and leaves in the step that ends it.
 """
 from __future__ import annotations
 
 import logging
 import random
 import time
-
-import torch
+from collections import deque
 
 from tokenmill_amd.cache.manager import CacheManager
 from tokenmill_amd.cache.pool import CachePools
 from tokenmill_amd.config.engine_config import EngineConfig
 from tokenmill_amd.engine.loading import load_model, resolve_device, resolve_dtype
-from tokenmill_amd.engine.runner import ModelRunner, StepEntry
-from tokenmill_amd.engine.scheduler import Scheduler
-from tokenmill_amd.engine.sequence import RequestOutput, Sequence
+from tokenmill_amd.engine.request import Request, RequestOutput
+from tokenmill_amd.engine.runner import ModelRunner
+from tokenmill_amd.engine.scheduler import Scheduler, StepPlan
+from tokenmill_amd.engine.sizing import num_cache_pages
 from tokenmill_amd.sampling.sampler import Sampler, SamplingParams
 
 log = logging.getLogger("tokenmill_amd.engine")
 
+TUNE_CANDIDATES = 16        # library algorithms timed per shape with tune_gemm
+STEP_TIMES_KEPT = 8192      # most recent step times kept for a histogram
+
+DOES_NOT_FIT = "prompt does not fit in the KV cache"
+
 
 class RequestRejected(ValueError):
-    """The request can never be served (for example, its prompt is longer than max_model_len)."""
-
-
-def num_cache_pages(cfg: EngineConfig, model, dtype, device, peak_bytes: int) -> int:
-    """Pages per layer group: --num-blocks, else --kv-cache-mb, else what is left of
-    GPU memory x utilization after weights and peak activations (reference
-    src/infer/engine/engine.py:44-84)."""
-    if cfg.num_blocks is not None:
-        pages = cfg.num_blocks
-    else:
-        per_page = CachePools.bytes_per_token(model, dtype) * cfg.block_size
-        if cfg.kv_cache_mb is not None:
-            budget = int(cfg.kv_cache_mb * 2**20)
-        else:
-            total = torch.cuda.get_device_properties(device).total_memory
-            budget = int(total * cfg.gpu_memory_utilization) - peak_bytes
-            if budget <= 0:
-                raise RuntimeError("no memory left for the cache; lower --max-batched-tokens or raise utilization")
-        pages = budget // max(per_page, 1)
-        # no request can use more than max_num_seqs * max_model_len tokens
-        pages = min(pages, cfg.max_num_seqs * (-(-cfg.max_model_len // cfg.block_size)))
-    if pages < 2:
-        raise RuntimeError("cache budget too small for the paged pool")
-    return int(pages)
-
-
-TUNE_CANDIDATES = 16        # library algorithms timed per shape with tune_gemm
+    """The request can never be served as given (empty, too long, a token outside the vocabulary, an id in use)."""
 
 
 class LLMEngine:
@@ -67,8 +51,7 @@ class LLMEngine:
             from tokenmill_amd.hip import ops
             ops.gemm_library_tune(TUNE_CANDIDATES)
         self.eos_ids = set(getattr(model.config, "eos_token_ids", ()) or ())
-        peak = self._profile_peak_memory() if (cfg.num_blocks is None and cfg.kv_cache_mb is None) else 0
-        pages = num_cache_pages(cfg, model, self.dtype, self.device, peak)
+        pages = num_cache_pages(cfg, model, self.dtype, self.device)
         self.pools = CachePools(model, pages, cfg.block_size, cfg.max_num_seqs, self.dtype, self.device)
         self.cache = CacheManager(self.pools.windows, pages, cfg.block_size, cfg.max_num_seqs, cfg.watermark)
         self.runner = ModelRunner(model, self.pools, max_positions=cfg.max_model_len)
@@ -78,164 +61,126 @@ class LLMEngine:
             self.runner.step_graphs = StepGraphs(self.runner)
         self.scheduler = Scheduler(cfg, self.cache)
         self.sampler = Sampler(self.device)
-        self.seqs: dict[str, Sequence] = {}
-        self._rng = random.Random(cfg.seed)
-        self._offline_counter = 0
-        self.stats = {"steps": 0, "peak_running": 0, "prefill_steps": 0, "decode_steps": 0,
-                      "generated_tokens": 0, "busy_time": 0.0}
-        log.info("engine ready: %d pages of %d tokens per group (%.0f MiB), dtype %s, device %s", pages,
-                 cfg.block_size, self.pools.nbytes / 2**20, self.dtype, self.device)
+        self.requests: dict[str, Request] = {}           # every request that has not ended
+        self._seeds = random.Random(cfg.seed)            # stream seeds of requests that bring none
+        self._generate_calls = 0
+        self.stats = {"steps": 0, "prompt_steps": 0, "decode_steps": 0, "mixed_steps": 0, "tokens_out": 0,
+                      "tokens_in": 0, "busy_s": 0.0, "peak_live": 0}
+        self.step_seconds: deque[float] = deque(maxlen=STEP_TIMES_KEPT)
+        log.info("engine ready: %d pages of %d tokens per layer group (%.0f MiB), %s on %s", pages, cfg.block_size,
+                 self.pools.nbytes / 2**20, self.dtype, self.device)
 
-    def _profile_peak_memory(self) -> int:
-        """One dummy step at the largest batch the scheduler will build; returns the peak bytes the
-        allocator needed, weights included (reference src/infer/engine/model_runner.py:99-118)."""
-        cfg = self.cfg
-        n = cfg.max_num_batched_tokens
-        seg = min(n, cfg.max_model_len)
-        segs = [seg] * (n // seg) + ([n % seg] if n % seg else [])
-        pages = sum(-(-s // cfg.block_size) for s in segs)
-        pools = CachePools(self.model, pages, cfg.block_size, len(segs), self.dtype, self.device)
-        manager = CacheManager(pools.windows, pages, cfg.block_size, len(segs))
-        runner = ModelRunner(self.model, pools, max_positions=cfg.max_model_len)
-        torch.cuda.synchronize(self.device)
-        pool_bytes = pools.nbytes
-        torch.cuda.reset_peak_memory_stats(self.device)
-        entries = [StepEntry(manager.allocate(f"profile-{i}", s), 0, [0] * s, [s - 1]) for i, s in enumerate(segs)]
-        runner.step(entries)
-        torch.cuda.synchronize(self.device)
-        peak = torch.cuda.max_memory_allocated(self.device) - pool_bytes
-        del runner, pools, entries
-        torch.cuda.empty_cache()
-        return max(peak, 0)
-
-    # --- requests -----------------------------------------------------------------------------------------
+    # --- requests ---------------------------------------------------------------------------------
 
     def add_request(self, request_id: str, prompt_ids: list[int], params: SamplingParams,
-                    arrival_time: float | None = None) -> Sequence:
+                    arrival_time: float | None = None) -> Request:
+        vocab, limit = self.runner.vocab, self.cfg.max_model_len
+        if request_id in self.requests:
+            raise RequestRejected(f"request id {request_id!r} is in use")
         if not prompt_ids:
-            raise RequestRejected("prompt is empty")
-        if len(prompt_ids) >= self.cfg.max_model_len:
-            raise RequestRejected(f"prompt has {len(prompt_ids)} tokens; max_model_len is {self.cfg.max_model_len}")
-        if request_id in self.seqs:
-            raise RequestRejected(f"duplicate request id {request_id}")
-        vocab = self.runner.vocab
+            raise RequestRejected("the prompt is empty")
+        if len(prompt_ids) >= limit:
+            raise RequestRejected(f"the prompt has {len(prompt_ids)} tokens and max_model_len is {limit}: "
+                                  "no room for a generated token")
         if min(prompt_ids) < 0 or max(prompt_ids) >= vocab:
-            raise RequestRejected(f"a prompt token is outside the vocabulary of {vocab}")
-        seq = Sequence(request_id, list(prompt_ids), params,
-                       arrival_time=time.monotonic() if arrival_time is None else arrival_time)
-        seq.sample_seed = params.seed if params.seed is not None else self._rng.getrandbits(62)
-        self.seqs[request_id] = seq
-        self.scheduler.add(seq)
-        return seq
+            raise RequestRejected(f"the prompt holds a token outside the vocabulary of {vocab}")
+        seed = params.seed if params.seed is not None else self._seeds.getrandbits(62)
+        req = Request(request_id, prompt_ids, params, seed,
+                      time.monotonic() if arrival_time is None else arrival_time)
+        self.requests[request_id] = req
+        self.scheduler.enqueue(req)
+        return req
 
     def abort_request(self, request_id: str, reason: str = "abort") -> RequestOutput | None:
-        seq = self.seqs.pop(request_id, None)
-        if seq is None:
+        req = self.requests.get(request_id)
+        if req is None:
             return None
-        self.scheduler.finish(seq, reason)
-        seq.finish_time = time.monotonic()
-        return self._output(seq, [])
+        self._end(req, reason, time.monotonic())
+        return RequestOutput(req, [])
 
     def has_unfinished(self) -> bool:
-        return self.scheduler.has_unfinished()
+        return self.scheduler.busy()
 
     @property
     def num_waiting(self) -> int:
-        return len(self.scheduler.waiting)
+        return len(self.scheduler.queue)
 
-    # --- one step --------------------------------------------------------------------------------------------
+    @property
+    def num_running(self) -> int:
+        return len(self.scheduler.live)
+
+    def _end(self, req: Request, why: str, now: float, error: str | None = None) -> None:
+        self.scheduler.retire(req, why)
+        req.t_done, req.error = now, error
+        self.requests.pop(req.id, None)
+
+    # --- one step -----------------------------------------------------------------------------------
 
     def step(self) -> list[RequestOutput]:
-        outputs: list[RequestOutput] = []
-        t0 = time.perf_counter()
-        plan = self.scheduler.schedule()
-        for seq in plan.ignored:                          # can never fit in the cache
-            self.seqs.pop(seq.id, None)
-            self.scheduler.finish(seq, "length")
-            seq.finish_time = time.monotonic()
-            outputs.append(self._output(seq, [], error=None if seq.output_ids else
-                                        "prompt does not fit in the KV cache"))
-        if plan.empty:
-            return outputs
-        n_prefill_tokens = plan.num_prefill_tokens
-        sampled, tokens = self._execute(plan)
+        started = time.perf_counter()
+        plan = self.scheduler.plan()
+        out: list[RequestOutput] = []
+        for req in plan.unfit:
+            # an evicted request that has grown past the pool ends with what it has; a fresh one with an error
+            self._end(req, "length", time.monotonic(), None if req.n_generated else DOES_NOT_FIT)
+            out.append(RequestOutput(req, []))
+        if not plan:
+            return out
+        logits = self.runner.step(plan.entries)
+        winners = [plan.owners[i] for i in plan.yields]
+        tokens = self.sampler.sample(logits, [r.params for r in winners], [r.stream_seed for r in winners],
+                                     [r.n_generated for r in winners]) if winners else []
         now = time.monotonic()
-        for seq in plan.prefill_seqs:                     # a portion may cover only part of the prompt
-            seq.num_computed_tokens += plan.chunk(seq)
-        for seq in plan.decode_seqs:
-            seq.num_computed_tokens = seq.length
-        for seq in plan.seqs:
-            self.cache.release_behind_window(seq.cache, seq.num_computed_tokens)
-        for seq, tok in zip(sampled, tokens):
-            seq.output_ids.append(tok)
-            if seq.first_token_time is None:
-                seq.first_token_time = now
-            reason = self._stop_reason(seq, tok)
-            if reason:
-                self.scheduler.finish(seq, reason)
-                seq.finish_time = now
-                self.seqs.pop(seq.id, None)
-            outputs.append(self._output(seq, [tok]))
-        self._record_step(plan, n_prefill_tokens, time.perf_counter() - t0, len(sampled))
-        return outputs
+        release = self.cache.release_behind_window
+        for req, entry in zip(plan.owners, plan.entries):
+            req.cached += len(entry.tokens)
+            release(req.cache, req.cached)
+        for req, token in zip(winners, tokens):
+            req.tokens.append(token)
+            if req.t_first_token is None:
+                req.t_first_token = now
+            why = self._why_stop(req, token)
+            if why is not None:
+                self._end(req, why, now)
+            out.append(RequestOutput(req, [token]))
+        self._account(plan, len(tokens), time.perf_counter() - started)
+        return out
 
-    def _execute(self, plan) -> tuple[list[Sequence], list[int]]:
-        """The plan as one batch through the step function; samples one token for every decode and
-        for every portion that holds its request's last known token (reference
-        src/infer/engine/model_runner.py:76-97)."""
-        entries, sampled = [], []
-        for seq in plan.prefill_seqs:
-            start = seq.num_computed_tokens
-            n = plan.chunk(seq)
-            done = start + n == seq.length
-            entries.append(StepEntry(seq.cache, start, seq.all_token_ids[start:start + n], [n - 1] if done else []))
-            if done:
-                sampled.append(seq)
-        for seq in plan.decode_seqs:
-            entries.append(StepEntry(seq.cache, seq.length - 1, [seq.last_token], [0]))
-            sampled.append(seq)
-        logits = self.runner.step(entries)
-        if not sampled:
-            return [], []
-        tokens = self.sampler.sample(logits, [s.params for s in sampled], [s.sample_seed for s in sampled],
-                                     [s.num_output_tokens for s in sampled])
-        return sampled, tokens
-
-    def _stop_reason(self, seq: Sequence, tok: int) -> str | None:
-        if tok in self.eos_ids and not seq.params.ignore_eos:
+    def _why_stop(self, req: Request, token: int) -> str | None:
+        """"stop" at an end-of-sequence token (which stays in the output), "length" at the request's or the
+        model's limit (reference src/infer/engine/engine.py:206-216)."""
+        if token in self.eos_ids and not req.params.ignore_eos:
             return "stop"
-        if seq.num_output_tokens >= seq.params.max_tokens or seq.length >= self.cfg.max_model_len:
+        if req.n_generated >= req.params.max_tokens or req.n_tokens >= self.cfg.max_model_len:
             return "length"
         return None
 
-    def _output(self, seq: Sequence, new_tokens: list[int], error: str | None = None) -> RequestOutput:
-        return RequestOutput(seq.id, new_tokens, seq.is_finished, seq.finish_reason, seq.num_prompt_tokens,
-                             seq.num_output_tokens, seq.arrival_time, seq.first_token_time, seq.finish_time,
-                             seq.num_preemptions, error)
-
-    def _record_step(self, plan, n_prefill_tokens: int, step_time: float, n_generated: int) -> None:
+    def _account(self, plan: StepPlan, n_out: int, seconds: float) -> None:
         s = self.stats
+        n_decode, n_prompt = plan.n_decode, plan.n_prompt_tokens
         s["steps"] += 1
-        s["busy_time"] += step_time
-        s["prefill_steps" if plan.prefill_seqs else "decode_steps"] += 1
-        s["generated_tokens"] += n_generated
-        running = len(self.scheduler.running)
-        s["peak_running"] = max(s["peak_running"], running)
+        s["mixed_steps" if n_decode and n_prompt else ("decode_steps" if n_decode else "prompt_steps")] += 1
+        s["tokens_out"] += n_out
+        s["tokens_in"] += n_prompt + n_decode
+        s["busy_s"] += seconds
+        s["peak_live"] = max(s["peak_live"], len(plan.entries))
+        self.step_seconds.append(seconds)
         if self.cfg.debug_steps:
-            log.info("step=%d batch=%d prefill_tokens=%d decode_tokens=%d step_ms=%.2f kv_usage=%.3f "
-                     "waiting=%d running=%d preempted=%d", s["steps"], len(plan.seqs), n_prefill_tokens,
-                     len(plan.decode_seqs), step_time * 1e3, self.cache.usage(), len(self.scheduler.waiting),
-                     running, len(plan.preempted))
+            log.info("step %d: %d entries (%d prompt tokens + %d decodes) in %.2f ms; cache %.1f%% used; "
+                     "%d queued, %d live, %d evicted", s["steps"], len(plan.entries), n_prompt, n_decode,
+                     seconds * 1e3, 100 * self.cache.usage(), len(self.scheduler.queue), len(self.scheduler.live),
+                     len(plan.evicted))
 
-    # --- offline helper -----------------------------------------------------------------------------------------
+    # --- all at once ---------------------------------------------------------------------------------
 
     def generate(self, prompts: list[list[int]], params: SamplingParams | list[SamplingParams]) -> list[list[int]]:
-        """Run every prompt to completion through the step loop; returns output token ids in order."""
-        plist = params if isinstance(params, list) else [params] * len(prompts)
-        seqs = []
-        for p, sp in zip(prompts, plist):
-            self._offline_counter += 1
-            seqs.append(self.add_request(f"offline-{self._offline_counter}", p, sp))
-        while self.has_unfinished():
+        """Every prompt to its end through the step loop; the generated ids, in the prompts' order."""
+        each = params if isinstance(params, list) else [params] * len(prompts)
+        if len(each) != len(prompts):
+            raise ValueError(f"{len(prompts)} prompts but {len(each)} sampling parameters")
+        self._generate_calls += 1
+        reqs = [self.add_request(f"generate-{self._generate_calls}-{i}", p, sp)
+                for i, (p, sp) in enumerate(zip(prompts, each))]
+        while self.scheduler.busy():
             self.step()
-        return [s.output_ids for s in seqs]
+        return [r.generated for r in reqs]

@@ -25,16 +25,6 @@ def resolve_device(name: str) -> torch.device:
     return torch.device("cuda:0" if name == "auto" else name)
 
 
-def _load(model, tensors, dtype, device, pack_weights: bool) -> None:
-    from tokenmill_amd.parts.linear import Linear
-    before = Linear.keep_packed_copy
-    Linear.keep_packed_copy = pack_weights
-    try:
-        model.load(tensors, dtype, device)
-    finally:
-        Linear.keep_packed_copy = before
-
-
 def load_model(model_dir: str | Path, dtype: torch.dtype, device: torch.device, max_positions: int | None = None,
                pack_weights: bool = True):
     """The model that config.json names, with its weights on ``device``. ``pack_weights``: keep a second
@@ -42,7 +32,7 @@ def load_model(model_dir: str | Path, dtype: torch.dtype, device: torch.device, 
     arch, cfg = load_config(model_dir)
     model = arch.build_model(cfg, max_positions)
     tensors = read_checkpoint(model_dir, model.tensor_specs(), dtype, device, model.ignorable)
-    _load(model, tensors, dtype, device, pack_weights)
+    model.load(tensors, dtype, device, pack_weights=pack_weights)
     return model
 
 
@@ -70,5 +60,5 @@ def load_random_model(config: dict, seed: int, dtype: torch.dtype, device: torch
         else:
             t = torch.randn(spec.shape, generator=g, dtype=torch.float32, device=device) * std
         tensors[name] = t if spec.kind == "int" else t.to(storage_dtype(torch.bfloat16, spec.kind, dtype))
-    _load(model, tensors, dtype, device, pack_weights)
+    model.load(tensors, dtype, device, pack_weights=pack_weights)
     return model

@@ -1,19 +1,24 @@
-"""Decides, every step, which requests run a portion of their prompt, which decode one token, and
-who is preempted. It never touches the GPU.
+"""Plans one step: which requests run how many of their tokens, and who has to give pages back.
+Host only; the plan it returns is already the batch the step function takes.
 
-The decisions are the reference's (reference src/infer/engine/scheduler.py:29-242):
+Rules (the reference's decisions, reference src/infer/engine/scheduler.py:95-242; its scenarios are
+the vectors of tests/test_scheduler.py):
 
-* FCFS admission without skipping ahead, under the token budget, the cap on running requests and
-  the cache manager's watermark; a prompt larger than the whole budget runs alone.
-* Not chunked (default): a step is either whole-prompt prefills or decodes. ``prefill_first`` runs
-  a prefill step whenever the head of the queue can be admitted; ``decode_first`` only when nothing
-  runs or after ``max_waiting_steps`` decode steps.
-* Chunked (``enable_chunked_prefill``): every running request that is fully prefilled decodes; the
-  budget left goes to prompts already part-way, oldest first, then to new admissions; a prompt is
-  cut where the budget ends.
-* When pages run out (only decode growth can hit that): the most recently admitted request that
-  has not been served this step is preempted, its pages are given back, it goes to the FRONT of the
-  waiting queue and is recomputed from its prompt plus what it generated.
+* The queue is served first come, first served, and nobody overtakes: if the head cannot have its
+  pages now, nothing behind it is looked at. A head that could not fit an empty pool is handed
+  back as ``unfit``.
+* Admission takes pages for every token the request has (prompt and, after an eviction, what it
+  had generated), under the cache manager's watermark and the cap on live requests.
+* A step runs at most ``max_num_batched_tokens`` tokens. Whole-prompt mode (default): a step is
+  prompts only or decodes only; a prompt that does not fit what is left of the budget waits,
+  except that the first prompt of a step always runs. Mixed mode (``enable_chunked_prefill``):
+  every live request that has one token pending decodes, the budget left goes to prompts that are
+  part-way, oldest first, then to the queue; a prompt is cut where the budget ends.
+* ``prefill_first`` plans a prompt step whenever the queue's head can be admitted; ``decode_first``
+  only when nothing is live or after ``max_waiting_steps`` decode steps with someone waiting.
+* Pages run out only when a decoding request crosses a page edge. Then the most recently admitted
+  request that this plan has not served yet gives everything back (the request itself if it is the
+  last one), and returns to the FRONT of the queue with nothing cached.
 """
 from __future__ import annotations
 
@@ -22,193 +27,179 @@ from dataclasses import dataclass, field
 
 from tokenmill_amd.cache.manager import AllocStatus, CacheManager
 from tokenmill_amd.config.engine_config import EngineConfig
-from tokenmill_amd.engine.sequence import Sequence, Status
+from tokenmill_amd.engine.request import Phase, Request
+from tokenmill_amd.engine.runner import StepEntry
 
 
 @dataclass
-class SchedulerOutput:
-    prefill_seqs: list[Sequence] = field(default_factory=list)
-    decode_seqs: list[Sequence] = field(default_factory=list)
-    preempted: list[Sequence] = field(default_factory=list)
-    ignored: list[Sequence] = field(default_factory=list)         # can never fit in the cache
-    prefill_chunks: dict = field(default_factory=dict)            # chunked prefill: tokens this step
-    num_batched_tokens: int = 0
+class StepPlan:
+    """A step, as the step function takes it, and what the planning did on the side."""
+    entries: list[StepEntry] = field(default_factory=list)     # the n_decode decoding requests first, then prompts
+    owners: list[Request] = field(default_factory=list)        # owners[i] runs entries[i]
+    yields: list[int] = field(default_factory=list)            # entries whose last row gives the owner's next token
+    evicted: list[Request] = field(default_factory=list)       # gave their pages back, newest first
+    unfit: list[Request] = field(default_factory=list)         # can never be admitted
+    n_decode: int = 0                                          # entries that are one pending token of a live request
 
-    def chunk(self, seq: Sequence) -> int:
-        """Tokens a prefilling request computes this step."""
-        return self.prefill_chunks.get(seq, seq.num_new_tokens)
-
-    @property
-    def seqs(self) -> list[Sequence]:
-        return self.prefill_seqs + self.decode_seqs
+    def __bool__(self) -> bool:
+        return bool(self.entries)
 
     @property
-    def empty(self) -> bool:
-        return not self.prefill_seqs and not self.decode_seqs
+    def n_tokens(self) -> int:
+        return sum(len(e.tokens) for e in self.entries)
 
     @property
-    def num_prefill_tokens(self) -> int:
-        return sum(self.chunk(s) for s in self.prefill_seqs)
+    def n_prompt_tokens(self) -> int:
+        return self.n_tokens - self.n_decode
+
+    @property
+    def decoders(self) -> list[Request]:
+        return self.owners[:self.n_decode]
+
+    @property
+    def prompt_runners(self) -> list[Request]:
+        return self.owners[self.n_decode:]
+
+    def portion_of(self, req: Request) -> int:
+        """Tokens ``req`` runs in this step (0 if it is not part of it)."""
+        return next((len(e.tokens) for e, r in zip(self.entries, self.owners) if r is req), 0)
+
+    def run(self, req: Request, count: int, decode: bool = False) -> None:
+        """``req`` runs its next ``count`` tokens; it yields a token if that uses up what it has."""
+        start = req.cached
+        last = start + count == req.n_tokens
+        if last:
+            self.yields.append(len(self.entries))
+        self.entries.append(StepEntry(req.cache, start, req.tokens[start:start + count], [count - 1] if last else []))
+        self.owners.append(req)
+        self.n_decode += decode
 
 
 class Scheduler:
     def __init__(self, cfg: EngineConfig, cache: CacheManager):
-        self.cfg = cfg
         self.cache = cache
-        self.waiting: deque[Sequence] = deque()      # FCFS; preempted requests go back to the front
-        self.running: list[Sequence] = []            # admission order, oldest first
-        self.num_preemptions = 0
-        self._admit_counter = 0
-        self._decode_steps_since_prefill = 0
+        self.token_budget = cfg.max_num_batched_tokens
+        self.max_live = cfg.max_num_seqs
+        self.mixed = cfg.enable_chunked_prefill
+        self.prompts_first = cfg.policy == "prefill_first"
+        self.patience = cfg.max_waiting_steps
+        self.queue: deque[Request] = deque()
+        self.live: list[Request] = []             # in order of admission: the last is the newest
+        self.evictions = 0
+        self._decode_steps_with_someone_waiting = 0
 
-    # --- queues -----------------------------------------------------------------------------------------
+    # --- coming and going -----------------------------------------------------------------------
 
-    def add(self, seq: Sequence) -> None:
-        seq.status = Status.WAITING
-        self.waiting.append(seq)
+    def enqueue(self, req: Request) -> None:
+        req.phase = Phase.QUEUED
+        self.queue.append(req)
 
-    def has_unfinished(self) -> bool:
-        return bool(self.waiting or self.running)
+    def busy(self) -> bool:
+        return bool(self.queue) or bool(self.live)
 
-    def finish(self, seq: Sequence, reason: str) -> None:
-        """Give back everything the request holds. Safe for a request in any queue."""
-        if seq.status == Status.FINISHED:
-            return
-        if seq in self.running:
-            self.running.remove(seq)
-            self._release(seq)
-        else:
-            try:
-                self.waiting.remove(seq)
-            except ValueError:
-                pass
-        seq.status = Status.FINISHED
-        seq.finish_reason = reason
+    def retire(self, req: Request, why: str) -> None:
+        """The request ends here, wherever it stands; what it holds goes back. Idempotent."""
+        if req.phase is Phase.LIVE:
+            self.live.remove(req)
+            self._give_back(req)
+        elif req.phase is Phase.QUEUED and req in self.queue:
+            self.queue.remove(req)
+        if req.phase is not Phase.DONE:
+            req.phase, req.why_done = Phase.DONE, why
 
-    def _release(self, seq: Sequence) -> None:
-        if seq.cache is not None:
-            self.cache.free(seq.cache)
-            seq.cache = None
+    def _give_back(self, req: Request) -> None:
+        if req.cache is not None:
+            self.cache.free(req.cache)
+            req.cache = None
 
-    # --- the plan for one step ------------------------------------------------------------------------------
+    # --- one plan ---------------------------------------------------------------------------------
 
-    def schedule(self) -> SchedulerOutput:
-        out = SchedulerOutput()
-        if self.cfg.enable_chunked_prefill:
-            self._schedule_chunked(out)
-            out.num_batched_tokens = len(out.decode_seqs) + out.num_prefill_tokens
-            return out
-        if self._should_prefill():
-            self._schedule_prefills(out)
-            if out.prefill_seqs:
-                self._decode_steps_since_prefill = 0
-                out.num_batched_tokens = out.num_prefill_tokens
-                return out
-        self._schedule_decodes(self.running, out)
-        if self.waiting:
-            self._decode_steps_since_prefill += 1
-        out.num_batched_tokens = len(out.decode_seqs)
-        return out
-
-    def _should_prefill(self) -> bool:
-        if not self.waiting:
-            return False
-        if self.cfg.policy == "prefill_first" or not self.running:
-            return True
-        return self._decode_steps_since_prefill >= self.cfg.max_waiting_steps
-
-    def _admit(self, seq: Sequence) -> None:
-        seq.cache = self.cache.allocate(seq.id, seq.length)      # pages for every token it has, at once
-        seq.num_computed_tokens = 0
-        seq.status = Status.RUNNING
-        seq.admit_order = self._admit_counter
-        self._admit_counter += 1
-        self.running.append(seq)
-
-    def _head_status(self, out: SchedulerOutput):
-        """The head of the queue if it can be admitted now; drops heads that can never fit."""
-        while self.waiting:
-            seq = self.waiting[0]
-            status = self.cache.allocation_status(seq.length)
-            if status == AllocStatus.NEVER:
-                self.waiting.popleft()
-                out.ignored.append(seq)
-                continue
-            return seq if status == AllocStatus.OK else None        # LATER: nobody skips ahead
-        return None
-
-    def _schedule_prefills(self, out: SchedulerOutput) -> None:
-        budget = self.cfg.max_num_batched_tokens
-        while self.waiting and len(self.running) < self.cfg.max_num_seqs:
-            seq = self._head_status(out)
-            if seq is None:
-                break
-            # a prompt that does not fit what is left of the budget waits, unless it is the step's first
-            if seq.length > budget and out.prefill_seqs:
-                break
-            self.waiting.popleft()
-            self._admit(seq)
-            out.prefill_seqs.append(seq)
-            budget -= seq.num_new_tokens
-            if budget <= 0:
-                break
-
-    def _schedule_decodes(self, candidates: list[Sequence], out: SchedulerOutput,
-                          partial: list[Sequence] | None = None) -> None:
-        """Each candidate decodes one token. One that crosses a page edge needs a page; if none is
-        free the newest request not yet visited this step is preempted until it fits. With
-        ``partial`` (chunked mode) requests still inside their prompt are set aside into it instead
-        of decoding; until they are visited they can be preempted like any other."""
-        queue = sorted(candidates, key=lambda s: s.admit_order)
-        try_append, decode_seqs = self.cache.try_append, out.decode_seqs
-        i = 0                                               # queue[i:] are the requests not yet visited
-        while i < len(queue):
-            seq = queue[i]
-            i += 1
-            if partial is not None and seq.num_new_tokens > 1:
-                partial.append(seq)
-                continue
-            length = seq.length
-            while not try_append(seq.cache, length):
-                victim = queue.pop() if i < len(queue) else seq
-                self._preempt(victim, out)
-                if victim is seq:
+    def plan(self) -> StepPlan:
+        plan = StepPlan()
+        if self.mixed:
+            partway = self._plan_decodes(plan, set_aside_prompts=True)
+            room = self.token_budget - plan.n_decode
+            for req in partway:
+                if room <= 0:
                     break
-            else:
-                decode_seqs.append(seq)
-
-    def _schedule_chunked(self, out: SchedulerOutput) -> None:
-        budget = self.cfg.max_num_batched_tokens
-        # 1. fully prefilled requests decode (a prompt with exactly one uncached token is a decode)
-        partial: list[Sequence] = []
-        self._schedule_decodes(self.running, out, partial)
-        budget -= len(out.decode_seqs)
-        # 2. prompts already part-way, oldest first
-        for seq in partial:
-            if budget <= 0:
-                break
-            budget -= self._add_chunk(seq, budget, out)
-        # 3. new admissions, FCFS, pages for the whole prompt up front
-        while self.waiting and budget > 0 and len(self.running) < self.cfg.max_num_seqs:
-            seq = self._head_status(out)
-            if seq is None:
-                break
-            self.waiting.popleft()
-            self._admit(seq)
-            budget -= self._add_chunk(seq, budget, out)
+                room -= self._run_portion(plan, req, room)
+            self._admit(plan, room, cut=True)
+            return plan
+        if self.queue and (self.prompts_first or not self.live
+                           or self._decode_steps_with_someone_waiting >= self.patience):
+            self._admit(plan, self.token_budget, cut=False)
+            if plan:
+                self._decode_steps_with_someone_waiting = 0
+                return plan
+        self._plan_decodes(plan)
+        if self.queue:
+            self._decode_steps_with_someone_waiting += 1
+        return plan
 
     @staticmethod
-    def _add_chunk(seq: Sequence, budget: int, out: SchedulerOutput) -> int:
-        out.prefill_seqs.append(seq)
-        out.prefill_chunks[seq] = min(seq.num_new_tokens, budget)
-        return out.prefill_chunks[seq]
+    def _run_portion(plan: StepPlan, req: Request, room: int) -> int:
+        n = min(req.pending, room)
+        plan.run(req, n)
+        return n
 
-    def _preempt(self, seq: Sequence, out: SchedulerOutput) -> None:
-        self.running.remove(seq)
-        self._release(seq)
-        seq.num_computed_tokens = 0              # recompute prompt + generated tokens on resume
-        seq.status = Status.PREEMPTED
-        seq.num_preemptions += 1
-        self.num_preemptions += 1
-        self.waiting.appendleft(seq)             # front of the queue, original arrival time kept
-        out.preempted.append(seq)
+    def _admit(self, plan: StepPlan, room: int, cut: bool) -> None:
+        """Heads of the queue become live while they fit. ``cut``: a prompt may run only its first
+        ``room`` tokens now; otherwise it runs whole or waits (the step's first prompt always runs)."""
+        first = True
+        while self.queue and room > 0 and len(self.live) < self.max_live:
+            head = self.queue[0]
+            fits = self.cache.allocation_status(head.n_tokens)
+            if fits is AllocStatus.NEVER:
+                plan.unfit.append(self.queue.popleft())
+                continue
+            if fits is AllocStatus.LATER or (not cut and not first and head.n_tokens > room):
+                return
+            self.queue.popleft()
+            head.cache = self.cache.allocate(head.id, head.n_tokens)
+            head.cached = 0
+            head.phase = Phase.LIVE
+            self.live.append(head)
+            count = min(head.pending, room) if cut else head.pending
+            plan.run(head, count)
+            room -= count
+            first = False
+
+    def _plan_decodes(self, plan: StepPlan, set_aside_prompts: bool = False) -> list[Request]:
+        """Every live request with one token pending runs it, oldest first, growing by a page where its
+        length crosses a page edge. ``live[served:unserved_end]`` are the requests this plan has not
+        looked at yet; when a page is missing the last of them is evicted, so the window shrinks
+        from both ends and the loop ends when it is empty. Returns the live requests that are still
+        inside their prompt (only with ``set_aside_prompts``; they can be evicted until they are
+        reached, not after)."""
+        live = self.live
+        partway: list[Request] = []
+        served, unserved_end = 0, len(live)
+        while served < unserved_end:
+            req = live[served]
+            served += 1
+            if set_aside_prompts and req.pending > 1:
+                partway.append(req)
+                continue
+            grown = self.cache.try_append(req.cache, req.n_tokens)
+            while not grown:
+                unserved_end -= 1                       # live[unserved_end] is the newest not yet served
+                victim = live[unserved_end]
+                self._evict(victim, plan)
+                if victim is req:
+                    break
+                grown = self.cache.try_append(req.cache, req.n_tokens)
+            if grown:
+                plan.run(req, 1, decode=True)
+        if unserved_end < len(live):
+            # evicted newest first; at the front of the queue they stand oldest first again
+            self.queue.extendleft(reversed(live[unserved_end:]))
+            del live[unserved_end:]
+        return partway
+
+    def _evict(self, req: Request, plan: StepPlan) -> None:
+        self._give_back(req)
+        req.cached = 0
+        req.phase = Phase.QUEUED
+        req.evictions += 1
+        self.evictions += 1
+        plan.evicted.append(req)

@@ -31,13 +31,15 @@ def _skinny_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
             and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
 
 
-def linear(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, out: torch.Tensor, packed=None) -> torch.Tensor:
-    """out[M, N] = x[M, K] @ w[N, K]^T (+ bias). ``packed``: w in strip order, read instead where it serves."""
+def linear(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, out: torch.Tensor, packed=None,
+           library_first: bool = False) -> torch.Tensor:
+    """out[M, N] = x[M, K] @ w[N, K]^T (+ bias). ``packed``: w in strip order, read instead where it serves.
+    ``library_first``: the owner of w asks for the library's product at any row count (an output head)."""
     M = x.shape[0]
     if M == 0:
         return out
     if packed is not None and len(packed.parts) == 1 and out.stride(1) == 1 and _packed_ok(x, packed) \
-            and not (out.dtype == torch.float32 and bias is None and w.shape[0] >= 16384):
+            and not library_first:
         return ops.gemm_skinny(x, packed, bias, out)
     if x.dtype != torch.bfloat16:
         if ops.gemv_f32_ok(x, w, bias, out):                    # a decode step of the 32-bit path
@@ -45,9 +47,8 @@ def linear(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, out: tor
         return ops.gemm_nt_tiled(x, w, bias, out)
     skinny = _skinny_ok(x, w)
     library = w.dtype == torch.bfloat16 and x.stride(1) == 1 and out.stride(1) == 1
-    if library and out.dtype == torch.float32 and bias is None and w.shape[0] >= 16384:      # logits
-        if ops.gemm_library(x, w, None, out):
-            return out
+    if library and library_first and ops.gemm_library(x, w, bias, out):
+        return out
     if skinny and M <= SKINNY_ROWS:
         return ops.gemm_skinny(x, w, bias, out)
     if library and ops.gemm_library(x, w, bias, out):

@@ -58,10 +58,13 @@ class DecoderModel:
             specs.update(part.tensor_specs(prefix))
         return specs
 
-    def load(self, tensors: dict[str, torch.Tensor], dtype: torch.dtype, device) -> None:
+    def load(self, tensors: dict[str, torch.Tensor], dtype: torch.dtype, device, pack_weights: bool = True) -> None:
+        """Every part takes its tensors, then prepares what its kernels want beside them."""
         self.dtype, self.device = dtype, device
         for part, prefix in self._prefixed():
             part.load(tensors, prefix)
+        for part, _ in self._prefixed():
+            part.prepare(pack_weights)
 
     # --- what the cache manager must provide -------------------------------------------------------
 

@@ -40,6 +40,10 @@ class GQAttention(Mixer):
         self.qkv.load(tensors, prefix)
         self.o.load(tensors, prefix)
         self.position.load(tensors, prefix)
+
+    def prepare(self, pack_weights: bool) -> None:
+        if not pack_weights:
+            return
         if self.head_dim % 32 == 0:
             self.qkv.pack(lambda: ops.fused_qkv_strip_rows(self.num_heads, self.num_kv_heads, self.head_dim, self.hidden))
         self.o.pack(lambda: ops.skinny_strip_rows(self.hidden, self.q_size))

@@ -99,6 +99,10 @@ class Part:
     def load(self, tensors: dict[str, torch.Tensor], prefix: str) -> None:
         """Take this part's tensors (already on the device, in their storage type)."""
 
+    def prepare(self, pack_weights: bool) -> None:
+        """Called once after ``load``: make what the kernels want beside the checkpoint's tensors.
+        ``pack_weights``: whether second copies of matrices in a kernel's own order may be kept."""
+
 
 class Norm(Part):
     def add_norm(self, resid: torch.Tensor, delta: torch.Tensor | None, out_dtype: torch.dtype,

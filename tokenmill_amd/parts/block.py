@@ -32,6 +32,10 @@ class PreNormBlock(Part):
         for part, name in self._parts():
             part.load(tensors, prefix + name)
 
+    def prepare(self, pack_weights: bool) -> None:
+        for part, _ in self._parts():
+            part.prepare(pack_weights)
+
     def forward(self, resid: torch.Tensor, delta: torch.Tensor | None, step: StepContext, cache,
                 dtype: torch.dtype) -> torch.Tensor:
         """resid float32 [T, hidden], updated in place; returns the delta still to be added (None if the

@@ -32,7 +32,7 @@ class OutputHead(Part):
 
     def __init__(self, hidden: int, vocab: int, tied_to: TokenEmbedding | None, name: str = "lm_head"):
         self.hidden, self.vocab, self.tied_to = hidden, vocab, tied_to
-        self.proj = Linear(hidden, vocab, name, bias=False)
+        self.proj = Linear(hidden, vocab, name, bias=False, library_first=True)
 
     def tensor_specs(self, prefix: str):
         return {} if self.tied_to is not None else self.proj.tensor_specs(prefix)

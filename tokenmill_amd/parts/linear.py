@@ -14,18 +14,15 @@ from tokenmill_amd.weights.loader import TensorSpec
 
 
 class Linear(Part):
-    # Whether `pack` keeps the second, packed copy. The loaders set it from the engine's options before a
-    # model takes its tensors (twice the layer matrices in memory against faster decode steps).
-    keep_packed_copy = True
-
     def __init__(self, in_features: int, out_features: list[int] | int, names: list[str] | str,
-                 bias: bool = False):
+                 bias: bool = False, library_first: bool = False):
         self.in_features = in_features
         self.out_splits = [out_features] if isinstance(out_features, int) else list(out_features)
         self.names = [names] if isinstance(names, str) else list(names)
         assert len(self.names) == len(self.out_splits)
         self.out_features = sum(self.out_splits)
         self.has_bias = bias
+        self.library_first = library_first              # a wide matrix the library reads fastest at any row count
         self.weight: torch.Tensor | None = None
         self.bias: torch.Tensor | None = None
         self.packed: ops.PackedWeight | None = None     # the matrix again in the order the decode kernels read
@@ -53,7 +50,7 @@ class Linear(Part):
         row-major one. ``rows``: rows of a strip, or a function that gives them (asked only if the matrix
         is packed). A matrix of another type or not on a GPU is left as it is."""
         w = self.weight
-        if Linear.keep_packed_copy and w is not None and w.dtype == torch.bfloat16 and w.is_cuda:
+        if w is not None and w.dtype == torch.bfloat16 and w.is_cuda:
             self.packed = ops.pack_weight(w, rows() if callable(rows) else rows, parts)
 
     def use_weight(self, weight: torch.Tensor) -> None:
@@ -76,7 +73,8 @@ class Linear(Part):
             x = ops.convert(x.contiguous(), torch.empty(x.shape, dtype=w.dtype, device=x.device))
         inner_dtype = torch.float32 if x.dtype == torch.float32 else out_dtype
         out = torch.empty((x.shape[0], self.out_features), dtype=inner_dtype, device=x.device)
-        gemm.linear(x, w, self.bias, out, packed=self.packed if x.dtype == w.dtype else None)
+        gemm.linear(x, w, self.bias, out, packed=self.packed if x.dtype == w.dtype else None,
+                    library_first=self.library_first)
         if out.dtype != out_dtype:
             out = ops.convert(out, torch.empty(out.shape, dtype=out_dtype, device=out.device))
         return out

@@ -22,6 +22,10 @@ class SwiGLU(FeedForward):
     def load(self, tensors, prefix: str) -> None:
         self.gate_up.load(tensors, prefix)
         self.down.load(tensors, prefix)
+
+    def prepare(self, pack_weights: bool) -> None:
+        if not pack_weights:
+            return
         self.gate_up.pack(16, [self.intermediate, self.intermediate])
         self.down.pack(lambda: ops.skinny_strip_rows(self.hidden, self.intermediate))
 

@@ -1,6 +1,6 @@
 """Trace replay: feed given token ids through a model step by step and write logits.
 
-    bin/trace_run --model DIR --dtype bfloat16|float32 --out DIR --max-tokens N
+    bin/trace_run --model DIR --dtype bfloat16|float32 --out DIR --max-tokens N [--block-size P]
 
 Steps are read from standard input, one JSON object a line:
 
@@ -19,14 +19,15 @@ import json
 import sys
 from pathlib import Path
 
-PAGE_SIZE = 16          # tokens per cache page (the engine's default --block-size)
+PAGE_SIZE = 16          # tokens per cache page unless --block-size says otherwise (the engine's default)
 ROUND_TO = 64           # --max-tokens counts each request's tokens rounded up to this
 
 
 class ReplaySession:
     """The engine pieces a replay drives: model, cache pools, cache manager and the step function."""
 
-    def __init__(self, model_dir, dtype_name: str, max_tokens: int, max_requests: int = 16):
+    def __init__(self, model_dir, dtype_name: str, max_tokens: int, max_requests: int = 16,
+                 page_size: int = PAGE_SIZE):
         from tokenmill_amd.cache import CacheManager
         from tokenmill_amd.cache.pool import CachePools
         from tokenmill_amd.engine.loading import load_model, resolve_device, resolve_dtype
@@ -36,11 +37,16 @@ class ReplaySession:
         library()                                # compiles the kernels at the first call of a fresh checkout
         device = resolve_device("auto")
         dtype = resolve_dtype(dtype_name)
+        if page_size < 1:
+            raise ValueError("--block-size must be at least 1")
         max_tokens = -(-max_tokens // ROUND_TO) * ROUND_TO
         self.model = load_model(model_dir, dtype, device, max_positions=max_tokens)
-        self.num_pages = max_tokens // PAGE_SIZE
-        self.pools = CachePools(self.model, self.num_pages, PAGE_SIZE, max_requests, dtype, device)
-        self.manager = CacheManager(self.pools.windows, self.num_pages, PAGE_SIZE, max_requests)
+        self.page_size = page_size
+        # every request's tokens count rounded up to ROUND_TO; a page that does not divide that may leave
+        # one page per request part empty beyond it
+        self.num_pages = -(-max_tokens // page_size) + (0 if ROUND_TO % page_size == 0 else max_requests)
+        self.pools = CachePools(self.model, self.num_pages, page_size, max_requests, dtype, device)
+        self.manager = CacheManager(self.pools.windows, self.num_pages, page_size, max_requests)
         self.runner = ModelRunner(self.model, self.pools, max_positions=max_tokens)
         self.lengths: dict[str, int] = {}
 
@@ -89,14 +95,15 @@ def main(argv=None) -> int:
     p.add_argument("--max-tokens", type=int, required=True,
                    help="most tokens live requests hold at any time (each rounded up to a multiple of 64)")
     p.add_argument("--max-requests", type=int, default=16, help="most requests live at a time")
+    p.add_argument("--block-size", type=int, default=PAGE_SIZE, help="tokens per cache page")
     args = p.parse_args(argv)
 
     print("[trace_run] loading the engine ...", flush=True)
-    session = ReplaySession(args.model, args.dtype, args.max_tokens, args.max_requests)
+    session = ReplaySession(args.model, args.dtype, args.max_tokens, args.max_requests, args.block_size)
     out_dir = Path(args.out)
     out_dir.mkdir(parents=True, exist_ok=True)
     print(f"[trace_run] ready: {type(session.model.config).__name__}, {args.dtype}, "
-          f"{session.num_pages} pages of {PAGE_SIZE}", flush=True)
+          f"{session.num_pages} pages of {session.page_size}", flush=True)
     for line in sys.stdin:
         line = line.strip()
         if not line:
