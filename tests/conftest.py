@@ -35,8 +35,15 @@ TINY_C = qwen2_config(num_hidden_layers=2, hidden_size=120, num_attention_heads=
                       head_dim=48, intermediate_size=200, vocab_size=307, rope_theta=50000.0, rms_norm_eps=3e-6,
                       tie_word_embeddings=False)
 
+# A head size and a group the published shapes have (64; seven query heads on one kv head), and weights wide
+# enough that attention is peaked and the logits spread over several units: a wrong key or mask moves them far.
+TINY_D = qwen2_config(num_hidden_layers=2, hidden_size=448, num_attention_heads=7, num_key_value_heads=1,
+                      intermediate_size=600, vocab_size=500, rope_theta=1e6, rms_norm_eps=1e-6,
+                      tie_word_embeddings=False, eos_token_id=2)
+
 # (config, weight seed, std of matrices and biases, std of the norm weights around 1)
-TINY = {"A": (TINY_A, 0, 0.02, 0.0), "B": (TINY_B, 1, 0.02, 0.1), "C": (TINY_C, 2, 0.08, 0.2)}
+TINY = {"A": (TINY_A, 0, 0.02, 0.0), "B": (TINY_B, 1, 0.02, 0.1), "C": (TINY_C, 2, 0.08, 0.2),
+        "D": (TINY_D, 3, 0.06, 0.1)}
 
 
 @pytest.fixture(scope="session")
@@ -68,6 +75,23 @@ class Plain:
         if key not in self._cache:
             self._cache[key] = self.P.forward_logits(self.w, self.cfg, list(ids), dt)
         return self._cache[key]
+
+    def bf16_noise(self, lengths=(96, 61, 30), orders=None) -> float:
+        """How far the bfloat16 logits of this model move when only the order of the 32-bit sums changes:
+        the largest difference, over a few random sequences, between the plain implementation's usual
+        summation order and each of its other ones. Measured, per model, on the CPU; the bfloat16
+        comparisons take their bound from it."""
+        if "noise" not in self._cache:
+            worst = 0.0
+            for i, n in enumerate(lengths):
+                ids = random_ids(n, self.cfg["vocab"], 9000 + i)
+                a = self.logits(ids, torch.bfloat16)
+                for k in range(1, orders or self.P.NUM_ORDERS):
+                    with self.P.summation_order(k):
+                        b = self.P.forward_logits(self.w, self.cfg, ids, torch.bfloat16)
+                    worst = max(worst, float((a - b).abs().max()))
+            self._cache["noise"] = worst
+        return self._cache["noise"]
 
 
 @pytest.fixture(scope="session")

@@ -31,6 +31,45 @@ def rnd(x: torch.Tensor, dt: torch.dtype) -> torch.Tensor:
     return x if dt == torch.float32 else x.to(dt).to(torch.float32)
 
 
+# The order in which the 32-bit sums of the products are taken. 0: one sum over the whole inner
+# dimension (whatever order torch's routine has). k >= 1: partial sums over pieces of 16, 24, 32, 40 or
+# 48 elements, added last piece first for odd k and first piece first for even k. All are correct; in
+# bfloat16 a rounding falls the other way here and there, and how far such runs of the SAME model
+# drift apart is the noise floor below which no bfloat16 comparison can look (the reference measures
+# its 16-bit floor the same way, with two batchings of one model, which make its library take other
+# kernels: reference baselines/make_golden.py:195-217). The orders k >= 1 also round the softmax
+# weights before the division by their sum instead of after it (``_weighted_values``).
+_SUM_ORDER = 0
+_PIECES = (16, 24, 32, 40, 48)
+NUM_ORDERS = 1 + 2 * len(_PIECES)
+
+
+class summation_order:
+    def __init__(self, order: int):
+        self.order = order
+
+    def __enter__(self):
+        global _SUM_ORDER
+        self.before, _SUM_ORDER = _SUM_ORDER, self.order
+
+    def __exit__(self, *exc):
+        global _SUM_ORDER
+        _SUM_ORDER = self.before
+
+
+def _matmul(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """a [M, K] @ b [K, N] in 32-bit, in the current summation order."""
+    piece = _PIECES[((_SUM_ORDER - 1) // 2) % len(_PIECES)]
+    if _SUM_ORDER == 0 or a.shape[-1] <= piece:
+        return a @ b
+    starts = range(0, a.shape[-1], piece)
+    total = None
+    for lo in (reversed(starts) if _SUM_ORDER % 2 else starts):
+        part = a[..., lo:lo + piece] @ b[lo:lo + piece]
+        total = part if total is None else total + part
+    return total
+
+
 # ---------------------------------------------------------------------------------------------
 # reading a model folder
 # ---------------------------------------------------------------------------------------------
@@ -107,10 +146,22 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = No
            dt=torch.float32, out_dt=None) -> torch.Tensor:
     """y = x W^T + b with W [out, in] (torch's F.linear as used at reference
     src/infer/model/layers.py:144,150,163-164 and src/infer/model/qwen2.py:51-52)."""
-    y = rnd(x, dt) @ rnd(weight, dt).t()
+    y = _matmul(rnd(x, dt), rnd(weight, dt).t())
     if bias is not None:
         y = y + rnd(bias, dt)
     return rnd(y, dt if out_dt is None else out_dt)
+
+
+def _weighted_values(scores: torch.Tensor, v: torch.Tensor, dt) -> torch.Tensor:
+    """softmax(scores) @ v with the softmax in 32-bit and its weights rounded to the storage type before
+    they multiply the values (reference src/infer/model/layers.py:81-82). In the other summation orders the
+    weights are rounded BEFORE they are divided by their sum (exp(score - max), rounded, times v, over the
+    32-bit sum): the order a kernel that sees the keys block by block has to take. Both round each weight
+    once, to the same relative precision."""
+    if _SUM_ORDER == 0:
+        return _matmul(rnd(torch.softmax(scores, dim=-1), dt), v)
+    e = torch.exp(scores - scores.max(dim=-1, keepdim=True).values)
+    return _matmul(rnd(e, dt), v) / e.sum(dim=-1, keepdim=True)
 
 
 def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float,
@@ -136,8 +187,29 @@ def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: f
         vh = v[:, h // group, :]
         scores = (q[:, h, :] @ kh.t()) * scale
         scores = scores.masked_fill(~allowed, float("-inf"))
-        probs = rnd(torch.softmax(scores, dim=-1), dt)
-        out[:, h, :] = probs @ vh
+        out[:, h, :] = _weighted_values(scores, vh, dt)
+    return rnd(out, dt)
+
+
+def attention_rows(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, first_pos: int, scale: float,
+                   dt=torch.float32, window: int | None = None) -> torch.Tensor:
+    """The same attention for the queries at positions first_pos, first_pos + 1, ... only (what a
+    portion of a long prompt, or one decoded token, computes): q [n, H, D] against all of k, v
+    [L, KVH, D]; query i of them sees keys j <= first_pos + i. With first_pos = 0 and n = L it is
+    ``causal_attention`` (tested), whose L x L scores a context of thousands of keys cannot afford."""
+    n, H, D = q.shape
+    L, kvh = k.shape[0], k.shape[1]
+    group = H // kvh
+    out = torch.empty(n, H, D, dtype=torch.float32)
+    i = first_pos + torch.arange(n)[:, None]
+    j = torch.arange(L)[None, :]
+    allowed = j <= i
+    if window is not None:
+        allowed = allowed & (j > i - window)
+    for h in range(H):
+        scores = (q[:, h, :] @ k[:, h // group, :].t()) * scale
+        scores = scores.masked_fill(~allowed, float("-inf"))
+        out[:, h, :] = _weighted_values(scores, v[:, h // group, :], dt)
     return rnd(out, dt)
 
 

@@ -12,7 +12,7 @@ import torch
 
 from conftest import ROOT, TINY, random_ids
 from plain import qwen2_plain as P
-from tolerances import REL
+from tolerances import check_greedy_token, logits_bound, near_ties
 
 pytestmark = pytest.mark.gpu
 
@@ -28,19 +28,25 @@ def make_engine(model_dir, dtype_name, **kw):
 
 
 def verify(plain, prompt, out, dt, params=None, seed=0):
-    """Every generated token is what the plain implementation picks after the same tokens."""
+    """Every generated token is what the plain implementation (in the same precision) picks after the same
+    tokens, or a near-tie with it under the measured bound. Returns the number of such exemptions; they can
+    never be more than the near-ties among the rows (asserted)."""
     logits = plain.logits(list(prompt) + list(out), dt)[len(prompt) - 1:-1]
-    scale = max(1.0, float(logits.abs().max()))
-    gap = 2 * REL[dt] * scale
+    noise = plain.bf16_noise() if dt == torch.bfloat16 else None
     exempt = 0
     for n, (row, tok) in enumerate(zip(logits, out)):
         if params is None or params.greedy:
-            assert row[tok] >= row.max() - gap, f"token {n}: {tok} is not the argmax ({row[tok]} vs {row.max()})"
-            exempt += int(tok != int(row.argmax()))
+            exempt += check_greedy_token(row, tok, dt, noise, f"token {n}")
         else:
             want, margin = P.sample_token(row, params.temperature, params.top_k, params.top_p, seed, n)
-            assert tok == want or margin < 20 * REL[dt], f"token {n}: sampled {tok}, plain {want} (margin {margin})"
-            exempt += int(tok != want)
+            if tok != want:
+                # logits off by at most the bound move every probability, and so the point where the random
+                # number falls in the cumulative distribution, by at most 2 * bound / temperature
+                allowed = 2 * logits_bound(row, dt, noise) / params.temperature
+                assert margin <= allowed, f"token {n}: sampled {tok}, plain {want} (margin {margin:.3e} > {allowed:.3e})"
+                exempt += 1
+    if params is None or params.greedy:
+        assert exempt <= near_ties(logits, dt, noise)
     return exempt
 
 
@@ -53,7 +59,7 @@ def test_greedy_generation_whole_prompts(model_dirs, plains, dtype_name):
     outs = eng.generate(prompts, SamplingParams(max_tokens=16, ignore_eos=True))
     assert [len(o) for o in outs] == [16, 16, 16]
     flips = sum(verify(plains["A"], p, o, DTYPES[dtype_name]) for p, o in zip(prompts, outs))
-    assert flips == 0 or dtype_name == "bfloat16"
+    assert flips == 0 or dtype_name == "bfloat16"       # (bfloat16: never more than the near-ties, checked by verify)
     assert not eng.scheduler.live and eng.cache.num_free_pages == eng.cache.num_pages
     assert eng.stats["prompt_steps"] == 1 and eng.stats["decode_steps"] == 15 and eng.stats["tokens_out"] == 48
 
@@ -77,6 +83,8 @@ def test_sampled_generation_chunked_and_mixed(model_dirs, plains, dtype_name):
     alone = make_engine(model_dirs["B"], dtype_name, block_size=8).generate([prompts[2]], params[2])[0]
     if dtype_name == "float32":
         assert alone == outs[2]
+    else:                                               # a rounding may fall the other way in another batch: near-ties only
+        verify(plains["B"], prompts[2], alone, torch.bfloat16, params[2], seed=102)
 
 
 @pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
@@ -234,7 +242,8 @@ def test_command_line_random_weights(model_dirs):
     assert first == again
     assert first != other
     named = run(3, "tiny-a")
-    assert [len(o) for o in named] == [8, 8] and all(0 <= t < 256 for o in named for t in o)
+    by_path = run(3, str(ROOT / "tokenmill_amd" / "config" / "shapes" / "tiny-a.json"))
+    assert [len(o) for o in named] == [8, 8] and named == by_path and named != first
 
 
 @pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
@@ -370,3 +379,71 @@ def test_steps_run_kernel_by_kernel_when_a_capture_fails(model_dirs, plains, mon
     assert eng.runner.graphs.failed == {1} and eng.runner.graphs.replays == 0
     assert eng.runner.step_graphs.failed == {(32, 1, 0, 1)} and (64, 1, 0, 1) in eng.runner.step_graphs.captured
     assert eng.cache.num_free_pages == eng.cache.num_pages
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_graphs_with_portions_and_a_starved_pool(model_dirs, plains, dtype_name):
+    """Graph replays, prompt portions and evictions together: so few pages that requests lose theirs and are
+    recomputed while decode steps and mixed steps replay from graphs. A decode graph keeps, per row of its
+    batch, whose block table the row holds (only new pages are written); a request that comes back after an
+    eviction has another table on other pages and must not find its old one there."""
+    from tokenmill_amd import SamplingParams
+    lengths = [9, 30, 17, 4, 26, 12, 21, 7, 33, 15, 2, 28]
+    prompts = [random_ids(n, 384, 900 + i) for i, n in enumerate(lengths)]
+    params = [SamplingParams(max_tokens=14 + 3 * (i % 5), ignore_eos=True) for i in range(len(prompts))]
+    outs = {}
+    for graphs in (False, True):
+        eng = make_engine(model_dirs["B"], dtype_name, block_size=4, kv_cache_mb=None, num_blocks=36,
+                          hip_graphs=graphs, max_num_seqs=5, max_num_batched_tokens=16,
+                          enable_chunked_prefill=True, max_model_len=96)
+        outs[graphs] = eng.generate(prompts, params)
+        assert eng.scheduler.evictions > 0, "the pool must be small enough to evict"
+        eng.cache.check_invariants()
+        assert eng.cache.num_free_pages == eng.cache.num_pages and not eng.scheduler.live
+        if graphs:
+            assert eng.runner.graphs.replays > 20 and eng.runner.step_graphs.replays > 0
+    for p, o, sp in zip(prompts, outs[True], params):
+        assert len(o) == sp.max_tokens
+        verify(plains["B"], p, o, DTYPES[dtype_name])
+    assert outs[True] == outs[False]
+
+
+def test_decode_graphs_over_contexts_that_need_the_split_attention(model_dirs, plains):
+    """max_model_len 1,024 makes the decode graphs launch the split attention (chunks of 256 keys merged
+    afterwards), as every real run does; the contexts grow across 256 and 512 keys while they replay."""
+    from tokenmill_amd import SamplingParams
+    lengths = [250, 505, 30, 761]
+    prompts = [random_ids(n, 384, 950 + i) for i, n in enumerate(lengths)]
+    sp = SamplingParams(max_tokens=14, ignore_eos=True)
+    outs = {}
+    for graphs in (False, True):
+        eng = make_engine(model_dirs["B"], "bfloat16", block_size=16, kv_cache_mb=16, hip_graphs=graphs,
+                          max_num_seqs=4, max_num_batched_tokens=1024, max_model_len=1024)
+        outs[graphs] = eng.generate(prompts, sp)
+        if graphs:
+            assert eng.runner.graphs.replays >= 12
+        eng.cache.check_invariants()
+        assert eng.cache.num_free_pages == eng.cache.num_pages
+    for p, o in zip(prompts, outs[True]):
+        verify(plains["B"], p, o, torch.bfloat16)
+    assert outs[True] == outs[False]
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_generation_with_peaked_attention_at_a_published_head_size(model_dirs, plains, dtype_name):
+    """Configuration D (head size 64, seven query heads on one kv head, weights wide enough that a single
+    key can carry a query): whole prompts and portions mixed with decodes, the pool so small that pages are
+    handed out again."""
+    from tokenmill_amd import SamplingParams
+    prompts = [random_ids(n, 500, 970 + i) for i, n in enumerate([3, 70, 33, 18, 120, 47, 9, 64])]
+    sp = SamplingParams(max_tokens=12, ignore_eos=True)
+    dt = DTYPES[dtype_name]
+    whole = make_engine(model_dirs["D"], dtype_name, max_num_seqs=8, kv_cache_mb=None, num_blocks=40)
+    cut = make_engine(model_dirs["D"], dtype_name, max_num_seqs=4, kv_cache_mb=None, num_blocks=24,
+                      enable_chunked_prefill=True, max_num_batched_tokens=20)
+    flips = 0
+    for eng in (whole, cut):
+        for p, o in zip(prompts, eng.generate(prompts, sp)):
+            flips += verify(plains["D"], p, o, dt)
+        assert eng.cache.num_free_pages == eng.cache.num_pages
+    assert flips == 0 or dtype_name == "bfloat16"       # (bfloat16: never more than the near-ties, checked by verify)

@@ -147,10 +147,11 @@ def test_gemm_tiled(ops, dt, M, N, K):
     assert torch.equal(one[0], out32[M - 1])
 
 
-def paged_case(dt, lens, q_lens, H, KVH, D, page, seed, spike=None, ramp=None):
+def paged_case(dt, lens, q_lens, H, KVH, D, page, seed, spike=None, ramp=None, ramp_slope=1.0):
     """Random requests laid out in shuffled pages. Returns device operands and the CPU truth.
-    ramp: a request whose scores rise steadily with the key's position (about 5 units of log2 per 32
-    keys), so that the running maximum of a flash-style kernel keeps moving."""
+    spike = (request, key[, size]): one far key that carries the request's last query. ramp: a request (or
+    a set of them) whose scores rise steadily with the key's position (about 5 * ramp_slope units of log2
+    per 32 keys), so that the running maximum of a flash-style kernel keeps moving."""
     g = torch.Generator().manual_seed(seed)
     S = len(lens)
     n_pages = sum(-(-n // page) for n in lens) + 3
@@ -166,13 +167,13 @@ def paged_case(dt, lens, q_lens, H, KVH, D, page, seed, spike=None, ramp=None):
         v = torch.randn(n, KVH, D, generator=g).to(dt)
         qq = torch.randn(n, H, D, generator=g).to(dt)
         if spike and spike[0] == s:                                  # one far key that must dominate the last query
-            _, far = spike
+            far, size = spike[1], (spike[2] if len(spike) > 2 else 12.0)
             k[far] *= 0.0
-            k[far, :, 0] = 12.0
+            k[far, :, 0] = size
             qq[n - 1] *= 0.0
-            qq[n - 1, :, 0] = 12.0
-        if ramp is not None and ramp == s:
-            k[:, :, 1] = (torch.arange(n, dtype=torch.float32)[:, None] * (0.15 * (64 / D) ** 0.5)).to(dt)
+            qq[n - 1, :, 0] = size
+        if ramp is not None and (s in ramp if isinstance(ramp, (set, tuple)) else ramp == s):
+            k[:, :, 1] = (torch.arange(n, dtype=torch.float32)[:, None] * (0.15 * ramp_slope * (64 / D) ** 0.5)).to(dt)
             qq[:, :, 1] = 6.0
         for i in range(-(-n // page)):
             tables[s, i] = perm[used]

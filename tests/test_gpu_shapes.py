@@ -49,7 +49,70 @@ def test_layer_sizes_of_the_published_shapes(tmp_path, name, dtypes):
         got = run_trace(session, steps)
         assert len(got) == 3 + 2 + 10 + 1
         for (rid, p), row in got.items():
-            assert_logits_close(row, plain.logits(ids[rid], dt)[p], dt, f"{name} shape {dtype_name} {rid} position {p}")
+            assert_logits_close(row, plain.logits(ids[rid], dt)[p], dt, f"{name} shape {dtype_name} {rid} position {p}",
+                                plain.bf16_noise((40, 25)) if dt == torch.bfloat16 else None)
         assert not session.manager.live
         del session
         torch.cuda.empty_cache()
+
+
+LAYERS = {
+    "0.5B": qwen2_config(num_hidden_layers=2, hidden_size=896, num_attention_heads=14, num_key_value_heads=2,
+                         intermediate_size=4864, vocab_size=1000, rope_theta=1e6, rms_norm_eps=1e-6,
+                         tie_word_embeddings=True),
+    "7B": qwen2_config(num_hidden_layers=2, hidden_size=3584, num_attention_heads=28, num_key_value_heads=4,
+                       intermediate_size=18944, vocab_size=1000, rope_theta=1e6, rms_norm_eps=1e-6,
+                       tie_word_embeddings=False),
+}
+
+
+@pytest.fixture(scope="module")
+def layer_models(tmp_path_factory):
+    from conftest import Plain
+    from tokenmill_amd.weights import write_random_model
+    made = {}
+
+    def get(name):
+        if name not in made:
+            d = write_random_model(LAYERS[name], tmp_path_factory.mktemp(f"layers{name}"), seed=8, std=0.02, norm_std=0.1)
+            made[name] = (d, Plain(d))
+        return made[name]
+
+    return get
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["0.5B", "7B"])
+def test_every_cut_at_the_layer_sizes_of_the_published_shapes(layer_models, monkeypatch, name, dtype_name):
+    """Two layers of the 0.5B and of the 7B shape (small vocabulary), replayed whole, with the last 32 tokens
+    one by one, in portions down to two tokens, and mixed with up to four live requests on so few pages that
+    they are used again: the fast paths of the real sizes (head size 64 and 128, groups of 7, the products
+    that start at the norm, and for steps of 17 to 48 rows the products that keep the input in LDS) under
+    every way of cutting, against the plain implementation."""
+    from tokenmill_amd.hip import ops
+    from tokenmill_amd.replay import ReplaySession
+    from test_gpu_replay import assert_all_given_back, check, mixed, portions, prefill_then_decode, run_trace, whole
+
+    d, plain = layer_models(name)
+    dt = {"float32": torch.float32, "bfloat16": torch.bfloat16}[dtype_name]
+    calls = {"panel": 0, "fused": 0}
+    real_panel, real_fused = ops.panel_qkv_rope, ops.fused_norm_qkv_rope
+    monkeypatch.setattr(ops, "panel_qkv_rope", lambda *a, **k: (calls.__setitem__("panel", calls["panel"] + 1), real_panel(*a, **k))[1])
+    monkeypatch.setattr(ops, "fused_norm_qkv_rope", lambda *a, **k: (calls.__setitem__("fused", calls["fused"] + 1), real_fused(*a, **k))[1])
+    lengths = [70, 41, 100, 56, 33, 88, 120, 64]
+    reqs = {f"r{i}": random_ids(n, 1000, 600 + i) for i, n in enumerate(lengths)}
+    session = ReplaySession(d, dtype_name, 4 * 128)            # four live requests of at most 128 tokens: 32 pages
+    assert sum(-(-n // 16) for n in lengths) > session.num_pages
+    steps = mixed(reqs, seed=12, live=4, max_portion=14)
+    sizes = [sum(len(e["tokens"]) for e in st["entries"]) for st in steps]
+    assert any(17 <= n <= 48 for n in sizes) and any(n <= 16 for n in sizes)
+    for what, trace in (("whole", whole(reqs)), ("prefill+decode", prefill_then_decode(reqs)),
+                        ("portions", portions(reqs)), ("mixed", steps)):
+        got = run_trace(session, trace)
+        check(got, plain, reqs, dt, f"{name} layers, {dtype_name}, {what}")
+        assert_all_given_back(session)
+    if dtype_name == "bfloat16":
+        assert calls["fused"] > 0
+        assert calls["panel"] > 0 or name == "7B"             # a width of 3,584 does not fit a block's LDS
+    del session
+    torch.cuda.empty_cache()
