@@ -79,6 +79,19 @@ int tm_attn_prefill_f32(const void* q, int q_stride, void* out, int out_stride, 
 int tm_argmax_work_chunks(int V);
 int tm_argmax_rows(const float* logits, int R, int V, int* out, float* work_v, int* work_i, hipStream_t stream);
 
+// The argmax again, for callers that cannot allocate device memory: code under HIP graph capture, tight
+// serving loops, harnesses that forbid hipMalloc. (The reference has no counterpart: its argmax is a
+// torch call that allocates as it likes.) Same result as tm_argmax_rows. The chunk candidates of the
+// two-stage path go to a fixed array of 512 KiB that each GPU holds from the library's load to the
+// process's end; the call allocates nothing and frees nothing. R * tm_argmax_work_chunks(V) may be at
+// most tm_argmax_rows_static_max_pairs() (65,536: 256 rows of a 1M-entry vocabulary, 1,724 rows of
+// 151,936 entries); more is refused with TM_ERR_ARG before anything is launched. All calls on one GPU
+// share that GPU's array: two calls whose kernels can overlap there (different streams, or threads
+// without an order between them) race; calls on one stream are ordered and safe. The device of
+// `stream` must be the current device.
+int tm_argmax_rows_static_max_pairs(void);
+int tm_argmax_rows_static(const float* logits, int R, int V, int* out, hipStream_t stream);
+
 size_t tm_sample_work_bytes(int R, int V);
 int tm_sample_rows(const float* logits, int R, int V, const float* temperature, const int* top_k,
                    const float* top_p, const float* u, int* out, void* work, size_t work_bytes, int stages,

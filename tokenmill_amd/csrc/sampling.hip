@@ -9,6 +9,8 @@
 #include "common.h"
 #include "api.h"
 
+#include <mutex>
+
 #define SM_NT 1024
 
 // monotonic map float -> uint32 (larger float, larger key)
@@ -130,6 +132,62 @@ extern "C" int tm_argmax_rows(const float* logits, int R, int V, int* out, float
     argmax_partial_kernel<<<dim3(R, NB), AM_NT, 0, stream>>>(logits, V, chunk, work_v, work_i, nullptr, 0);
     TM_CHECK_LAUNCH();
     argmax_final_kernel<<<R, TM_WAVE, 0, stream>>>(work_v, work_i, NB, out);
+    TM_CHECK_LAUNCH();
+    return TM_OK;
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// The same argmax for callers that cannot allocate: the chunk candidates of the two-stage path live in
+// a fixed array in device memory that is part of this library's image on every GPU it runs on.
+//
+// `argmax_scratch` names that array. In host code the name is only a handle for the runtime (not a
+// device address): its address on the current device is asked for once per device
+// (hipGetSymbolAddress) and kept; the kernels get that address as an argument, exactly as they get
+// the caller's work buffers in tm_argmax_rows.
+#define AM_STATIC_PAIRS (64 * 1024)                       // most (row, chunk) candidates: 512 KiB per GPU
+#define AM_STATIC_DEVICES 64
+static __device__ __align__(256) unsigned char argmax_scratch[AM_STATIC_PAIRS * (sizeof(float) + sizeof(int))];
+
+static void* g_argmax_scratch[AM_STATIC_DEVICES];         // device address of the array, per device
+static std::mutex g_argmax_scratch_mutex;
+
+// The array's address on the device that is current now; null if the runtime cannot give it.
+static void* argmax_scratch_here() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= AM_STATIC_DEVICES) return nullptr;
+    std::lock_guard<std::mutex> lock(g_argmax_scratch_mutex);
+    if (!g_argmax_scratch[dev]) {
+        void* p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(argmax_scratch)) != hipSuccess) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        g_argmax_scratch[dev] = p;
+    }
+    return g_argmax_scratch[dev];
+}
+
+extern "C" int tm_argmax_rows_static_max_pairs(void) { return AM_STATIC_PAIRS; }
+
+extern "C" int tm_argmax_rows_static(const float* logits, int R, int V, int* out, hipStream_t stream) {
+    if (R <= 0) return TM_OK;
+    if (V <= 0 || !logits || !out) return TM_ERR_ARG;
+    const int NB = tm_argmax_work_chunks(V);
+    if (NB == 1) {                                         // a narrow row: one block, no scratch at all
+        argmax_rows_kernel<<<R, SM_NT, 0, stream>>>(logits, V, out);
+        TM_CHECK_LAUNCH();
+        return TM_OK;
+    }
+    if ((long long)R * NB > AM_STATIC_PAIRS) return TM_ERR_ARG;      // beyond the fixed array: refused, nothing launched
+    unsigned char* base = (unsigned char*)argmax_scratch_here();
+    if (!base) return TM_ERR_LAUNCH;
+    float* part_v = (float*)base;                                      // [R, NB]
+    int* part_i = (int*)(base + (size_t)AM_STATIC_PAIRS * sizeof(float));   // [R, NB]
+    // Nothing has to start at zero: the first kernel writes every (row, chunk) entry that the second reads.
+    const int chunk = (V + NB - 1) / NB;
+    argmax_partial_kernel<<<dim3(R, NB), AM_NT, 0, stream>>>(logits, V, chunk, part_v, part_i, nullptr, 0);
+    TM_CHECK_LAUNCH();
+    argmax_final_kernel<<<R, TM_WAVE, 0, stream>>>(part_v, part_i, NB, out);
     TM_CHECK_LAUNCH();
     return TM_OK;
 }

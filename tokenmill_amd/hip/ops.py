@@ -728,3 +728,19 @@ def fused_lds_fits(M: int, K: int) -> bool:
     rows = 4 if M <= 4 else (8 if M <= 8 else 16)
     waves = 8 if K >= 2048 else 4
     return rows * (K + 8) * 2 + 4 * waves * 2 * 64 * 5 + 1024 <= 160 * 1024
+
+
+def argmax_rows_static(logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """``argmax_rows`` without any allocation: the chunk candidates go to a fixed array the library holds on
+    each GPU. For callers that cannot allocate; calls that may overlap on one GPU must not be made."""
+    _gpu(logits, out)
+    R, V = logits.shape
+    _need(logits.dtype == torch.float32 and logits.is_contiguous(), "argmax: logits must be contiguous float32 [R, V]")
+    _ints(out, R, "out")
+    lib = library()
+    pairs, most = R * lib.tm_argmax_work_chunks(c_int(V)), lib.tm_argmax_rows_static_max_pairs()
+    _need(pairs <= most or lib.tm_argmax_work_chunks(c_int(V)) == 1,
+          f"argmax (static): {R} rows of {V} logits need {pairs} chunk candidates; the fixed array holds {most}")
+    _need(logits.device.index == torch.cuda.current_device(), "argmax (static): the logits' GPU must be the current device")
+    _check(lib.tm_argmax_rows_static(_p(logits), c_int(R), c_int(V), _p(out), _stream()), "argmax_rows_static")
+    return out
