@@ -10,6 +10,7 @@ from __future__ import annotations
 
 import torch
 
+from tokenmill_amd import profiling
 from tokenmill_amd.hip import attention as attn_kernels
 from tokenmill_amd.hip import gemm, ops
 from tokenmill_amd.parts.base import (KVCacheSpec, KVCacheView, Mixer, NormedInput, PositionEncoding, StepContext,
@@ -88,15 +89,29 @@ class GQAttention(Mixer):
                            cache.k if write else None, cache.v if write else None)
         return q
 
+    def _attention_cost(self, step: StepContext, elem: int) -> tuple[int, int]:
+        """Every key and value of the step's requests read once, q read and the output written; two
+        products of 2 * head_dim flops per (query, visible key, head)."""
+        keys_read = pairs = 0
+        for start, n in zip(step.start_positions, step.q_lens):
+            keys_read += min(start + n, self.window + n - 1) if self.window else start + n
+            for i in range(n):
+                pairs += min(start + i + 1, self.window) if self.window else start + i + 1
+        moved = 2 * keys_read * self.kv_size * elem + 2 * step.num_tokens * self.q_size * elem
+        return moved, 4 * pairs * self.num_heads * self.head_dim
+
     def forward(self, x, step: StepContext, cache: KVCacheView, residual: torch.Tensor | None = None):
-        q = self._fused_qkv(x, step, cache)
-        if q is None:
-            x = as_tensor(x)
-            q = self._panel_qkv(x, step, cache)
-        if q is None:
-            q = self.qkv.forward(x)                                        # [T, (H + 2 KVH) D], q first
-            self.position.encode_and_store(q, self.num_heads, self.num_kv_heads, self.head_dim, step, cache)
+        with profiling.label("qkv", lambda: self.qkv.cost(step.num_tokens)):       # with norm, rotary and cache write where fused
+            q = self._fused_qkv(x, step, cache)
+            if q is None:
+                x = as_tensor(x)
+                q = self._panel_qkv(x, step, cache)
+            if q is None:
+                q = self.qkv.forward(x)                                    # [T, (H + 2 KVH) D], q first
+                self.position.encode_and_store(q, self.num_heads, self.num_kv_heads, self.head_dim, step, cache)
         out = torch.empty((q.shape[0], self.q_size), dtype=q.dtype, device=q.device)
-        attn_kernels.paged_attention(q, out, cache, step, self.num_heads, self.num_kv_heads, self.head_dim,
-                                     self.scale, self.window or 0)
-        return self.o.forward(out, accumulate_into=residual)
+        with profiling.label("attention", lambda: self._attention_cost(step, q.element_size())):
+            attn_kernels.paged_attention(q, out, cache, step, self.num_heads, self.num_kv_heads, self.head_dim,
+                                         self.scale, self.window or 0)
+        with profiling.label("o_proj", lambda: self.o.cost(step.num_tokens)):
+            return self.o.forward(out, accumulate_into=residual)

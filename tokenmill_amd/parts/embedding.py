@@ -3,6 +3,7 @@ from __future__ import annotations
 
 import torch
 
+from tokenmill_amd import profiling
 from tokenmill_amd.hip import ops
 from tokenmill_amd.parts.base import Part
 from tokenmill_amd.parts.linear import Linear
@@ -24,7 +25,8 @@ class TokenEmbedding(Part):
 
     def forward(self, token_ids: torch.Tensor) -> torch.Tensor:
         out = torch.empty((token_ids.numel(), self.hidden), dtype=torch.float32, device=token_ids.device)
-        return ops.embed_gather(self.weight, token_ids, out)
+        with profiling.label("embed", lambda: (out.numel() * (self.weight.element_size() + 4), 0)):
+            return ops.embed_gather(self.weight, token_ids, out)
 
 
 class OutputHead(Part):
@@ -44,4 +46,5 @@ class OutputHead(Part):
             self.proj.load(tensors, prefix)
 
     def forward(self, h: torch.Tensor) -> torch.Tensor:
-        return self.proj.forward(h, out_dtype=torch.float32)
+        with profiling.label("head", lambda: self.proj.cost(h.shape[0], out_bytes=4)):
+            return self.proj.forward(h, out_dtype=torch.float32)

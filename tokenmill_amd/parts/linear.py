@@ -53,6 +53,16 @@ class Linear(Part):
         if w is not None and w.dtype == torch.bfloat16 and w.is_cuda:
             self.packed = ops.pack_weight(w, rows() if callable(rows) else rows, parts)
 
+    def cost(self, rows: int, in_bytes: int | None = None, out_bytes: int | None = None) -> tuple[int, int]:
+        """(bytes, flops) the product has to move and do for ``rows`` rows: the matrix once, the input and
+        the output (``in_bytes`` / ``out_bytes`` per element, default the matrix's element size)."""
+        e = self.weight.element_size()
+        n, k = self.out_features, self.in_features
+        moved = n * k * e + rows * k * (e if in_bytes is None else in_bytes) + rows * n * (e if out_bytes is None else out_bytes)
+        if self.bias is not None:
+            moved += self.bias.numel() * self.bias.element_size()
+        return moved, 2 * rows * n * k
+
     def use_weight(self, weight: torch.Tensor) -> None:
         """Share another part's matrix (a tied output head)."""
         self.weight = weight

@@ -4,6 +4,7 @@ from __future__ import annotations
 
 import torch
 
+from tokenmill_amd import profiling
 from tokenmill_amd.hip import gemm, ops
 from tokenmill_amd.parts.base import FeedForward, NormedInput, StepContext, as_tensor
 from tokenmill_amd.parts.linear import Linear
@@ -30,6 +31,14 @@ class SwiGLU(FeedForward):
         self.down.pack(lambda: ops.skinny_strip_rows(self.hidden, self.intermediate))
 
     def forward(self, x, step: StepContext | None = None, residual: torch.Tensor | None = None):
+        rows = x.num_tokens if isinstance(x, NormedInput) else x.shape[0]
+        with profiling.label("gate_up", lambda: self.gate_up.cost(rows)):          # with norm and SiLU*up where fused
+            act = self._activation(x)
+        with profiling.label("down", lambda: self.down.cost(rows)):
+            return self.down.forward(act, accumulate_into=residual)
+
+    def _activation(self, x) -> torch.Tensor:
+        """silu(gate(x)) * up(x), [T, intermediate]."""
         w = self.gate_up.weight
         act = None
         if isinstance(x, NormedInput) and x.dtype == torch.bfloat16 and self.gate_up.bias is None and \
@@ -44,4 +53,4 @@ class SwiGLU(FeedForward):
             if not (w.dtype == x.dtype and self.gate_up.bias is None
                     and gemm.gate_up_silu(x, w, act, packed=self.gate_up.packed)):
                 ops.silu_mul(self.gate_up.forward(x), act)
-        return self.down.forward(act, accumulate_into=residual)
+        return act

@@ -4,6 +4,7 @@ from __future__ import annotations
 
 import torch
 
+from tokenmill_amd import profiling
 from tokenmill_amd.hip import ops
 from tokenmill_amd.parts.base import Norm
 from tokenmill_amd.weights.loader import TensorSpec
@@ -26,7 +27,9 @@ class RMSNorm(Norm):
     def add_norm(self, resid, delta, out_dtype, rows=None):
         n = resid.shape[0] if rows is None else rows.numel()
         out = torch.empty((n, self.hidden), dtype=out_dtype, device=resid.device)
-        return ops.add_rmsnorm(resid, delta, self.weight, self.eps, out, rows)
+        with profiling.label("norm", lambda: (n * self.hidden * (4 + (0 if rows is not None else 4) + out.element_size()
+                                                                 + (out.element_size() if delta is not None else 0)), 0)):
+            return ops.add_rmsnorm(resid, delta, self.weight, self.eps, out, rows)
 
     def rms_params(self):
         return self.weight, self.eps

@@ -17,6 +17,7 @@ from dataclasses import dataclass, field
 
 import torch
 
+from tokenmill_amd import profiling
 from tokenmill_amd.hip import ops
 
 _M64 = (1 << 64) - 1
@@ -62,6 +63,11 @@ class Sampler:
         R = logits.shape[0]
         if R == 0:
             return []
+        with profiling.label("sample", lambda: (logits.numel() * 4, 0)):
+            return self._sample(logits, params, seeds, counters)
+
+    def _sample(self, logits, params, seeds, counters) -> list[int]:
+        R = logits.shape[0]
         out = torch.empty(R, dtype=torch.int32, device=logits.device)
         if all(p.greedy for p in params):
             ops.argmax_rows(logits, out)
