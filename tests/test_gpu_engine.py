@@ -117,31 +117,29 @@ def test_same_tokens_under_every_cutting_and_a_starved_pool(model_dirs, plains, 
 
 def test_steps_of_17_to_48_tokens_take_the_panel_products(model_dirs, plains, monkeypatch):
     """24 requests decoding together, and prompt steps of 20 to 40 tokens: the q|k|v and gate|up products
-    that keep the normed input in LDS run (counted), and every token is the plain implementation's."""
+    that keep the normed input in LDS run (counted, in the library's step program and in the parts' own
+    code), and every token is the plain implementation's."""
     from tokenmill_amd import SamplingParams
     from tokenmill_amd.hip import ops
-    calls = {"qkv": 0, "gate_up": 0}
-    real_qkv, real_gu = ops.panel_qkv_rope, ops.panel_gate_up_silu
-
-    def counted_qkv(*a, **k):
-        calls["qkv"] += 1
-        return real_qkv(*a, **k)
-
-    def counted_gu(*a, **k):
-        calls["gate_up"] += 1
-        return real_gu(*a, **k)
-
-    monkeypatch.setattr(ops, "panel_qkv_rope", counted_qkv)
-    monkeypatch.setattr(ops, "panel_gate_up_silu", counted_gu)
-    eng = make_engine(model_dirs["B"], "bfloat16", max_num_batched_tokens=40)
     prompts = [random_ids(1 + (7 * i) % 19, 384, 300 + i) for i in range(24)]
+    layers = 3
+    eng = make_engine(model_dirs["B"], "bfloat16", max_num_batched_tokens=40)
+    assert eng.runner.program is not None
     outs = eng.generate(prompts, SamplingParams(max_tokens=10, ignore_eos=True))
     for p, o in zip(prompts, outs):
         assert len(o) == 10
         verify(plains["B"], p, o, torch.bfloat16)
-    layers = 3
-    assert calls["qkv"] >= 9 * layers and calls["gate_up"] == calls["qkv"]       # the decode steps of 24 tokens at least
+    took = eng.runner.program.counters()
+    assert took["qkv_panel"] >= 9 * layers and took["gate_up_panel"] == took["qkv_panel"]      # the decode steps of 24 tokens at least
     assert eng.cache.num_free_pages == eng.cache.num_pages
+    calls = {"qkv": 0, "gate_up": 0}
+    real_qkv, real_gu = ops.panel_qkv_rope, ops.panel_gate_up_silu
+    monkeypatch.setattr(ops, "panel_qkv_rope", lambda *a, **k: (calls.__setitem__("qkv", calls["qkv"] + 1), real_qkv(*a, **k))[1])
+    monkeypatch.setattr(ops, "panel_gate_up_silu", lambda *a, **k: (calls.__setitem__("gate_up", calls["gate_up"] + 1), real_gu(*a, **k))[1])
+    by_parts = make_engine(model_dirs["B"], "bfloat16", max_num_batched_tokens=40, step_program=False)
+    assert by_parts.runner.program is None
+    assert by_parts.generate(prompts, SamplingParams(max_tokens=10, ignore_eos=True)) == outs
+    assert calls["qkv"] == took["qkv_panel"] and calls["gate_up"] == took["gate_up_panel"]
 
 
 def test_without_the_packed_copy_of_the_matrices(model_dirs, plains):
@@ -447,3 +445,25 @@ def test_generation_with_peaked_attention_at_a_published_head_size(model_dirs, p
             flips += verify(plains["D"], p, o, dt)
         assert eng.cache.num_free_pages == eng.cache.num_pages
     assert flips == 0 or dtype_name == "bfloat16"       # (bfloat16: never more than the near-ties, checked by verify)
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,page", [("A", 16), ("B", 8), ("B", 16), ("C", 16), ("D", 16)])
+def test_the_step_program_gives_the_bits_of_the_parts_own_code(model_dirs, name, page, dtype_name):
+    """A step run by the library's step program (one call) and the same step launched kernel by kernel from
+    the parts' Python code choose the same kernels in the same order: equal logits, bit for bit, over whole
+    prompts, portions, single tokens and mixed steps with reused pages."""
+    from tokenmill_amd.replay import ReplaySession
+    from test_gpu_replay import make_requests, mixed, portions, prefill_then_decode, run_trace
+    reqs = make_requests(name, [37, 64, 21, 90, 48, 33, 75, 18], 14)
+    traces = prefill_then_decode(reqs) + portions(reqs) + mixed(reqs, seed=15)
+    program = ReplaySession(model_dirs[name], dtype_name, 4 * 128, page_size=page)
+    parts = ReplaySession(model_dirs[name], dtype_name, 4 * 128, page_size=page)
+    assert program.runner.program is not None
+    parts.runner.program = None
+    for rec in traces:
+        a, b = program.run_step(rec), parts.run_step(rec)
+        assert (a is None) == (b is None)
+        if a is not None:
+            assert (a == b).all(), f"step {rec['step']} of {len(traces)}"
+    assert program.runner.program.runs == len(traces)

@@ -89,16 +89,11 @@ def test_every_cut_at_the_layer_sizes_of_the_published_shapes(layer_models, monk
     they are used again: the fast paths of the real sizes (head size 64 and 128, groups of 7, the products
     that start at the norm, and for steps of 17 to 48 rows the products that keep the input in LDS) under
     every way of cutting, against the plain implementation."""
-    from tokenmill_amd.hip import ops
     from tokenmill_amd.replay import ReplaySession
     from test_gpu_replay import assert_all_given_back, check, mixed, portions, prefill_then_decode, run_trace, whole
 
     d, plain = layer_models(name)
     dt = {"float32": torch.float32, "bfloat16": torch.bfloat16}[dtype_name]
-    calls = {"panel": 0, "fused": 0}
-    real_panel, real_fused = ops.panel_qkv_rope, ops.fused_norm_qkv_rope
-    monkeypatch.setattr(ops, "panel_qkv_rope", lambda *a, **k: (calls.__setitem__("panel", calls["panel"] + 1), real_panel(*a, **k))[1])
-    monkeypatch.setattr(ops, "fused_norm_qkv_rope", lambda *a, **k: (calls.__setitem__("fused", calls["fused"] + 1), real_fused(*a, **k))[1])
     lengths = [70, 41, 100, 56, 33, 88, 120, 64]
     reqs = {f"r{i}": random_ids(n, 1000, 600 + i) for i, n in enumerate(lengths)}
     session = ReplaySession(d, dtype_name, 4 * 128)            # four live requests of at most 128 tokens: 32 pages
@@ -111,8 +106,18 @@ def test_every_cut_at_the_layer_sizes_of_the_published_shapes(layer_models, monk
         got = run_trace(session, trace)
         check(got, plain, reqs, dt, f"{name} layers, {dtype_name}, {what}")
         assert_all_given_back(session)
+    took = session.runner.program.counters()
     if dtype_name == "bfloat16":
-        assert calls["fused"] > 0
-        assert calls["panel"] > 0 or name == "7B"             # a width of 3,584 does not fit a block's LDS
+        assert took["qkv_from_norm"] > 0 and took["gate_up_from_norm"] > 0 and took["qkv_plain"] > 0
+        assert took["qkv_panel"] > 0 or name == "7B"          # a width of 3,584 does not fit a block's LDS
+    else:
+        assert took["qkv_plain"] > 0 and took["qkv_from_norm"] == 0
+    # the same mixed trace launched from the parts' own code: the same bits
+    by_parts = ReplaySession(d, dtype_name, 4 * 128)
+    by_parts.runner.program = None
+    again = run_trace(by_parts, steps)
+    for key, row in run_trace(session, steps).items():
+        assert torch.equal(row, again[key]), f"{name} layers, {dtype_name}: {key}"
+    del by_parts
     del session
     torch.cuda.empty_cache()

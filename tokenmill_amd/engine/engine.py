@@ -54,7 +54,7 @@ class LLMEngine:
         pages = num_cache_pages(cfg, model, self.dtype, self.device)
         self.pools = CachePools(model, pages, cfg.block_size, cfg.max_num_seqs, self.dtype, self.device)
         self.cache = CacheManager(self.pools.windows, pages, cfg.block_size, cfg.max_num_seqs, cfg.watermark)
-        self.runner = ModelRunner(model, self.pools, max_positions=cfg.max_model_len)
+        self.runner = ModelRunner(model, self.pools, max_positions=cfg.max_model_len, step_program=cfg.step_program)
         if cfg.hip_graphs:
             from tokenmill_amd.engine.graphs import DecodeGraphs, StepGraphs
             self.runner.graphs = DecodeGraphs(self.runner, cfg)

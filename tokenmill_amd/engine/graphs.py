@@ -175,12 +175,12 @@ class DecodeGraphs:
         side.wait_stream(torch.cuda.current_stream())
         # a first run outside the graph: lazy set-up happens here, and the library's products are timed now
         with torch.cuda.stream(side), ops.gemm_library_tune_at_once():
-            runner.model.forward(step, runner.pools.views)
+            runner.forward(step)
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
-            bk.logits = runner.model.forward(step, runner.pools.views)
+            bk.logits = runner.forward(step)
         bk.graph = graph
 
 
@@ -288,11 +288,11 @@ class StepGraphs:
         side.wait_stream(torch.cuda.current_stream())
         # a first run outside the graph: lazy set-up happens here, and the library's products are timed now
         with torch.cuda.stream(side), ops.gemm_library_tune_at_once():
-            runner.model.forward(step, runner.pools.views)
+            runner.forward(step)
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
-            slot.logits = runner.model.forward(step, runner.pools.views)
+            slot.logits = runner.forward(step)
         slot.graph = graph
         return slot

@@ -16,6 +16,7 @@ from dataclasses import dataclass, field
 import numpy as np
 import torch
 
+from tokenmill_amd import profiling
 from tokenmill_amd.cache.manager import RELEASED, RequestCache
 from tokenmill_amd.cache.pool import CachePools
 from tokenmill_amd.parts.base import GroupStep, StepContext
@@ -35,9 +36,14 @@ class StepError(ValueError):
 
 
 class ModelRunner:
-    def __init__(self, model, pools: CachePools, max_positions: int):
+    def __init__(self, model, pools: CachePools, max_positions: int, step_program: bool = True):
         self.model = model
         self.pools = pools
+        # the model's launch sequence as one call into the kernel library, where every part has an operation there
+        self.program = None
+        if step_program and getattr(model, "run", None) is not None and getattr(model, "dtype", None) is not None:
+            from tokenmill_amd.engine.program import StepProgram
+            self.program = StepProgram.compile(model, pools)
         self.page_size = pools.page_size
         self.max_positions = max_positions
         self.device = model.device
@@ -302,4 +308,11 @@ class ModelRunner:
             if logits is not None:
                 return logits
         ctx, _ = self.prepare(entries)
-        return self.model.forward(ctx, self.pools.views)
+        return self.forward(ctx)
+
+    def forward(self, step: StepContext) -> torch.Tensor:
+        """The step's float32 logits [R, vocab]: through the library's step program where the model has
+        one, else (and while per-operation times are being collected) through the parts' own code."""
+        if self.program is not None and not profiling.on():
+            return self.program.run(step)
+        return self.model.forward(step, self.pools.views)
