@@ -278,6 +278,13 @@ def build_toy_state_model(cfg: ToyConfig, max_positions=None):
 
         def forward(self, x, step, cache, residual=None):
             x = as_tensor(x)
+            if step.max_q_len == 1:
+                # single tokens: index operations on the device alone, which a HIP graph can record (the
+                # padding rows of a replayed step carry a slot that belongs to no request)
+                slots = step.state_slots.long()
+                state = cache.state.index_select(0, slots) * self.decay + x.float()
+                cache.state.index_copy_(0, slots, state)
+                return self.proj.forward(state.to(x.dtype))
             out = torch.empty_like(x)
             cu = step.cu_q_lens.tolist()
             slots = step.state_slots.tolist()
@@ -350,6 +357,30 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path, dtype_na
             assert_logits_close(row, want, dt, f"toy state model, {name}, {rid} position {p}", noise)
         session.manager.check_invariants()
         assert not session.manager.live
+    # through the engine: the decode steps of a model with per-request state replay from graphs like any
+    # other's (this mixer's single-token path is capturable), with requests coming and going in the batch;
+    # a mixer that does not say so turns the graphs off for its model, loudly, and the tokens are the same
+    from tokenmill_amd import EngineConfig, LLMEngine, SamplingParams
+    prompts = [random_ids(n, 200, 350 + i) for i, n in enumerate([12, 3, 30, 7, 21, 16, 9, 25, 5, 18])]
+    params = [SamplingParams(max_tokens=6 + 3 * (i % 4), ignore_eos=True) for i in range(len(prompts))]
+    outs = {}
+    for mode in ("eager", "graphs", "refused"):
+        eng = LLMEngine(EngineConfig(model=str(d), dtype=dtype_name, block_size=8, num_blocks=64, max_model_len=64,
+                                     max_num_seqs=4, max_num_batched_tokens=64, watermark=0.0, hip_graphs=mode != "eager"))
+        assert eng.runner.program is None                     # a mixer the library's step program does not know
+        if mode == "refused":
+            for layer in eng.model.layers[::2]:
+                layer.mixer.capturable = False
+            from tokenmill_amd.engine.graphs import DecodeGraphs
+            eng.runner.graphs = DecodeGraphs(eng.runner, eng.cfg)
+            assert not eng.runner.graphs.stateful_ok
+        outs[mode] = eng.generate(prompts, params)
+        if mode == "graphs":
+            assert eng.runner.graphs.replays > 10
+        if mode == "refused":
+            assert eng.runner.graphs.replays == 0
+        assert eng.cache.num_free_pages == eng.cache.num_pages
+    assert outs["graphs"] == outs["eager"] == outs["refused"]
 
 
 # ----------------------------------------------------------------------------------------------- windows, a layer twice, a shared cache

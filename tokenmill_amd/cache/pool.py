@@ -49,13 +49,19 @@ class CachePools:
                 views[j] = KVCacheView(self.k[g][idx], self.v[g][idx], g, True)
         for j, spec in enumerate(specs):
             if isinstance(spec, StateSpec):
-                self.states[j] = torch.zeros((num_state_slots, *spec.shape), dtype=spec.dtype, device=device)
+                # one row more than there are slots: where the padding rows of a replayed step put their state
+                self.states[j] = torch.zeros((num_state_slots + 1, *spec.shape), dtype=spec.dtype, device=device)
                 views[j] = StateView(self.states[j])
         for j, call in enumerate(model.run):
             if call.cache_of is not None:
                 src = views[call.cache_of]
                 views[j] = KVCacheView(src.k, src.v, src.group, False) if isinstance(src, KVCacheView) else src
         self.views = views
+
+    @property
+    def padding_state_slot(self) -> int:
+        """The state row that belongs to no request."""
+        return self.num_state_slots
 
     @property
     def windows(self) -> list[int | None]:

@@ -86,10 +86,19 @@ class DecodeGraphs:
         self.failed: set[int] = set()                       # bucket sizes whose capture failed: those steps run eagerly
         self.replays = 0
         self._copied = torch.cuda.Event()
+        # A model with per-request state replays its decode steps too (the slot of each row is data like its
+        # block table; a row of padding updates a slot that belongs to nobody), if its mixers say that they
+        # can be recorded. Otherwise every step of it runs kernel by kernel, and that is said once, here.
+        model = runner.model
+        holders = [model.layers[call.layer].mixer for j, call in enumerate(model.run) if j in runner.pools.states]
+        refusing = [type(m).__name__ for m in holders if not getattr(m, "capturable", False)]
+        self.stateful_ok = not refusing
+        if refusing:
+            log.warning("HIP graphs are off for this model: %s keeps per-request state and does not declare itself "
+                        "capturable; its steps are launched kernel by kernel", ", ".join(sorted(set(refusing))))
 
     def can_run(self, entries) -> bool:
-        return (0 < len(entries) <= self.sizes[-1] and all(len(e.tokens) == 1 for e in entries)
-                and not self.runner.pools.states)
+        return 0 < len(entries) <= self.sizes[-1] and all(len(e.tokens) == 1 for e in entries) and self.stateful_ok
 
     def _bucket(self, n: int) -> _Bucket:
         B = next(b for b in self.sizes if b >= n)
@@ -123,7 +132,7 @@ class DecodeGraphs:
         ctx[n:] = 1
         host[bk.ctx[0]:bk.ctx[1]] = ctx
         state = host[bk.state[0]:bk.state[1]]
-        state[:] = 0
+        state[:] = runner.pools.padding_state_slot
         state[:n] = [e.cache.state_slot for e in entries]
         for g in range(len(runner.pools.groups)):
             slots = host[bk.g_slot[g][0]:bk.g_slot[g][1]]
@@ -171,6 +180,12 @@ class DecodeGraphs:
         runner = self.runner
         step = bk.context(self.max_positions)
         torch.cuda.synchronize()
+        # The run before the capture really executes: keys and values written twice are the same keys and
+        # values, but per-request state would be advanced twice. For that run every row's state is the
+        # row that belongs to nobody; the requests' own slots come back before the replay.
+        slots = bk.view(bk.state)
+        real_slots = slots.clone()
+        slots.fill_(runner.pools.padding_state_slot)
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         # a first run outside the graph: lazy set-up happens here, and the library's products are timed now
@@ -181,6 +196,7 @@ class DecodeGraphs:
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             bk.logits = runner.forward(step)
+        slots.copy_(real_slots)
         bk.graph = graph
 
 
@@ -234,7 +250,7 @@ class StepGraphs:
 
     def can_run(self, entries) -> bool:
         if self.runner.pools.states:
-            return False
+            return False        # state is advanced token by token inside a portion, from the host's view of the step
         portions = sum(1 for e in entries if len(e.tokens) > 1)
         if portions == 0 or len(entries) - portions > self.max_singles or any(len(e.want) > 1 for e in entries):
             return False

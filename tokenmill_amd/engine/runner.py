@@ -149,7 +149,7 @@ class ModelRunner:
             pos[:] = 0
             seq_of[:] = 0
             ctx_lens[:] = 1
-            slots_state[:] = 0
+            slots_state[:] = self.pools.padding_state_slot
             rows[:] = 0
             for g in range(n_groups):
                 g_slot[g][0][:] = -1

@@ -158,6 +158,12 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
+    # Can a step of single tokens through this mixer be recorded into a HIP graph? Yes if ``forward`` works on
+    # the step's device tensors alone for such a step (index operations with ``state_slots``, kernels);
+    # no if it needs their values on the host (``.tolist()``, ``.item()``) or allocates by them. Only asked
+    # of mixers with per-request state: their decode steps are then replayed like any other model's.
+    capturable = True
+
     def cache_spec(self) -> KVCacheSpec | StateSpec | None:
         return None
 
