@@ -147,6 +147,41 @@ def test_gemm_tiled(ops, dt, M, N, K):
     assert torch.equal(one[0], out32[M - 1])
 
 
+@pytest.mark.parametrize("M,N,K", [(17, 896, 896), (300, 1152, 896), (2048, 9728, 896), (130, 896, 4864), (70, 308, 120),
+                                   (1, 64, 32), (129, 132, 20)])
+def test_gemm_f32_on_the_matrix_unit(ops, M, N, K):
+    """The float32 product of prompt-sized steps: as exact as a chain of 32-bit multiply-adds in ascending k
+    (this kernel and the vector-unit kernel it stands in for are both held against a 64-bit product; it may be
+    as far from it as that kernel plus one rounding of the largest value: the matrix unit must not lose digits
+    the multiply-add chain keeps), bias added, row-strided operands, and a row's bits do not depend on the other
+    rows of the call or on the tile shape they put it in."""
+    torch.manual_seed(41)
+    a, w, b = torch.randn(M, K), torch.randn(N, K) * 0.1, torch.randn(N)
+    want = (a.double() @ w.double().t())
+    out = torch.empty(M, N, device=DEV)
+    ops.gemm_f32_mfma(a.to(DEV), w.to(DEV), None, out)
+    chain = torch.empty(M, N, device=DEV)
+    ops.gemm_nt_tiled(a.to(DEV), w.to(DEV), None, chain)
+    chain_err = float((chain.cpu().double() - want).abs().max())
+    # (the two sum in different orders, so their largest errors over millions of elements differ by a few per cent)
+    bound = 1.25 * chain_err + 2.0 ** -23 * float(want.abs().max())
+    err = float((out.cpu().double() - want).abs().max())
+    assert err <= bound
+    ops.gemm_f32_mfma(a.to(DEV), w.to(DEV), b.to(DEV), out)
+    assert float((out.cpu().double() - (want + b.double())).abs().max()) <= bound + 2.0 ** -22
+    wide = torch.zeros(M, K + 12, device=DEV)
+    wide[:, :K] = a.to(DEV)
+    out_w = torch.zeros(M, N + 8, device=DEV)
+    ops.gemm_f32_mfma(wide[:, :K], w.to(DEV), b.to(DEV), out_w[:, :N])
+    assert torch.equal(out_w[:, :N], out) and float(out_w[:, N:].abs().max()) == 0
+    rows = [M - 1] if M < 40 else [0, 37, M - 1]
+    few = torch.empty(len(rows), N, device=DEV)
+    ops.gemm_f32_mfma(a[rows].contiguous().to(DEV), w.to(DEV), b.to(DEV), few)
+    assert torch.equal(few, out[rows])
+    with pytest.raises(ops.KernelArgumentError):
+        ops.gemm_f32_mfma(torch.zeros(4, 18, device=DEV), torch.zeros(8, 18, device=DEV), None, torch.empty(4, 8, device=DEV))
+
+
 def paged_case(dt, lens, q_lens, H, KVH, D, page, seed, spike=None, ramp=None, ramp_slope=1.0):
     """Random requests laid out in shuffled pages. Returns device operands and the CPU truth.
     spike = (request, key[, size]): one far key that carries the request's last query. ramp: a request (or

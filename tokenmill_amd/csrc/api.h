@@ -23,6 +23,13 @@ int tm_convert(const void* in, int in_dtype, void* out, int out_dtype, long long
 int tm_gemm_nt_tiled(const void* A, int lda, const void* W, const void* bias, int bias_dtype, void* C, int ldc,
                      int M, int N, int K, int in_dtype, int out_dtype, hipStream_t stream);
 
+// The float32 product on the 32-bit matrix unit: all operands float32, K, N and the row strides multiples of 4,
+// 16-byte aligned (tm_gemm_f32_mfma_fits says whether a product is taken).
+int tm_gemm_f32_mfma_fits(const void* A, int lda, const void* W, const void* bias, const void* C, int ldc, int M, int N,
+                          int K);
+int tm_gemm_f32_mfma(const float* A, int lda, const float* W, const float* bias, float* C, int ldc, int M, int N, int K,
+                     hipStream_t stream);
+
 int tm_attn_paged_generic(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
                           const void* v_pool, const int* block_tables, int table_width, const int* seq_of_token,
                           const int* positions, int T, int H, int KVH, int D, int page, float scale, int window,

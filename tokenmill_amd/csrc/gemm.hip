@@ -3,8 +3,8 @@
 //                                     src/infer/model/qwen2.py:51-52)
 //
 // gemm_nt_tiled: an LDS-tiled kernel on the vector ALU with 32-bit multiply-adds only. It is the
-// matrix product of the true 32-bit path, and the fallback of the bfloat16 path for shapes its
-// MFMA kernels refuse. Each output element is accumulated over k = 0..K-1 in ascending order by one
+// matrix product of the true 32-bit path for shapes the 32-bit matrix-unit kernel (gemm_f32_mfma.hip)
+// does not take, and the fallback of the bfloat16 path for shapes its MFMA kernels refuse. Each output element is accumulated over k = 0..K-1 in ascending order by one
 // thread, so a row's result does not depend on how many other rows the call holds.
 #include "common.h"
 #include "api.h"

@@ -98,6 +98,9 @@ struct Run {
             const bool gemv = L.dtype == TM_F32 && out_dtype == TM_F32 && (L.bias_dtype == TM_NONE || L.bias_dtype == TM_F32) &&
                               M <= 16 && L.K % 4 == 0 && ldx % 4 == 0 && aligned(x_, 16) && aligned(L.w, 16);
             if (gemv) return tm_gemv_f32((const float*)x_, ldx, (const float*)L.w, (const float*)L.bias, (float*)out, ldc, M, L.N, L.K, stream);
+            if (L.dtype == TM_F32 && out_dtype == TM_F32 && (L.bias_dtype == TM_NONE || L.bias_dtype == TM_F32) &&
+                tm_gemm_f32_mfma_fits(x_, ldx, L.w, L.bias, out, ldc, M, L.N, L.K))
+                return tm_gemm_f32_mfma((const float*)x_, ldx, (const float*)L.w, (const float*)L.bias, (float*)out, ldc, M, L.N, L.K, stream);
             return tm_gemm_nt_tiled(x_, ldx, L.w, L.bias, L.bias_dtype, out, ldc, M, L.N, L.K, dtype, out_dtype, stream);
         }
         const bool skinny = skinny_ok(L, x_, ldx, dtype);

@@ -1,7 +1,8 @@
 """Which matrix-product kernel a Linear runs.
 
-float32: the LDS-tiled kernel with 32-bit multiply-adds (a true 32-bit product, fixed summation
-order), or up to 16 rows a matrix-vector kernel of the same kind that streams the matrix once.
+float32: up to 16 rows a matrix-vector kernel with 32-bit multiply-adds that streams the matrix once;
+beyond that the kernel on the 32-bit matrix unit (32-bit products and sums, a fixed summation order),
+or for shapes it does not take the LDS-tiled kernel on the vector unit (the same guarantees).
 bfloat16: up to 16 rows (decode steps) the MFMA kernels of this library that stream the matrix once
 (from its packed copy where the Linear keeps one) and carry the layer's epilogue (bias, rotary +
 cache write, SiLU·up, residual add) or start at the norm; from 17 to 48 rows the q|k|v and gate|up
@@ -44,6 +45,8 @@ def linear(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, out: tor
     if x.dtype != torch.bfloat16:
         if ops.gemv_f32_ok(x, w, bias, out):                    # a decode step of the 32-bit path
             return ops.gemv_f32(x, w, bias, out)
+        if ops.gemm_f32_mfma_ok(x, w, bias, out):               # a prompt-sized step of it: the 32-bit matrix unit
+            return ops.gemm_f32_mfma(x, w, bias, out)
         return ops.gemm_nt_tiled(x, w, bias, out)
     skinny = _skinny_ok(x, w)
     library = w.dtype == torch.bfloat16 and x.stride(1) == 1 and out.stride(1) == 1

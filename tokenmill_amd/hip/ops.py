@@ -275,6 +275,37 @@ def gemv_f32(a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, out: t
     return out
 
 
+def gemm_f32_mfma_ok(a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, out: torch.Tensor) -> bool:
+    """Does the float32 product on the 32-bit matrix unit take these operands?"""
+    if not (a.dtype == w.dtype == out.dtype == torch.float32 and (bias is None or bias.dtype == torch.float32)
+            and a.dim() == 2 and a.stride(1) == 1 and out.stride(1) == 1 and w.is_contiguous()):
+        return False
+    M, K = a.shape
+    lda = a.stride(0) if M > 1 else max(K, a.stride(0))
+    ldc = out.stride(0) if M > 1 else max(w.shape[0], out.stride(0))
+    return bool(library().tm_gemm_f32_mfma_fits(_p(a), c_int(lda), _p(w), _p(bias), _p(out), c_int(ldc), c_int(M),
+                                                c_int(w.shape[0]), c_int(K)))
+
+
+def gemm_f32_mfma(a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, out: torch.Tensor) -> torch.Tensor:
+    """out[M, N] = a[M, K] @ w[N, K]^T (+ bias[N]), everything float32, on the 32-bit matrix unit: 32-bit
+    products and sums in an order that depends on K only. K, N and the row strides must be multiples of 4
+    and the operands 16-byte aligned."""
+    _gpu(a, w, bias, out)
+    _need(gemm_f32_mfma_ok(a, w, bias, out), "gemm_f32_mfma: float32 operands, K, N and row strides multiples of 4, 16-byte aligned")
+    M, K = a.shape
+    N = w.shape[0]
+    _need(w.shape[1] == K and tuple(out.shape) == (M, N), "gemm_f32_mfma: w [N, K], out [M, N]")
+    if bias is not None:
+        _need(tuple(bias.shape) == (N,) and bias.is_contiguous(), "gemm_f32_mfma: bias must be [N]")
+    _need(M <= 64 * 65535, "gemm_f32_mfma: too many rows for one launch")
+    lda = a.stride(0) if M > 1 else max(K, a.stride(0))
+    ldc = out.stride(0) if M > 1 else max(N, out.stride(0))
+    _check(library().tm_gemm_f32_mfma(_p(a), c_int(lda), _p(w), _p(bias), _p(out), c_int(ldc), c_int(M), c_int(N),
+                                      c_int(K), _stream()), "gemm_f32_mfma")
+    return out
+
+
 def attn_paged_generic(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                        block_tables: torch.Tensor, seq_of_token: torch.Tensor, positions: torch.Tensor,
                        H: int, KVH: int, D: int, scale: float, window: int = 0) -> torch.Tensor:
