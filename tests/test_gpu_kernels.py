@@ -147,8 +147,8 @@ def test_gemm_tiled(ops, dt, M, N, K):
     assert torch.equal(one[0], out32[M - 1])
 
 
-@pytest.mark.parametrize("M,N,K", [(17, 896, 896), (300, 1152, 896), (2048, 9728, 896), (130, 896, 4864), (70, 308, 120),
-                                   (1, 64, 32), (129, 132, 20)])
+@pytest.mark.parametrize("M,N,K", [(17, 896, 896), (300, 1152, 896), (2048, 9728, 896), (130, 896, 4864), (70, 308, 112),
+                                   (1, 64, 32), (129, 132, 16)])
 def test_gemm_f32_on_the_matrix_unit(ops, M, N, K):
     """The float32 product of prompt-sized steps: as exact as a chain of 32-bit multiply-adds in ascending k
     (this kernel and the vector-unit kernel it stands in for are both held against a 64-bit product; it may be

@@ -23,7 +23,7 @@ int tm_convert(const void* in, int in_dtype, void* out, int out_dtype, long long
 int tm_gemm_nt_tiled(const void* A, int lda, const void* W, const void* bias, int bias_dtype, void* C, int ldc,
                      int M, int N, int K, int in_dtype, int out_dtype, hipStream_t stream);
 
-// The float32 product on the 32-bit matrix unit: all operands float32, K, N and the row strides multiples of 4,
+// The float32 product on the 32-bit matrix unit: all operands float32, K a multiple of 16, N and the row strides of 4,
 // 16-byte aligned (tm_gemm_f32_mfma_fits says whether a product is taken).
 int tm_gemm_f32_mfma_fits(const void* A, int lda, const void* W, const void* bias, const void* C, int ldc, int M, int N,
                           int K);

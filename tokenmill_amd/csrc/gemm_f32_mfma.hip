@@ -33,19 +33,27 @@ __global__ __launch_bounds__(256) void gemm_nt_mfma_f32_kernel(const float* __re
     const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
     const int lrow = tid / 4, lq = tid % 4;                   // this thread's row and 4-k piece of a tile
 
+    // No load stands under a test (a tested load is waited for where the test ends, one at a time): rows
+    // beyond the matrices read their first rows instead, and what those give is never stored; K is a
+    // multiple of the tile's 16, so no piece lies beyond it.
     mf_f32x4 ra[A_LOADS], rw[W_LOADS];
+    const float* a_src[A_LOADS];
+    const float* w_src[W_LOADS];
+#pragma unroll
+    for (int e = 0; e < A_LOADS; ++e) {
+        const int m = m0 + lrow + 64 * e;
+        a_src[e] = A + (size_t)(m < M ? m : 0) * lda + 4 * lq;
+    }
+#pragma unroll
+    for (int e = 0; e < W_LOADS; ++e) {
+        const int n = n0 + lrow + 64 * e;
+        w_src[e] = W + (size_t)(n < N ? n : 0) * K + 4 * lq;
+    }
     auto gload = [&](int k0) {
-        const int k = k0 + 4 * lq;
 #pragma unroll
-        for (int e = 0; e < A_LOADS; ++e) {
-            const int m = m0 + lrow + 64 * e;
-            ra[e] = (m < M && k < K) ? *(const mf_f32x4*)(A + (size_t)m * lda + k) : mf_f32x4{0.f, 0.f, 0.f, 0.f};
-        }
+        for (int e = 0; e < A_LOADS; ++e) ra[e] = *(const mf_f32x4*)(a_src[e] + k0);
 #pragma unroll
-        for (int e = 0; e < W_LOADS; ++e) {
-            const int n = n0 + lrow + 64 * e;
-            rw[e] = (n < N && k < K) ? *(const mf_f32x4*)(W + (size_t)n * K + k) : mf_f32x4{0.f, 0.f, 0.f, 0.f};
-        }
+        for (int e = 0; e < W_LOADS; ++e) rw[e] = *(const mf_f32x4*)(w_src[e] + k0);
     };
     auto sstore = [&](int buf) {
 #pragma unroll
@@ -104,10 +112,10 @@ __global__ __launch_bounds__(256) void gemm_nt_mfma_f32_kernel(const float* __re
     }
 }
 
-// Can the matrix-unit kernel take this product? (float32 everywhere, rows 16-byte aligned and whole 4-element pieces)
+// Can the matrix-unit kernel take this product? (float32 everywhere, K a multiple of 16, N of 4, rows 16-byte aligned)
 extern "C" int tm_gemm_f32_mfma_fits(const void* A, int lda, const void* W, const void* bias, const void* C, int ldc,
                                      int M, int N, int K) {
-    return M > 0 && N > 0 && K > 0 && K % 4 == 0 && N % 4 == 0 && lda % 4 == 0 && ldc % 4 == 0 && lda >= K && ldc >= N &&
+    return M > 0 && N > 0 && K > 0 && K % MF_BK == 0 && N % 4 == 0 && lda % 4 == 0 && ldc % 4 == 0 && lda >= K && ldc >= N &&
            ((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0 && ((uintptr_t)C % 16) == 0 && ((uintptr_t)bias % 16) == 0;
 }
 

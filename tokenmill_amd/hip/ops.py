@@ -289,10 +289,10 @@ def gemm_f32_mfma_ok(a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None
 
 def gemm_f32_mfma(a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, out: torch.Tensor) -> torch.Tensor:
     """out[M, N] = a[M, K] @ w[N, K]^T (+ bias[N]), everything float32, on the 32-bit matrix unit: 32-bit
-    products and sums in an order that depends on K only. K, N and the row strides must be multiples of 4
+    products and sums in an order that depends on K only. K must be a multiple of 16, N and the row strides of 4,
     and the operands 16-byte aligned."""
     _gpu(a, w, bias, out)
-    _need(gemm_f32_mfma_ok(a, w, bias, out), "gemm_f32_mfma: float32 operands, K, N and row strides multiples of 4, 16-byte aligned")
+    _need(gemm_f32_mfma_ok(a, w, bias, out), "gemm_f32_mfma: float32 operands, K a multiple of 16, N and row strides of 4, 16-byte aligned")
     M, K = a.shape
     N = w.shape[0]
     _need(w.shape[1] == K and tuple(out.shape) == (M, N), "gemm_f32_mfma: w [N, K], out [M, N]")
