@@ -1,14 +1,16 @@
 // Paged attention for portions of prompts in true 32-bit, flash style on the 32-bit MFMA
 // (v_mfma_f32_16x16x4_f32: 32-bit inputs, 32-bit products and sums; no reduced-precision mode).
 //
-//   A wavefront takes 16 consecutive query tokens of one request (a "tile") and one query head and
-//   walks the keys its tile may see in blocks of 16, in ascending position, with an online softmax:
-//   a query at position p sees keys lo..p, lo = 0 or p - window + 1
+//   A block takes 16 consecutive query tokens of one request (a "tile") and one query head. The keys
+//   the tile may see are cut into blocks of 16 at absolute positions; the block's four wavefronts take
+//   every fourth key block each (key block kb goes to wavefront kb % 4), in ascending position with an
+//   online softmax of their own, and their four partial results are merged through LDS in the order of
+//   the wavefronts: a query at position p sees keys lo..p, lo = 0 or p - window + 1
 //                               (reference src/infer/kv/context.py:70-75, src/infer/model/layers.py:100-107).
-//   The four wavefronts of a block are four heads that share a kv head, on the same tile: they read
-//   the same keys and values at about the same time, so those come from the CU's cache after the
-//   first. Key blocks are aligned to absolute positions and no sum is split between wavefronts, so a
-//   token's result depends on its request only.
+//   Which wavefront takes a key block hangs on the key's position only, so a token's result depends
+//   on its request only. The longest tile of a 2,048-token prompt walks 32 key blocks a wavefront
+//   instead of 128; the heads of a kv head run in blocks of their own and share its keys through the
+//   second-level cache.
 //
 //   S^T = K Q^T   A = keys  [16 keys x 4 d]   B = Q^T [4 d x 16 tokens]   (D / 4 steps; the lanes of
 //                 group g = lane / 16 hold d = g D/4 .. (g + 1) D/4 - 1 of their key / token, so a
@@ -21,10 +23,10 @@
 
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
-#define AF_HEADS 4          // wavefronts of a block = query heads of one kv head
+#define AF_SPLIT 4          // wavefronts of a block; each takes every fourth key block
 
 template <int D>
-__global__ __launch_bounds__(64 * AF_HEADS) void attn_prefill_f32_kernel(
+__global__ __launch_bounds__(64 * AF_SPLIT) void attn_prefill_f32_kernel(
     const float* __restrict__ q, int q_stride, float* __restrict__ out, int out_stride,
     const float* __restrict__ k_pool, const float* __restrict__ v_pool, const int* __restrict__ block_tables,
     int table_width, const int* __restrict__ tiles, int H, int KVH, int page_shift, float scale, int window) {
@@ -32,12 +34,8 @@ __global__ __launch_bounds__(64 * AF_HEADS) void attn_prefill_f32_kernel(
     constexpr int NDT = D / 16;         // 16-row tiles of d
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / TM_WAVE);
     const int lane = threadIdx.x % TM_WAVE, r = lane % 16, g = lane / 16;
-    const int G = H / KVH;
-    const int splits = (G + AF_HEADS - 1) / AF_HEADS;
-    const int kvh = blockIdx.y / splits;
-    const int hg = (blockIdx.y % splits) * AF_HEADS + wave;             // this wavefront's head within the group
-    if (hg >= G) return;                                                // (no block-wide barrier in this kernel)
-    const int h = kvh * G + hg;
+    const int h = blockIdx.y;
+    const int kvh = h / (H / KVH);
     const int* tl = tiles + (size_t)blockIdx.x * 4;
     const int s = tl[0], row0 = tl[1], valid = tl[2], pos0 = tl[3];
     const int* table = block_tables + (size_t)s * table_width;
@@ -60,7 +58,9 @@ __global__ __launch_bounds__(64 * AF_HEADS) void attn_prefill_f32_kernel(
 #pragma unroll
     for (int dt = 0; dt < NDT; ++dt) o[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-    for (int key0 = first_key & ~15; key0 <= last_key; key0 += 16) {
+    const int kb_first = first_key >> 4, kb_last = last_key >> 4;
+    for (int kb = kb_first + ((wave - kb_first) & (AF_SPLIT - 1)); kb <= kb_last; kb += AF_SPLIT) {
+        const int key0 = kb << 4;
         const int pg = table[key0 >> page_shift];
         const int in_page = key0 & (page - 1);
         // keys: lane (r, g) holds K[key0 + r][g DQ .. g DQ + DQ - 1]
@@ -124,12 +124,41 @@ __global__ __launch_bounds__(64 * AF_HEADS) void attn_prefill_f32_kernel(
     // o[dt][i] = sum for d = 16 dt + 4 g + i of token r; the column's sum is spread over its four lanes
     l += __shfl_xor(l, 16, TM_WAVE);
     l += __shfl_xor(l, 32, TM_WAVE);
-    if (r < valid) {
-        const float inv = 1.f / l;
-        float* orow = out + (size_t)(row0 + r) * out_stride + (size_t)h * D;
+    // the four wavefronts' partial results meet in LDS; a wavefront that had no key block brings m = -inf, l = 0, o = 0
+    __shared__ float m_s[AF_SPLIT][16], l_s[AF_SPLIT][16];
+    __shared__ __attribute__((aligned(16))) float o_s[AF_SPLIT][16][D + 4];
+    if (g == 0) {
+        m_s[wave][r] = m;
+        l_s[wave][r] = l;
+    }
 #pragma unroll
-        for (int dt = 0; dt < NDT; ++dt)
-            *(f32x4_t*)(orow + 16 * dt + 4 * g) = f32x4_t{o[dt][0] * inv, o[dt][1] * inv, o[dt][2] * inv, o[dt][3] * inv};
+    for (int dt = 0; dt < NDT; ++dt) *(f32x4_t*)&o_s[wave][r][16 * dt + 4 * g] = o[dt];
+    __syncthreads();
+    const int tok = threadIdx.x >> 4;
+    if (tok < valid) {
+        float mw[AF_SPLIT], sw[AF_SPLIT], top = -INFINITY, sum = 0.f;
+#pragma unroll
+        for (int w = 0; w < AF_SPLIT; ++w) {
+            mw[w] = m_s[w][tok];
+            top = fmaxf(top, mw[w]);
+        }
+#pragma unroll
+        for (int w = 0; w < AF_SPLIT; ++w) {
+            sw[w] = (mw[w] == -INFINITY) ? 0.f : expf(mw[w] - top);     // a token always sees its own key: top is finite
+            sum += l_s[w][tok] * sw[w];
+        }
+        const float inv = 1.f / sum;
+        float* orow = out + (size_t)(row0 + tok) * out_stride + (size_t)h * D;
+        for (int d = (threadIdx.x & 15) * 4; d < D; d += 64) {
+            f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int w = 0; w < AF_SPLIT; ++w) {
+                const f32x4_t part = *(const f32x4_t*)&o_s[w][tok][d];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[i] += part[i] * sw[w];
+            }
+            *(f32x4_t*)(orow + d) = f32x4_t{acc[0] * inv, acc[1] * inv, acc[2] * inv, acc[3] * inv};
+        }
     }
 }
 
@@ -145,15 +174,13 @@ extern "C" int tm_attn_prefill_f32(const void* q, int q_stride, void* out, int o
         (q_stride % 4) || (out_stride % 4) || ((uintptr_t)q % 16) || ((uintptr_t)out % 16) || ((uintptr_t)k_pool % 16) ||
         ((uintptr_t)v_pool % 16) || q_stride < H * D || out_stride < H * D || !(scale > 0.f))
         return TM_ERR_ARG;
-    const int G = H / KVH;
-    const int splits = (G + AF_HEADS - 1) / AF_HEADS;
-    if ((long long)KVH * splits > 65535) return TM_ERR_ARG;
+    if (H > 65535) return TM_ERR_ARG;
     int page_shift = 0;
     while ((1 << page_shift) < page) ++page_shift;
-    dim3 grid(n_tiles, KVH * splits);
+    dim3 grid(n_tiles, H);
 #define TM_PREFILL_F32_CASE(DD)                                                                                   \
     case DD:                                                                                                      \
-        attn_prefill_f32_kernel<DD><<<grid, 64 * AF_HEADS, 0, stream>>>(                                          \
+        attn_prefill_f32_kernel<DD><<<grid, 64 * AF_SPLIT, 0, stream>>>(                                          \
             (const float*)q, q_stride, (float*)out, out_stride, (const float*)k_pool, (const float*)v_pool,       \
             block_tables, table_width, tiles, H, KVH, page_shift, scale, window);                                 \
         break
