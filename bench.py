@@ -56,6 +56,8 @@ def main() -> int:
     ap.add_argument("--config", default=None, help="a config.json or a shipped shape's name (7b, 32b): run it instead of the 0.5B shape")
     ap.add_argument("--no-graphs", action="store_true", help="launch decode steps kernel by kernel")
     ap.add_argument("--no-tune", action="store_true", help="keep the library's first choice of matrix-product algorithm")
+    ap.add_argument("--tune-every", action="store_true",
+                    help="captured shapes also try every algorithm the library holds, not only its heuristic's candidates")
     ap.add_argument("--skip-points", action="store_true", help="only the headline batch and the prefill")
     ap.add_argument("--skip-kernels", action="store_true", help="no per-operation kernel trace")
     ap.add_argument("--part", default="all", choices=["all", "decode", "prefill", "offline", "mixed7b", "preempt32b"],
@@ -112,7 +114,7 @@ def main() -> int:
         pages = batch * (-(-(prompt_len + args.steps + args.warmup + extra_steps + 64) // BLOCK_SIZE)) + 8
         cfg = EngineConfig(dtype=args.dtype, block_size=BLOCK_SIZE, num_blocks=pages, max_model_len=max_model_len,
                            max_num_seqs=max(batch, 1), max_num_batched_tokens=max(prompt_len, batch),
-                           watermark=0.0, hip_graphs=not args.no_graphs, tune_gemm=not args.no_tune)
+                           watermark=0.0, hip_graphs=not args.no_graphs, tune_gemm=not args.no_tune, tune_gemm_every=args.tune_every and not args.no_tune)
         return LLMEngine(cfg, model=model)
 
     def account(fn) -> tuple[float, float]:
@@ -231,7 +233,7 @@ def main() -> int:
         cfg = EngineConfig(dtype=args.dtype, block_size=BLOCK_SIZE, num_blocks=args.offline_seqs * per_seq + 64,
                            max_model_len=max_model_len, max_num_seqs=args.offline_seqs, max_num_batched_tokens=2048,
                            enable_chunked_prefill=args.chunked, hip_graphs=not args.no_graphs,
-                           tune_gemm=not args.no_tune)
+                           tune_gemm=not args.no_tune, tune_gemm_every=args.tune_every and not args.no_tune)
         eng = LLMEngine(cfg, model=model)
         sp = SamplingParams(max_tokens=args.offline_gen, ignore_eos=True)
         serve(eng, prompts(min(n, 2 * args.offline_seqs), args.offline_prompt), sp)
@@ -247,7 +249,7 @@ def main() -> int:
         pages = seqs * (-(-(4096 + gen_tokens) // BLOCK_SIZE)) + 64
         cfg = EngineConfig(dtype=args.dtype, block_size=BLOCK_SIZE, num_blocks=pages, max_model_len=max_model_len,
                            max_num_seqs=seqs, max_num_batched_tokens=budget, enable_chunked_prefill=True,
-                           hip_graphs=not args.no_graphs, tune_gemm=not args.no_tune)
+                           hip_graphs=not args.no_graphs, tune_gemm=not args.no_tune, tune_gemm_every=args.tune_every and not args.no_tune)
         eng = LLMEngine(cfg, model=model)
         sp = SamplingParams(max_tokens=gen_tokens, ignore_eos=True)
         serve(eng, [prompts(1, L)[0] for L in lengths[:8]], SamplingParams(max_tokens=8, ignore_eos=True))    # warm-up
@@ -272,7 +274,7 @@ def main() -> int:
         n, gen_tokens, pages = args.requests or 64, 64, 8192
         cfg = EngineConfig(dtype=args.dtype, block_size=BLOCK_SIZE, num_blocks=pages, max_model_len=max_model_len,
                            max_num_seqs=n, max_num_batched_tokens=2048, watermark=0.0,
-                           hip_graphs=not args.no_graphs, tune_gemm=not args.no_tune)
+                           hip_graphs=not args.no_graphs, tune_gemm=not args.no_tune, tune_gemm_every=args.tune_every and not args.no_tune)
         eng = LLMEngine(cfg, model=model)
         sp = SamplingParams(max_tokens=gen_tokens, ignore_eos=True)
         serve(eng, prompts(2), SamplingParams(max_tokens=4, ignore_eos=True))                                 # warm-up
@@ -329,7 +331,7 @@ def main() -> int:
         "dtype": "bf16" if dtype == torch.bfloat16 else "fp32", "data": "synthetic token ids, random weights",
         "config": {**sizes(), "global_batch": args.batch, "seq_len": prompt_len, "context": dec["context"],
                    "max_model_len": max_model_len, "block_size": BLOCK_SIZE, "parallelism": "single GPU",
-                   "hip_graphs": not args.no_graphs, "tune_gemm": not args.no_tune, "packed_weights": True},
+                   "hip_graphs": not args.no_graphs, "tune_gemm": ("every" if args.tune_every else True) if not args.no_tune else False, "packed_weights": True},
         "prefill": {"value": round(prompt_len / pre["s"], 1), "tokens": prompt_len, "ms": round(pre["s"] * 1e3, 3),
                     "frac": round(pre["flops"] / pre["s"] / profiling.PEAK_FLOPS_S[args.dtype], 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": peak_gbs, "unit": "GB/s",

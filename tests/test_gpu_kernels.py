@@ -601,6 +601,34 @@ def test_gemm_library(ops, M, N, K, tune, after):
         ops.gemm_library_tune(0)
 
 
+@pytest.mark.parametrize("M,N,K", [(64, 896, 4864), (333, 1152, 896)])
+def test_gemm_library_tries_every_algorithm(ops, M, N, K):
+    """With `every`, a shape timed at its first call also runs each algorithm the library holds for the
+    operand types once and times the fastest few; whichever is kept, the product is the product:
+    with a bias, with float32 out, at a shape whose matrix comes from memory (timed with flushed
+    caches) and at one whose rows dominate."""
+    torch.manual_seed(14)
+    dt = torch.bfloat16
+    a, w, b = q(torch.randn(M, K), dt), q(torch.randn(N, K) * 0.1, dt), q(torch.randn(N), dt)
+    want = a @ w.t()
+    da, dw, db = a.to(dt).to(DEV), w.to(dt).to(DEV), b.to(dt).to(DEV)
+    ops.gemm_library_tune(8, 1, every=True)
+    try:
+        for bias, add in ((db, b), (None, 0.0)):
+            out = torch.full((M, N), 7.0, dtype=dt, device=DEV)
+            assert ops.gemm_library(da, dw, bias, out)
+            torch.testing.assert_close(out.float().cpu(), q(want + add, dt), **tol(dt))
+            again = torch.empty_like(out)
+            assert ops.gemm_library(da, dw, bias, again) and torch.equal(again, out)
+        out32 = torch.full((M, N), 7.0, dtype=torch.float32, device=DEV)
+        assert ops.gemm_library(da, dw, None, out32)
+        torch.testing.assert_close(out32.cpu(), want, rtol=1e-4, atol=1e-4 * K ** 0.5)
+    finally:
+        ops.gemm_library_tune(0)
+    with pytest.raises(ops.KernelArgumentError):
+        ops.gemm_library_tune(0, 1, every=True)
+
+
 def test_gemm_library_takes_a_candidate_whose_workspace_fits(ops):
     """At 8,192 rows of the gate|up product the library's first choice asks for more workspace than it is
     given: the plan takes the first candidate that fits instead of refusing the shape (a refused shape

@@ -75,7 +75,7 @@ int tm_attn_prefill_mfma(const void* q, int q_stride, void* out, int out_stride,
 int tm_gemv_f32(const float* A, int lda, const float* W, const float* bias, float* C, int ldc, int M, int N, int K,
                 hipStream_t stream);
 
-int tm_gemm_library_tune(int n, int after);
+int tm_gemm_library_tune(int n, int after, int every);
 int tm_gemm_library(const void* A, int lda, const void* W, int ldw, const void* bias, int bias_dtype, void* C, int ldc,
                     int out_f32, int M, int N, int K, void* workspace, size_t workspace_bytes, hipStream_t stream);
 

@@ -11,11 +11,16 @@
 // leading dimension lda; result [N, M] with leading dimension ldc. The bias has one entry per row
 // of that result, i.e. per output feature, and is added to the 32-bit sum before rounding.
 #include <hipblaslt/hipblaslt.h>
+#include <hipblaslt/hipblaslt-ext.hpp>
 
+#include <algorithm>
 #include <cstdio>
 #include <cstdlib>
+#include <cstring>
 #include <mutex>
 #include <unordered_map>
+#include <utility>
+#include <vector>
 
 #include "common.h"
 #include "api.h"
@@ -74,6 +79,11 @@ Library& lib() {
 // With TOKENMILL_TUNE_LOG set in the environment every timing is printed to stderr.
 int g_tune_candidates = 0;
 int g_tune_after = 3;
+// Beyond the heuristic's candidates, a shape that is timed at its first call (its caller is about to
+// replay it from a graph) also has every algorithm the library holds for the operand types tried:
+// one quick run each, the fastest few timed like the heuristic's candidates. About a second a shape.
+bool g_tune_every = false;
+constexpr int SHORT_LIST = 12;
 
 struct Operands {
     const void *A, *W, *bias;
@@ -104,7 +114,7 @@ void* flush_buffer(int device) {
 // whichever algorithm wrote it last, up to rounding); with `flush` each run follows a flush of the
 // caches. Negative if it fails.
 float time_algo(hipblasLtHandle_t handle, const Plan& p, const hipblasLtMatmulAlgo_t& algo, const Operands& op,
-                void* flush) {
+                void* flush, bool quick = false) {
     const float one = 1.f, zero = 0.f;
     hipEvent_t t0, t1;
     if (hipEventCreate(&t0) != hipSuccess) return -1.f;
@@ -112,7 +122,7 @@ float time_algo(hipblasLtHandle_t handle, const Plan& p, const hipblasLtMatmulAl
         hipEventDestroy(t0);
         return -1.f;
     }
-    const int WARM = 2, TIMED = flush ? 5 : 20;
+    const int WARM = quick ? 1 : 2, TIMED = quick ? (flush ? 1 : 3) : (flush ? 5 : 20);
     float total = 0.f;
     bool ok = true;
     if (!flush) {       // operands in cache: the runs follow each other without a gap, one time for all of them
@@ -195,54 +205,156 @@ bool make_plan(hipblasLtHandle_t handle, const PlanKey& k, size_t workspace_byte
     return p.ok;
 }
 
+// Every algorithm the library holds for the plan's types that takes this product, short-listed by one
+// quick run each: the fastest SHORT_LIST are appended to `pool`.
+void add_every(hipblasLtHandle_t handle, const PlanKey& k, const Plan& p, const Operands& op, void* flush,
+               std::vector<hipblasLtMatmulHeuristicResult_t>& pool) {
+    const hipDataType in_t = HIP_R_16BF, out_t = k.out_f32 ? HIP_R_32F : HIP_R_16BF;
+    std::vector<hipblasLtMatmulHeuristicResult_t> all;
+    if (hipblaslt_ext::getAllAlgos(handle, hipblaslt_ext::GemmType::HIPBLASLT_GEMM, HIPBLAS_OP_T, HIPBLAS_OP_N, in_t, in_t,
+                                   out_t, out_t, HIPBLAS_COMPUTE_32F, all) != HIPBLAS_STATUS_SUCCESS)
+        return;
+    const float one = 1.f, zero = 0.f;
+    std::vector<std::pair<float, size_t>> quick;
+    for (size_t i = 0; i < all.size(); ++i) {
+        size_t need = 0;
+        if (hipblaslt_ext::matmulIsAlgoSupported(handle, p.desc, &one, p.w, p.a, &zero, p.c, p.c, all[i].algo, need) !=
+                HIPBLAS_STATUS_SUCCESS || need > op.workspace_bytes)
+            continue;
+        all[i].workspaceSize = need;
+        all[i].state = HIPBLAS_STATUS_SUCCESS;
+        const float ms = time_algo(handle, p, all[i].algo, op, flush, true);
+        if (ms > 0.f) quick.push_back({ms, i});
+    }
+    std::sort(quick.begin(), quick.end());
+    for (size_t i = 0; i < quick.size() && i < (size_t)SHORT_LIST; ++i) pool.push_back(all[quick[i].second]);
+    if (getenv("TOKENMILL_TUNE_LOG"))
+        fprintf(stderr, "[tokenmill_amd] M=%d N=%d K=%d: %zu algorithms, %zu take the product\n", k.M, k.N, k.K, all.size(),
+                quick.size());
+}
+
+// max |x - y| and max |x| over n values, as the bits of non-negative floats (which order like integers).
+template <typename T>
+__global__ void max_difference_kernel(const T* __restrict__ x, const T* __restrict__ y, size_t n, unsigned* __restrict__ out) {
+    float diff = 0.f, top = 0.f;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+        const float a = Elem<T>::load(x + i), b = Elem<T>::load(y + i);
+        const float d = fabsf(a - b);
+        diff = (d == d) ? fmaxf(diff, d) : INFINITY;       // a NaN on either side counts as a difference
+        top = fmaxf(top, fabsf(a));
+    }
+    for (int o = TM_WAVE / 2; o > 0; o >>= 1) {
+        diff = fmaxf(diff, __shfl_xor(diff, o, TM_WAVE));
+        top = fmaxf(top, __shfl_xor(top, o, TM_WAVE));
+    }
+    if (threadIdx.x % TM_WAVE == 0) {
+        atomicMax(out, __float_as_uint(diff));
+        atomicMax(out + 1, __float_as_uint(top));
+    }
+}
+
+// Does `algo` give what the heuristic's first choice `first` gives, up to the rounding of the sums?
+// An algorithm that the heuristic did not name is only kept if it does. Needs a dense result (ldc == N).
+bool same_result(hipblasLtHandle_t handle, const PlanKey& k, const Plan& p, const Operands& op,
+                 const hipblasLtMatmulAlgo_t& first, const hipblasLtMatmulAlgo_t& algo) {
+    if (k.ldc != k.N) return false;
+    const size_t n = (size_t)k.M * k.N, bytes = n * (k.out_f32 ? 4 : 2);
+    void* other = nullptr;
+    unsigned* found = nullptr;
+    if (hipMalloc(&other, bytes) != hipSuccess || hipMalloc((void**)&found, 2 * sizeof(unsigned)) != hipSuccess) {
+        (void)hipGetLastError();
+        if (other) hipFree(other);
+        return false;
+    }
+    const float one = 1.f, zero = 0.f;
+    bool ok = hipMemsetAsync(found, 0, 2 * sizeof(unsigned), op.stream) == hipSuccess;
+    ok = ok && hipblasLtMatmul(handle, p.desc, &one, op.W, p.w, op.A, p.a, &zero, other, p.c, other, p.c, &first,
+                               op.workspace, op.workspace_bytes, op.stream) == HIPBLAS_STATUS_SUCCESS;
+    ok = ok && hipblasLtMatmul(handle, p.desc, &one, op.W, p.w, op.A, p.a, &zero, op.C, p.c, op.C, p.c, &algo,
+                               op.workspace, op.workspace_bytes, op.stream) == HIPBLAS_STATUS_SUCCESS;
+    if (ok) {
+        if (k.out_f32)
+            max_difference_kernel<float><<<256, 256, 0, op.stream>>>((const float*)other, (const float*)op.C, n, found);
+        else
+            max_difference_kernel<bf16_t><<<256, 256, 0, op.stream>>>((const bf16_t*)other, (const bf16_t*)op.C, n, found);
+    }
+    unsigned host[2] = {0, 0};
+    ok = ok && hipMemcpyAsync(host, found, sizeof(host), hipMemcpyDeviceToHost, op.stream) == hipSuccess &&
+         hipStreamSynchronize(op.stream) == hipSuccess;
+    hipFree(other);
+    hipFree(found);
+    if (!ok) return false;
+    float diff, top;
+    memcpy(&diff, &host[0], 4);
+    memcpy(&top, &host[1], 4);
+    // two orders of a 32-bit sum, rounded once to the output type: a few units of the largest value's last place
+    const float allowed = top * (k.out_f32 ? 1.f / 4096 : 1.f / 32);
+    return diff <= allowed;
+}
+
 // Times up to g_tune_candidates of the library's candidates on the caller's own operands and keeps
 // the fastest. Needs the stream to run now: never called while it is being captured into a graph.
 void time_plan(hipblasLtHandle_t handle, const PlanKey& k, const Operands& op, Plan& p) {
-    hipblasLtMatmulHeuristicResult_t found[MAX_CANDIDATES];
-    int n_found = 0;
+    std::vector<hipblasLtMatmulHeuristicResult_t> pool;
     if (p.found) {
-        n_found = p.n_found < g_tune_candidates ? p.n_found : g_tune_candidates;
-        for (int i = 0; i < n_found; ++i) found[i] = p.found[i];
+        const int n = p.n_found < g_tune_candidates ? p.n_found : g_tune_candidates;
+        pool.assign(p.found, p.found + n);
         delete[] p.found;
         p.found = nullptr;
         p.n_found = 0;
     } else {                                // the plan was made before timing was switched on
-        n_found = candidates(handle, p, op.workspace_bytes, g_tune_candidates, found);
+        hipblasLtMatmulHeuristicResult_t found[MAX_CANDIDATES];
+        const int n = candidates(handle, p, op.workspace_bytes, g_tune_candidates, found);
+        pool.assign(found, found + n);
     }
-    if (n_found < 2) return;
+    const size_t named = pool.size();       // the candidates before this index are the heuristic's
     if (k.bias_dtype != TM_NONE)
         hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &op.bias, sizeof(op.bias));
-    // The heuristic's first choice stays unless another candidate beats it clearly (timings of a
-    // few runs scatter by some percent).
     // Flushed where the matrix is the larger part of what the product reads and writes (few
     // rows: the matrix comes from HBM in a real step); with many rows the activations, which the
     // kernel before has just written, are the larger part, and those are in cache in a step too.
     const size_t out_size = k.out_f32 ? 4 : 2;
     const bool cold = (size_t)k.N * k.K * 2 > (size_t)k.M * k.K * 2 + (size_t)k.M * k.N * out_size;
     void* flush = cold ? flush_buffer(k.device) : nullptr;
-    float best_ms = 0.f, first_ms = -1.f;
-    int best = -1, first = -1;
-    for (int i = 0; i < n_found; ++i) {
-        if (found[i].state != HIPBLAS_STATUS_SUCCESS || found[i].workspaceSize > op.workspace_bytes) continue;
-        const float ms = time_algo(handle, p, found[i].algo, op, flush);
+    if (g_tune_every && g_tune_after == 1) add_every(handle, k, p, op, flush, pool);
+    if (pool.size() < 2) return;
+    // The heuristic's first choice stays unless another candidate beats it clearly (timings of a
+    // few runs scatter by some percent).
+    std::vector<std::pair<float, size_t>> timed;
+    float first_ms = -1.f;
+    int first = -1;
+    for (size_t i = 0; i < pool.size(); ++i) {
+        if (pool[i].state != HIPBLAS_STATUS_SUCCESS || pool[i].workspaceSize > op.workspace_bytes) continue;
+        const float ms = time_algo(handle, p, pool[i].algo, op, flush);
         if (getenv("TOKENMILL_TUNE_LOG")) fprintf(stderr, " %.4f", ms);
         if (ms < 0.f) continue;
         if (first < 0) {
-            first = i;
+            first = (int)i;
             first_ms = ms;
         }
-        if (best < 0 || ms < best_ms) {
-            best = i;
-            best_ms = ms;
-        }
+        timed.push_back({ms, i});
     }
-    if (first >= 0 && best_ms > 0.93f * first_ms) best = first;
+    if (first < 0) return;                  // nothing could be timed: the plan stays as it is
+    std::stable_sort(timed.begin(), timed.end());
+    int best = first;
+    float best_ms = first_ms;
+    for (const auto& cand : timed) {
+        if (cand.first > 0.93f * first_ms) break;
+        // an algorithm the heuristic did not name must give the first choice's result
+        if (cand.second >= named && !same_result(handle, k, p, op, pool[first].algo, pool[cand.second].algo)) {
+            fprintf(stderr, "[tokenmill_amd] M=%d N=%d K=%d: a faster algorithm gave another result and is left out\n",
+                    k.M, k.N, k.K);
+            continue;
+        }
+        best = (int)cand.second;
+        best_ms = cand.first;
+        break;
+    }
     if (getenv("TOKENMILL_TUNE_LOG"))
-        fprintf(stderr, "[tokenmill_amd] timed M=%d N=%d K=%d %s: %d candidates, first %.4f ms, best %.4f ms, kept #%d\n",
-                k.M, k.N, k.K, cold ? "cold" : "warm", n_found, first_ms, best_ms, best);
-    if (best < 0) return;                   // nothing could be timed: the plan stays as it is
-    p.algo = found[best].algo;
-    p.workspace = found[best].workspaceSize;
+        fprintf(stderr, "[tokenmill_amd] timed M=%d N=%d K=%d %s: %zu candidates (%zu the heuristic's), first %.4f ms, best %.4f ms, kept #%d\n",
+                k.M, k.N, k.K, cold ? "cold" : "warm", pool.size(), named, first_ms, best_ms, best);
+    p.algo = pool[best].algo;
+    p.workspace = pool[best].workspaceSize;
 }
 
 }  // namespace
@@ -251,11 +363,14 @@ void time_plan(hipblasLtHandle_t handle, const PlanKey& k, const Operands& op, P
 // called the `after`-th time with the same matrix outside a graph capture, and the fastest is kept; n = 0 keeps the
 // library's first choice (the default). after = 1 times a shape at its first call: for a caller
 // that is about to capture the step into a graph and replay it.
-extern "C" int tm_gemm_library_tune(int n, int after) {
-    if (n < 0 || n > MAX_CANDIDATES || after < 1) return TM_ERR_ARG;
+// every != 0: a shape timed at its first call (after = 1) also tries every algorithm the library holds
+// for the operand types, beyond the heuristic's n (about a second a shape).
+extern "C" int tm_gemm_library_tune(int n, int after, int every) {
+    if (n < 0 || n > MAX_CANDIDATES || after < 1 || (every && n < 2)) return TM_ERR_ARG;
     std::lock_guard<std::mutex> guard(lib().lock);
     g_tune_candidates = n;
     g_tune_after = after;
+    g_tune_every = every != 0;
     return TM_OK;
 }
 

@@ -49,7 +49,7 @@ class LLMEngine:
         self.model = model
         if cfg.tune_gemm:
             from tokenmill_amd.hip import ops
-            ops.gemm_library_tune(TUNE_CANDIDATES)
+            ops.gemm_library_tune(TUNE_CANDIDATES, every=cfg.tune_gemm_every)
         self.eos_ids = set(getattr(model.config, "eos_token_ids", ()) or ())
         pages = num_cache_pages(cfg, model, self.dtype, self.device)
         self.pools = CachePools(model, pages, cfg.block_size, cfg.max_num_seqs, self.dtype, self.device)

@@ -191,31 +191,35 @@ def library_workspace(device: torch.device) -> torch.Tensor:
 
 
 TUNE_AFTER_CALLS = 3        # a shape's candidates are timed when it is called this often (most shapes of a serving run come once)
-_tune = {"candidates": 0, "after": TUNE_AFTER_CALLS}
+_tune = {"candidates": 0, "after": TUNE_AFTER_CALLS, "every": False}
 
 
-def gemm_library_tune(candidates: int, after: int = TUNE_AFTER_CALLS) -> None:
+def gemm_library_tune(candidates: int, after: int = TUNE_AFTER_CALLS, every: bool = False) -> None:
     """From now on a shape that is called the ``after``-th time with the same matrix (outside a graph capture) has up to
     ``candidates`` of the library's algorithms timed on its own operands, and the fastest is kept
-    (0: the library's first choice, untimed)."""
+    (0: the library's first choice, untimed). With ``every`` a shape that is timed at its first call
+    (``after`` = 1, see ``gemm_library_tune_at_once``) also tries every algorithm the library holds for
+    the operand types, not only those its heuristic names: about a second a shape, and an algorithm
+    found that way is kept only if it gives the first choice's result."""
     _need(0 <= candidates <= 32 and after >= 1, "gemm_library_tune: 0 to 32 candidates, after >= 1 calls")
-    _check(library().tm_gemm_library_tune(c_int(candidates), c_int(after)), "gemm_library_tune")
-    _tune["candidates"], _tune["after"] = candidates, after
+    _need(not every or candidates >= 2, "gemm_library_tune: every algorithm is tried beside at least 2 candidates")
+    _check(library().tm_gemm_library_tune(c_int(candidates), c_int(after), c_int(1 if every else 0)), "gemm_library_tune")
+    _tune["candidates"], _tune["after"], _tune["every"] = candidates, after, every
 
 
 @contextlib.contextmanager
 def gemm_library_tune_at_once():
     """Inside, a shape is timed at its first call (if timing is on at all): for the run before a
     graph capture, whose shapes are about to be replayed many times."""
-    candidates, after = _tune["candidates"], _tune["after"]
+    candidates, after, every = _tune["candidates"], _tune["after"], _tune["every"]
     if candidates < 2:
         yield
         return
-    gemm_library_tune(candidates, 1)
+    gemm_library_tune(candidates, 1, every)
     try:
         yield
     finally:
-        gemm_library_tune(candidates, after)
+        gemm_library_tune(candidates, after, every)
 
 
 def gemm_library(a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, out: torch.Tensor) -> bool:
