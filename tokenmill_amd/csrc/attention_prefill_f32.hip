@@ -12,9 +12,10 @@
 //   instead of 128; the heads of a kv head run in blocks of their own and share its keys through the
 //   second-level cache.
 //
-//   S^T = K Q^T   A = keys  [16 keys x 4 d]   B = Q^T [4 d x 16 tokens]   (D / 4 steps; the lanes of
-//                 group g = lane / 16 hold d = g D/4 .. (g + 1) D/4 - 1 of their key / token, so a
-//                 lane's operands of all steps are one contiguous run of D/4 values)
+//   S^T = K Q^T   A = keys  [16 keys x 4 d]   B = Q^T [4 d x 16 tokens]   (D / 4 steps; which d a step
+//                 multiplies is free as long as keys and queries agree: the lanes of group g = lane / 16
+//                 hold d = 16 c + 4 g .. + 3 for c = 0 .. D/16 - 1 of their key / token, so one 16-byte
+//                 load of the four groups of a key is one run of 64 bytes)
 //   O^T = V^T P^T A = V^T   [16 d x 4 keys]   B = P^T [4 keys x 16 tokens]: in step i the lanes of
 //                 group g hold key 4 g + i, which is where the S^T accumulators already have it
 //                 (register i of the same lane) and what one 16-byte load of V[d][4 g .. 4 g + 3] gives.
@@ -50,7 +51,7 @@ __global__ __launch_bounds__(64 * AF_SPLIT) void attn_prefill_f32_kernel(
 #pragma unroll
     for (int c = 0; c < DQ; c += 4) {
         f32x4_t t = {0.f, 0.f, 0.f, 0.f};
-        if (r < valid) t = *(const f32x4_t*)(q + (size_t)(row0 + r) * q_stride + (size_t)h * D + g * DQ + c);
+        if (r < valid) t = *(const f32x4_t*)(q + (size_t)(row0 + r) * q_stride + (size_t)h * D + 4 * c + 4 * g);
         qf[c] = t[0]; qf[c + 1] = t[1]; qf[c + 2] = t[2]; qf[c + 3] = t[3];
     }
     float m = -INFINITY, l = 0.f;       // running maximum of the scaled scores of this lane's column; this lane's share of the sum
@@ -59,16 +60,20 @@ __global__ __launch_bounds__(64 * AF_SPLIT) void attn_prefill_f32_kernel(
     for (int dt = 0; dt < NDT; ++dt) o[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
     const int kb_first = first_key >> 4, kb_last = last_key >> 4;
-    for (int kb = kb_first + ((wave - kb_first) & (AF_SPLIT - 1)); kb <= kb_last; kb += AF_SPLIT) {
+    int kb = kb_first + ((wave - kb_first) & (AF_SPLIT - 1));
+    // a key block's page id is asked for one block ahead (always at an entry this tile may see)
+    int pg_next = table[((kb <= kb_last ? kb : kb_last) << 4) >> page_shift];
+    for (; kb <= kb_last; kb += AF_SPLIT) {
         const int key0 = kb << 4;
-        const int pg = table[key0 >> page_shift];
+        const int pg = pg_next;
+        pg_next = table[((kb + AF_SPLIT <= kb_last ? kb + AF_SPLIT : kb) << 4) >> page_shift];
         const int in_page = key0 & (page - 1);
-        // keys: lane (r, g) holds K[key0 + r][g DQ .. g DQ + DQ - 1]
-        const float* kr = k_pool + ((((size_t)pg << page_shift) + in_page + r) * KVH + kvh) * D + g * DQ;
+        // keys: lane (r, g) holds K[key0 + r][16 c + 4 g .. + 3], c = 0 .. D/16 - 1
+        const float* kr = k_pool + ((((size_t)pg << page_shift) + in_page + r) * KVH + kvh) * D + 4 * g;
         float kf[DQ];
 #pragma unroll
         for (int c = 0; c < DQ; c += 4) {
-            const f32x4_t t = *(const f32x4_t*)(kr + c);
+            const f32x4_t t = *(const f32x4_t*)(kr + 4 * c);
             kf[c] = t[0]; kf[c + 1] = t[1]; kf[c + 2] = t[2]; kf[c + 3] = t[3];
         }
         // values: lane (r, g) holds V[d = 16 dt + r][key0 + 4 g .. + 3]
