@@ -197,6 +197,25 @@ def test_stop_rules_abort_and_rejections(model_dirs):
     tiny_pool.add_request("big", random_ids(60, 256, 73), SamplingParams(max_tokens=4))
     outs = tiny_pool.step()
     assert outs[0].finished and outs[0].error == "prompt does not fit in the KV cache"
+    # a request that has been here longer than request_timeout ends with "timeout", live or queued, and gives
+    # its pages back; a younger one goes on (reference src/infer/engine/engine.py:213-216)
+    import time
+    timed = make_engine(model_dirs["A"], "float32", request_timeout=1000.0, max_num_seqs=1)
+    old = timed.add_request("old", prompt, SamplingParams(max_tokens=50, ignore_eos=True))
+    queued = timed.add_request("old-queued", prompt, SamplingParams(max_tokens=50, ignore_eos=True),
+                               arrival_time=time.monotonic() - 2000.0)
+    young = timed.add_request("young", prompt, SamplingParams(max_tokens=3, ignore_eos=True))
+    outs = timed.step()
+    assert [(o.request_id, o.finish_reason) for o in outs if o.finished] == [("old-queued", "timeout")]
+    assert queued.why_done == "timeout" and not queued.generated
+    old.t_arrived -= 2000.0
+    outs = timed.step()
+    assert ("old", "timeout") in [(o.request_id, o.finish_reason) for o in outs]
+    assert 1 <= len(old.generated) < 50
+    while timed.has_unfinished():
+        timed.step()
+    assert young.why_done == "length" and len(young.generated) == 3
+    assert timed.cache.num_free_pages == timed.cache.num_pages
 
 
 def test_long_decoding_and_the_first_tokens_of_a_sequence(model_dirs, plains):

@@ -118,8 +118,15 @@ class LLMEngine:
 
     def step(self) -> list[RequestOutput]:
         started = time.perf_counter()
-        plan = self.scheduler.plan()
         out: list[RequestOutput] = []
+        if self.cfg.request_timeout:
+            # a request that has been here too long ends before the step is planned, queued or live,
+            # and gives its pages back (reference src/infer/engine/engine.py:169-170,213-216)
+            too_old = time.monotonic() - self.cfg.request_timeout
+            for req in [r for r in self.requests.values() if r.t_arrived < too_old]:
+                self._end(req, "timeout", time.monotonic())
+                out.append(RequestOutput(req, []))
+        plan = self.scheduler.plan()
         for req in plan.unfit:
             # an evicted request that has grown past the pool ends with what it has; a fresh one with an error
             self._end(req, "length", time.monotonic(), None if req.n_generated else DOES_NOT_FIT)
