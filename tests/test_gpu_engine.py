@@ -218,6 +218,29 @@ def test_stop_rules_abort_and_rejections(model_dirs):
     assert timed.cache.num_free_pages == timed.cache.num_pages
 
 
+def test_the_pool_is_sized_three_ways(model_dirs):
+    """Pages as given; from a byte budget; or from what the card has left after the weights and the largest
+    step, never more than `max_num_seqs` requests of `max_model_len` tokens can use (reference
+    src/infer/engine/engine.py:44-84). Fewer than two pages is an error."""
+    from tokenmill_amd import SamplingParams
+    from tokenmill_amd.cache.pool import CachePools
+    given = make_engine(model_dirs["A"], "float32", kv_cache_mb=None, num_blocks=11)
+    assert given.cache.num_pages == 11
+    per_page = CachePools.bytes_per_token(given.model, torch.float32) * 16
+    assert per_page == 2 * 2 * 2 * 16 * 4 * 16               # K and V, 2 layers, 2 kv heads of 16, float32, 16 tokens
+    budget = make_engine(model_dirs["A"], "float32", kv_cache_mb=1.0)
+    assert budget.cache.num_pages == 2**20 // per_page
+    auto = make_engine(model_dirs["A"], "bfloat16", kv_cache_mb=None, max_num_seqs=3, max_model_len=100,
+                       max_num_batched_tokens=64, hip_graphs=True)
+    assert auto.cache.num_pages == 3 * 7                      # the card has room for far more than the requests can use
+    out = auto.generate([random_ids(9, 256, 90)], SamplingParams(max_tokens=5, ignore_eos=True))
+    assert len(out[0]) == 5 and auto.cache.num_free_pages == auto.cache.num_pages
+    with pytest.raises(RuntimeError, match="fewer than two pages"):
+        make_engine(model_dirs["A"], "float32", kv_cache_mb=None, num_blocks=1)
+    with pytest.raises(RuntimeError, match="fewer than two pages"):
+        make_engine(model_dirs["A"], "float32", kv_cache_mb=per_page * 1.5 / 2**20)
+
+
 def test_long_decoding_and_the_first_tokens_of_a_sequence(model_dirs, plains):
     """A 2-token prompt decoded for 230 tokens across many pages; and 1-token prompts."""
     from tokenmill_amd import SamplingParams
