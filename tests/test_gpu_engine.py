@@ -509,3 +509,50 @@ def test_the_step_program_gives_the_bits_of_the_parts_own_code(model_dirs, name,
         if a is not None:
             assert (a == b).all(), f"step {rec['step']} of {len(traces)}"
     assert program.runner.program.runs == len(traces)
+
+
+def test_the_step_program_refuses_what_its_kernels_do_not_run(model_dirs):
+    """The library's step program checks a step by itself (it is reached without the checks of the Python
+    wrappers): a context beyond the rotary table, a block table narrower than the context, a layer group the
+    step does not bring and a workspace that is too small are refused before the kernel that would read
+    beyond them is launched."""
+    import ctypes
+    from tokenmill_amd.engine import program as prog
+    from tokenmill_amd.engine.runner import StepEntry
+    from tokenmill_amd.hip import ops
+    from tokenmill_amd.replay import ReplaySession
+    session = ReplaySession(model_dirs["A"], "bfloat16", 64)
+    runner, program = session.runner, session.runner.program
+    assert program is not None
+    cache = session.manager.allocate("r", 20)
+    step, _ = runner.prepare([StepEntry(cache, 0, random_ids(20, 256, 7), [19])])
+    want = program.run(step).clone()
+    assert torch.equal(program.run(step), want)                            # the step itself is fine, twice
+    for field, value in (("max_context_len", 65), ("num_decode", 2)):
+        saved = getattr(step, field)
+        setattr(step, field, value)
+        try:
+            with pytest.raises((ops.KernelArgumentError, RuntimeError)):
+                program.run(step)
+        finally:
+            setattr(step, field, saved)
+    narrow = step.groups[0].block_tables
+    step.groups[0].block_tables = narrow[:, :1]                            # one page of 16 for 20 positions
+    with pytest.raises((ops.KernelArgumentError, RuntimeError)):
+        program.run(step)
+    step.groups[0].block_tables = narrow
+    groups, step.groups = step.groups, []
+    with pytest.raises((ops.KernelArgumentError, RuntimeError)):
+        program.run(step)
+    step.groups = groups
+    # too small a workspace, straight at the entry point
+    lib = program._lib
+    s = prog.TmStep()
+    s.T = s.max_context_len = 20
+    s.S = s.R = 1
+    s.num_groups = 1
+    rc = lib.tm_program_run(program._handle, ctypes.byref(s), None, 16, None, 0, None, None)
+    assert rc == 1
+    assert torch.equal(program.run(step), want)                            # and nothing of this broke the program
+    session.manager.free(cache)
+

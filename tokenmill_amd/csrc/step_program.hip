@@ -165,6 +165,7 @@ struct Run {
         void* kp = a.write ? a.k_pool : nullptr;
         void* vp = a.write ? a.v_pool : nullptr;
         if (a.rot > 0 && s->max_context_len > a.max_positions) return TM_ERR_ARG;       // beyond the rotary table
+        if (!tables || W <= 0 || (long long)W * a.page < s->max_context_len) return TM_ERR_ARG;   // a table that does not reach the newest position
         const bool tables_fusable = a.rot == a.D && a.cos_t && a.sin_t;
         const bool bias_ok = !a.qkv.bias || aligned(a.qkv.bias, 16);
         const void* q = nullptr;

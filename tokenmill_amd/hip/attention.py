@@ -20,6 +20,10 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, cache: KVCacheView, st
     T, S, nd = step.num_tokens, step.num_seqs, step.num_decode
     tp = T - nd
     page = cache.k.shape[1]
+    # every kernel below walks a request's block table up to its newest position: the table must reach that far
+    if step.max_context_len > g.block_tables.shape[1] * page:
+        raise ops.KernelArgumentError(f"attention: a context of {step.max_context_len} positions and block tables of "
+                                      f"{g.block_tables.shape[1]} pages of {page}")
     done_prefill = done_decode = False
     if tp and step.prefill_tiles is not None and ops.attn_prefill_mfma_supported(qkv.dtype, H, KVH, D, page):
         ops.attn_prefill_mfma(qkv, out, cache.k, cache.v, g.block_tables, step.prefill_tiles, H, KVH, D, scale, window)
