@@ -88,6 +88,50 @@ def test_sampled_generation_chunked_and_mixed(model_dirs, plains, dtype_name):
 
 
 @pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_top_k_and_top_p_through_the_engine(model_dirs, plains, dtype_name):
+    """Temperature sampling with top-k and with top-p, prompts in portions beside decodes (the kernels alone
+    are compared with the plain sampler on equal logits in tests/test_gpu_kernels.py). In float32 every token
+    is the plain implementation's. In bfloat16 the logits differ by up to the measured bound b, which can move
+    a token across the edge of the kept set, so what is asserted is membership in the widest set that logits
+    within b of the plain ones could keep: for top-k a scaled logit within 2b/T of the k-th largest; for top-p
+    the least mass that can stand before the token (the tokens more than 2b/T above it, each probability
+    lowered by e^(-2b/T)) at most p."""
+    import math
+    from tokenmill_amd import SamplingParams
+    eng = make_engine(model_dirs["B"], dtype_name, block_size=8, enable_chunked_prefill=True, max_num_batched_tokens=20)
+    dt = DTYPES[dtype_name]
+    prompts = [random_ids(n, 384, 130 + i) for i, n in enumerate((9, 40, 24, 3, 33, 17))]
+    temp = 0.8
+    params = [SamplingParams(max_tokens=20, temperature=temp, seed=300 + i, ignore_eos=True,
+                             **({"top_k": 5} if i % 2 == 0 else {"top_p": 0.9})) for i in range(len(prompts))]
+    outs = eng.generate(prompts, params)
+    assert eng.cache.num_free_pages == eng.cache.num_pages
+    noise = plains["B"].bf16_noise() if dt == torch.bfloat16 else None
+    moved = 0
+    for i, (p, o, sp) in enumerate(zip(prompts, outs, params)):
+        assert len(o) == 20
+        logits = plains["B"].logits(p + o, dt)[len(p) - 1:-1]
+        for n, (row, tok) in enumerate(zip(logits, o)):
+            want, _ = P.sample_token(row, sp.temperature, sp.top_k, sp.top_p, 300 + i, n)
+            if dt == torch.float32:
+                assert tok == want, f"request {i} token {n}: {tok}, plain {want}"
+                continue
+            moved += tok != want
+            slack = 2 * logits_bound(row, dt, noise) / temp
+            z = row.double() / temp
+            if sp.top_k > 0:
+                kth = z.sort(descending=True).values[sp.top_k - 1]
+                assert z[tok] >= kth - slack, f"request {i} token {n}: {tok} is not among the {sp.top_k} largest, near-ties counted"
+            else:
+                probs = torch.softmax(z, dim=-1)
+                before = float(probs[z > z[tok] + slack].sum()) * math.exp(-slack)
+                assert before <= sp.top_p, f"request {i} token {n}: a mass of at least {before:.3f} stands before {tok}"
+    print(f"{dtype_name}: {moved} of 120 sampled tokens differ from the plain implementation's")
+    # a shift of b moves each probability by up to 2b/T = 3%: a few draws in a hundred fall that close to an edge
+    assert moved <= 24
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
 @pytest.mark.parametrize("chunked", [False, True])
 def test_same_tokens_under_every_cutting_and_a_starved_pool(model_dirs, plains, dtype_name, chunked):
     """16 prompts at once (reference tests/test_engine_greedy.py:25-88): small pages, small budgets,
