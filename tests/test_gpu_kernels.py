@@ -448,6 +448,44 @@ def test_sample_rows_keeps_ties_at_the_kth_value_in_vocabulary_order(ops):
     assert set(got) == {9000, 300}
 
 
+def kept_by_kernel(ops, row, t, k, p, n=8192):
+    """The tokens the sampler can return for one row: a fine grid of u over the kept distribution."""
+    us = [(i + 0.5) / n for i in range(n)]
+    return sorted(set(sample(ops, row.repeat(n, 1), [t] * n, [k] * n, [p] * n, us)))
+
+
+def test_sample_rows_cuts_the_nucleus_inside_ties_in_vocabulary_order(ops):
+    """Logits on a grid of 0.5, so that hundreds of entries share each value. The nucleus ends inside a run
+    of equal entries: they stay in vocabulary order while the mass before them is at most p (reference
+    src/infer/sampling.py:20-23 in sorted order; the plain implementation's stable sort makes that vocabulary
+    order), not all of them; with p near 0 exactly one of the entries that share the maximum stays; with top-k
+    cutting inside a run as well, the nucleus is taken over what top-k kept. -0.0 and +0.0 are one value."""
+    torch.manual_seed(5)
+    V = 4097
+    row = (torch.randn(V) * 2).round() / 2
+    for t, k, p in ((0.3, 2048, 0.5), (1.7, -1, 0.5), (0.8, -1, 0.5), (1.7, 5, 1e-6), (5.0, -1, 1e-6), (1.0, 7, 1.0),
+                    (1.0, 40, 0.95), (0.6, 12, 0.7), (2.5, 300, 0.33)):
+        want = torch.isfinite(P.filter_top_k_top_p(row / t, k, p)).nonzero().flatten().tolist()
+        got = kept_by_kernel(ops, row, t, k, p)
+        # a grid of 8,192 draws reaches every kept token whose share is above 1/8192: compare where that holds
+        probs = torch.softmax(P.filter_top_k_top_p(row / t, k, p).double(), -1)
+        reachable = [i for i in want if probs[i] > 2.0 / 8192]
+        assert set(got) <= set(want), f"t {t} k {k} p {p}: the kernel keeps {sorted(set(got) - set(want))[:8]} beyond the plain filter"
+        assert set(reachable) <= set(got), f"t {t} k {k} p {p}: the kernel drops {sorted(set(reachable) - set(got))[:8]}"
+    # the ties at the maximum with p near 0: the first of them in vocabulary order, whatever u is
+    top = (row == row.max()).nonzero().flatten().tolist()
+    assert len(top) > 1 and kept_by_kernel(ops, row, 1.7, -1, 1e-6, n=64) == [top[0]]
+    # signed zeros: a row of +0.0 and -0.0 is a row of equal entries
+    zeros = torch.zeros(100)
+    zeros[::3] = -0.0
+    assert kept_by_kernel(ops, zeros, 1.0, 7, 1.0, n=256) == list(range(7))
+    got = kept_by_kernel(ops, zeros, 1.0, -1, 0.305, n=1024)                  # mass before entry j is j / 100
+    assert got == list(range(len(got))) and len(got) in (31, 32)              # (j = 30 sits on the edge up to rounding)
+    out = torch.empty(1, dtype=torch.int32, device=DEV)
+    ops.argmax_rows(zeros[None].to(DEV), out)
+    assert out.item() == 0                                                    # the first of equal maxima, as torch.argmax
+
+
 def test_sample_rows_filters_on_the_references_vectors(ops):
     """reference tests/test_sampling.py:16-31: what top-k and top-p keep."""
     draws = [i / 64 + 1 / 128 for i in range(64)]

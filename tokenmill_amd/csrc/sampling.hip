@@ -15,7 +15,7 @@
 
 // monotonic map float -> uint32 (larger float, larger key)
 __device__ __forceinline__ uint32_t order_key(float f) {
-    uint32_t u = __float_as_uint(f);
+    uint32_t u = f == 0.f ? 0u : __float_as_uint(f);        // -0 and +0 are one value: one key
     return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 
@@ -212,8 +212,10 @@ extern "C" int tm_argmax_rows_static(const float* logits, int R, int V, int* out
 // All histogram sums are integers, so they do not depend on the order in which blocks add; the
 // float sums are taken in a fixed order that depends on V alone. A row's token depends on nothing
 // but the row, its parameters and u.
-// Ties at the k-th largest value are kept in vocabulary order until k entries are kept, as
-// torch.topk + scatter in the reference would keep k entries (reference src/infer/sampling.py:18-19).
+// Ties at the k-th largest value are kept in vocabulary order until k entries are kept, and ties at the
+// smallest value the nucleus reaches while the mass before them is at most p of the kept mass: the reference
+// keeps entries by their rank in a descending sort (reference src/infer/sampling.py:15-23), which leaves the
+// order of equal entries open; here, as in a stable sort, it is vocabulary order. -0 and +0 are equal.
 
 #define SR_NT 256
 #define SR_BINS 2048
@@ -253,10 +255,11 @@ __device__ __forceinline__ RowParams row_params(int r, int V, const float* tempe
 //   by count: the running count first reaches `limit`;
 //   by mass : the running weight would first exceed `limit`
 // (bucket 0 if that never happens), and the weight of the buckets above it added to `above`.
-// frac >= 0: limit = frac * (the histogram's total), returned through `limit` (first level by mass).
+// frac >= 0: limit = frac * (the histogram's total - drop), returned through `limit` (first level by mass;
+// drop: weight in the histogram that belongs to entries top-k does not keep after all, ties beyond its budget).
 __device__ void pick_bucket(const unsigned long long* __restrict__ hist, int bins, bool by_mass, double frac,
-                            unsigned long long& limit, unsigned long long& above, uint32_t& bucket,
-                            unsigned long long* s_scan /* SR_NT */, unsigned long long* s_res /* 2 */) {
+                            unsigned long long drop, unsigned long long& limit, unsigned long long& above,
+                            uint32_t& bucket, unsigned long long* s_scan /* SR_NT */, unsigned long long* s_res /* 2 */) {
     const int t = threadIdx.x, per = bins / SR_NT;
     unsigned long long local[SR_BINS / SR_NT];
     unsigned long long sum = 0;
@@ -275,7 +278,7 @@ __device__ void pick_bucket(const unsigned long long* __restrict__ hist, int bin
         __syncthreads();
     }
     const unsigned long long incl = s_scan[t], excl = incl - sum, total = s_scan[SR_NT - 1];
-    if (frac >= 0.0) limit = (unsigned long long)((double)total * frac);
+    if (frac >= 0.0) limit = (unsigned long long)((double)(total > drop ? total - drop : 0ull) * frac);
     auto reached = [&](unsigned long long run) { return by_mass ? run > limit : run >= limit; };
     if (t == SR_NT - 1 && !reached(above + total)) {     // never: bucket 0, everything above it counts
         s_res[0] = 0ull;
@@ -308,18 +311,41 @@ __device__ void pick_bucket(const unsigned long long* __restrict__ hist, int bin
 // row's three finished histograms; `above` = count / weight of the entries with a larger key.
 __device__ uint32_t descend(const unsigned long long* __restrict__ hist3, int levels, bool by_mass, double frac,
                             unsigned long long& limit, unsigned long long& above, uint32_t& mask,
-                            unsigned long long* s_scan, unsigned long long* s_res) {
+                            unsigned long long* s_scan, unsigned long long* s_res, unsigned long long drop = 0ull) {
     uint32_t prefix = 0;
     mask = 0;
     above = 0;
     for (int level = 0; level < levels; ++level) {
         uint32_t bucket;
-        pick_bucket(hist3 + (size_t)level * SR_BINS, level_bins(level), by_mass, level == 0 ? frac : -1.0, limit, above,
-                    bucket, s_scan, s_res);
+        pick_bucket(hist3 + (size_t)level * SR_BINS, level_bins(level), by_mass, level == 0 ? frac : -1.0, drop, limit,
+                    above, bucket, s_scan, s_res);
         prefix |= bucket << level_shift(level);
         mask |= (uint32_t)(level_bins(level) - 1) << level_shift(level);
     }
     return prefix;
+}
+
+// Where top-k ends in a row (block-wide, all threads call; the row's three count histograms are finished):
+// the key of the k-th largest entry, how many of the entries with that key stay (the first `budget` in
+// vocabulary order: the entries with a larger key are fewer than k, the ties fill up to k), and the weight
+// of the ties that do not stay (they are in the top-p histograms, which take every entry from that key up).
+struct KEdge {
+    uint32_t key;
+    int budget;
+    unsigned long long dropped;
+};
+__device__ KEdge k_edge(const unsigned long long* __restrict__ hist_k, const RowParams& rp,
+                        unsigned long long* s_scan, unsigned long long* s_res) {
+    unsigned long long limit = (unsigned long long)rp.k, above = 0;
+    uint32_t mask;
+    KEdge e;
+    e.key = descend(hist_k, 3, false, -1.0, limit, above, mask, s_scan, s_res);
+    const long long budget = (long long)rp.k - (long long)above;         // above: entries strictly larger
+    e.budget = budget > 0x7fffffffLL ? 0x7fffffff : (budget < 0 ? 0 : (int)budget);
+    const unsigned long long ties = hist_k[2 * SR_BINS + (e.key & (uint32_t)(level_bins(2) - 1))];
+    const unsigned long long cut = ties > (unsigned long long)e.budget ? ties - (unsigned long long)e.budget : 0ull;
+    e.dropped = cut * fix_weight(expf(key_value(e.key) - rp.zmax));
+    return e;
 }
 
 __global__ __launch_bounds__(TM_WAVE) void sample_rowmax_kernel(const float* __restrict__ part_v,
@@ -360,11 +386,13 @@ __global__ __launch_bounds__(SR_NT) void sample_hist_kernel(const float* __restr
     uint32_t floor_key = 0, prefix = 0, mask = 0;
     unsigned long long limit = 0, above = 0;
     if (BY_MASS) {
+        unsigned long long dropped = 0;
         if (rp.need_k) {
-            limit = (unsigned long long)rp.k;
-            floor_key = descend(hist_k, 3, false, -1.0, limit, above, mask, s_scan, s_res);
+            const KEdge e = k_edge(hist_k, rp, s_scan, s_res);
+            floor_key = e.key;
+            dropped = e.dropped;
         }
-        prefix = descend(hist_p, level, true, (double)rp.p, limit, above, mask, s_scan, s_res);
+        prefix = descend(hist_p, level, true, (double)rp.p, limit, above, mask, s_scan, s_res, dropped);
     } else {
         limit = (unsigned long long)rp.k;
         prefix = descend(hist_k, level, false, -1.0, limit, above, mask, s_scan, s_res);
@@ -390,12 +418,12 @@ __global__ __launch_bounds__(SR_NT) void sample_hist_kernel(const float* __restr
 
 // What a row keeps, as the last two stages need it.
 struct RowKeep {
-    uint32_t k_key, p_key;      // entries with key >= p_key stay (p_key >= k_key)
-    int ties_matter;            // entries equal to k_key stay only until tie_budget of them are kept
-    int tie_budget;
-};
+    uint32_t p_key;             // entries with a larger key stay, entries with a smaller one go
+    int ties_matter;            // entries equal to p_key stay only until tie_budget of them are kept, in
+    int tie_budget;             // vocabulary order (top-k: until k entries stay; top-p: while the mass before
+};                              // the entry is at most p; both: the smaller of the two)
 
-// The kept weight of one entry without the ties at k_key (0 if it is dropped or such a tie), and whether
+// The kept weight of one entry without the ties at p_key (0 if it is dropped or such a tie), and whether
 // it is such a tie.
 __device__ __forceinline__ float entry_weight(float logit, const RowParams& rp, const RowKeep& keep, bool& tie) {
     const float z = logit * rp.inv_t;
@@ -403,7 +431,7 @@ __device__ __forceinline__ float entry_weight(float logit, const RowParams& rp, 
     if (!(z == z)) return 0.f;
     const uint32_t key = order_key(z);
     if (key < keep.p_key) return 0.f;
-    if (keep.ties_matter && key == keep.k_key) {
+    if (keep.ties_matter && key == keep.p_key) {
         tie = true;
         return 0.f;
     }
@@ -450,21 +478,33 @@ __global__ __launch_bounds__(SR_NT) void sample_chunk_mass_kernel(const float* _
     if (rp.greedy) return;                               // block-uniform
     const unsigned long long* hist_k = hist_all + (size_t)r * SR_HIST_PER_ROW;
     const unsigned long long* hist_p = hist_k + 3 * SR_BINS;
-    RowKeep keep{0u, 0u, 0, 0};
-    unsigned long long limit = 0, above = 0;
-    uint32_t mask;
+    RowKeep keep{0u, 0, 0};
+    unsigned long long dropped = 0;
     if (rp.need_k) {
-        limit = (unsigned long long)rp.k;
-        keep.k_key = descend(hist_k, 3, false, -1.0, limit, above, mask, s_scan, s_res);
-        const long long budget = (long long)rp.k - (long long)above;     // above: entries strictly larger
-        keep.tie_budget = budget > 0x7fffffffLL ? 0x7fffffff : (int)budget;
+        const KEdge e = k_edge(hist_k, rp, s_scan, s_res);
+        keep.p_key = e.key;
+        keep.ties_matter = 1;
+        keep.tie_budget = e.budget;
+        dropped = e.dropped;
     }
-    keep.p_key = keep.k_key;
     if (rp.need_p) {
-        const uint32_t pk = descend(hist_p, 3, true, (double)rp.p, limit, above, mask, s_scan, s_res);
-        if (pk > keep.p_key) keep.p_key = pk;
+        // the smallest key the nucleus reaches; the entries with that key stay while the mass before them
+        // is at most p of the kept mass (reference src/infer/sampling.py:20-23: ties in sorted order, which
+        // here is vocabulary order; the first always stays): limit = p * mass, above = mass of larger keys
+        unsigned long long limit = 0, above = 0;
+        uint32_t mask;
+        const uint32_t pk = descend(hist_p, 3, true, (double)rp.p, limit, above, mask, s_scan, s_res, dropped);
+        if (!rp.need_k || pk >= keep.p_key) {
+            const unsigned long long w = fix_weight(expf(key_value(pk) - rp.zmax));
+            const unsigned long long room = limit > above ? limit - above : 0ull;
+            const unsigned long long fit = w ? room / w + 1ull : 0x7fffffffull;
+            const int by_mass = fit > 0x7fffffffull ? 0x7fffffff : (int)fit;
+            const bool same = rp.need_k && pk == keep.p_key;
+            keep.tie_budget = same && keep.tie_budget < by_mass ? keep.tie_budget : by_mass;
+            keep.p_key = pk;
+            keep.ties_matter = 1;
+        }
     }
-    keep.ties_matter = rp.need_k && keep.p_key == keep.k_key;
     if (c == 0 && threadIdx.x == 0) row_keep[r] = keep;
     const float* row = logits + (size_t)r * V;
     const int lo = c * chunk, hi = lo + chunk < V ? lo + chunk : V;
@@ -541,7 +581,7 @@ __global__ __launch_bounds__(SR_NT) void sample_pick_kernel(const float* __restr
     }
     const RowKeep keep = row_keep[r];
     const float u_row = u[r];
-    const float w_tie = keep.ties_matter ? expf(key_value(keep.k_key) - rp.zmax) : 0.f;
+    const float w_tie = keep.ties_matter ? expf(key_value(keep.p_key) - rp.zmax) : 0.f;
     // 1. the chunk that holds u * total, walking the chunks in vocabulary order
     for (int c = threadIdx.x; c < NB; c += SR_NT) {
         s_cw[c] = chunk_weight[(size_t)r * NB + c];
