@@ -1,6 +1,7 @@
 """Configurations of the architecture with the head sizes, groups and page sizes that neither the tiny
 configurations nor the published shapes have (head sizes 80, 96 and 112, groups of 1, 4 and 8, a head size
-given apart from hidden / heads, pages of 32 and 64), each through every way of cutting the work, in both
+given apart from hidden / heads, pages of 32 and 64, widths and feed-forward sizes that are no multiples of 8, 4
+or 2), each through every way of cutting the work, in both
 precisions, against the plain implementation: the kernels take every size the configuration allows, or
 another kernel does."""
 from __future__ import annotations
@@ -22,6 +23,14 @@ OTHER = {
     "d96-g1": (qwen2_config(num_hidden_layers=3, hidden_size=288, num_attention_heads=3, num_key_value_heads=3,
                             intermediate_size=360, vocab_size=1000, rope_theta=1e6, rms_norm_eps=3e-6,
                             tie_word_embeddings=False), 16, 0.02),
+    # widths, feed-forward sizes and vocabularies that are no multiples of 8, of 4 or of 2: the products that need
+    # aligned rows give way to the ones that do not
+    "odd-36": (qwen2_config(num_hidden_layers=2, hidden_size=36, num_attention_heads=2, num_key_value_heads=1, head_dim=16,
+                            intermediate_size=37, vocab_size=97, rope_theta=1e4, rms_norm_eps=1e-6,
+                            tie_word_embeddings=False), 16, 0.05),
+    "odd-250": (qwen2_config(num_hidden_layers=2, hidden_size=250, num_attention_heads=5, num_key_value_heads=1,
+                             head_dim=48, intermediate_size=333, vocab_size=501, rope_theta=1e4, rms_norm_eps=1e-6,
+                             tie_word_embeddings=True), 8, 0.05),
     "d16-g8": (qwen2_config(num_hidden_layers=3, hidden_size=256, num_attention_heads=16, num_key_value_heads=2,
                             intermediate_size=360, vocab_size=250, rope_theta=1e4, rms_norm_eps=1e-6,
                             tie_word_embeddings=True), 64, 0.05),
