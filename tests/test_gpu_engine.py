@@ -555,6 +555,28 @@ def test_the_step_program_gives_the_bits_of_the_parts_own_code(model_dirs, name,
     assert program.runner.program.runs == len(traces)
 
 
+def test_engines_with_different_options_in_one_process(model_dirs):
+    """Three engines (float32 eager; bfloat16 with graphs and chunking; bfloat16 with graphs and no packed
+    matrices) stepped in turn give the tokens each gives alone: no option travels through
+    state that the engines share (the kernel library, its plan cache and workspace, the graphs' pools)."""
+    from tokenmill_amd import SamplingParams
+    setups = [("A", "float32", dict(hip_graphs=False)),
+              ("B", "bfloat16", dict(hip_graphs=True, enable_chunked_prefill=True, max_num_batched_tokens=64)),
+              ("D", "bfloat16", dict(hip_graphs=True, pack_weights=False))]
+    prompts = {n: [random_ids(k, TINY[n][0]["vocab_size"], 50 + i) for i, k in enumerate((5, 33, 70, 17, 2, 48))] for n in "ABD"}
+    sp = SamplingParams(max_tokens=20, ignore_eos=True)
+    alone = {n: make_engine(model_dirs[n], dtype, max_num_seqs=8, **kw).generate(prompts[n], sp) for n, dtype, kw in setups}
+    engines = [(n, make_engine(model_dirs[n], dtype, max_num_seqs=8, **kw)) for n, dtype, kw in setups]
+    reqs = {n: [eng.add_request(f"{n}{i}", p, sp) for i, p in enumerate(prompts[n])] for n, eng in engines}
+    while any(eng.has_unfinished() for _, eng in engines):
+        for _, eng in engines:
+            if eng.has_unfinished():
+                eng.step()
+    for n, eng in engines:
+        assert [r.generated for r in reqs[n]] == alone[n], n
+        assert eng.cache.num_free_pages == eng.cache.num_pages
+
+
 def test_the_step_program_refuses_what_its_kernels_do_not_run(model_dirs):
     """The library's step program checks a step by itself (it is reached without the checks of the Python
     wrappers): a context beyond the rotary table, a block table narrower than the context, a layer group the
