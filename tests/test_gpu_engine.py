@@ -260,6 +260,10 @@ def test_stop_rules_abort_and_rejections(model_dirs):
         timed.step()
     assert young.why_done == "length" and len(young.generated) == 3
     assert timed.cache.num_free_pages == timed.cache.num_pages
+    # generate() runs a batch that arrives at once to its end: however long the batch takes, none of it times out
+    hurried = make_engine(model_dirs["A"], "float32", request_timeout=1e-9)
+    assert [len(o) for o in hurried.generate([prompt, prompt[:3]], SamplingParams(max_tokens=4, ignore_eos=True))] == [4, 4]
+    assert hurried.cfg.request_timeout == 1e-9
 
 
 def test_the_pool_is_sized_three_ways(model_dirs):

@@ -188,6 +188,12 @@ class LLMEngine:
         self._generate_calls += 1
         reqs = [self.add_request(f"generate-{self._generate_calls}-{i}", p, sp)
                 for i, (p, sp) in enumerate(zip(prompts, each))]
-        while self.scheduler.busy():
-            self.step()
+        # all of them arrive now and wait their turn: how long the whole batch takes is no reason to end the
+        # ones that come last, so no request times out while this loop runs
+        timeout, self.cfg.request_timeout = self.cfg.request_timeout, None
+        try:
+            while self.scheduler.busy():
+                self.step()
+        finally:
+            self.cfg.request_timeout = timeout
         return [r.generated for r in reqs]
