@@ -49,6 +49,27 @@ def test_config_refuses_what_it_cannot_run(bad, word):
         Qwen2Config.from_dict(dict(TINY_A, **bad))
 
 
+def test_a_context_or_head_size_the_model_cannot_run_is_refused_where_the_model_is_built():
+    """Not by the first step that reaches a kernel: the reference sizes its rotary table from
+    min(max_model_len, max_position_embeddings) at load (reference src/infer/model/qwen2.py:34)."""
+    from tokenmill_amd.engine.loading import check_positions
+    from tokenmill_amd.models.qwen2 import build_qwen2
+    cfg = Qwen2Config.from_dict(dict(TINY_A, max_position_embeddings=512))
+    check_positions(cfg, 512)
+    check_positions(cfg, None)
+    with pytest.raises(ConfigError, match="max_position_embeddings 512"):
+        check_positions(cfg, 513)
+    with pytest.raises(ConfigError, match="at least 1"):
+        check_positions(cfg, 0)
+    assert build_qwen2(cfg, 128).layers[0].mixer.position.max_positions == 128
+    # head sizes: even for the rotary pairs (the configuration's own rule), a multiple of 4 up to 256 for the kernels
+    for head_dim, hidden in ((6, 24), (260, 1040)):
+        bad = Qwen2Config.from_dict(dict(TINY_A, hidden_size=hidden, head_dim=head_dim))
+        with pytest.raises(ValueError, match=f"head size {head_dim}"):
+            build_qwen2(bad, 128)
+    build_qwen2(Qwen2Config.from_dict(dict(TINY_A, head_dim=20)), 128)
+
+
 def test_registry_chooses_by_config_json(tmp_path):
     assert "Qwen2ForCausalLM" in known_architectures()
     (tmp_path / "config.json").write_text(json.dumps(TINY_B))

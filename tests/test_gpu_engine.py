@@ -264,6 +264,44 @@ def test_stop_rules_abort_and_rejections(model_dirs):
     hurried = make_engine(model_dirs["A"], "float32", request_timeout=1e-9)
     assert [len(o) for o in hurried.generate([prompt, prompt[:3]], SamplingParams(max_tokens=4, ignore_eos=True))] == [4, 4]
     assert hurried.cfg.request_timeout == 1e-9
+    # ... while a request that came through add_request keeps its timeout during that loop
+    own = hurried.add_request("own", prompt, SamplingParams(max_tokens=4, ignore_eos=True))
+    assert [len(o) for o in hurried.generate([prompt], SamplingParams(max_tokens=4, ignore_eos=True))] == [4]
+    assert own.why_done == "timeout" and not hurried.has_unfinished()
+    # one prompt of a batch refused: nothing of the batch stays queued
+    with pytest.raises(RequestRejected):
+        hurried.generate([prompt, prompt[:4], []], SamplingParams(max_tokens=4))
+    assert not hurried.has_unfinished() and not hurried.requests
+
+
+def test_a_step_that_fails_ends_its_requests_and_gives_their_pages_back(model_dirs, monkeypatch):
+    """A step that raises (here: forced from the host) leaves no request live with pages that nobody will ever
+    free: the step's requests end with reason "error", the queue is untouched and served afterwards."""
+    from tokenmill_amd import SamplingParams
+    from tokenmill_amd.engine.runner import StepError
+    eng = make_engine(model_dirs["A"], "float32", max_num_seqs=2)
+    sp = SamplingParams(max_tokens=6, ignore_eos=True)
+    prompts = [random_ids(n, 256, 60 + n) for n in (9, 20, 5)]
+    want = make_engine(model_dirs["A"], "float32").generate([prompts[2]], sp)[0]
+    reqs = [eng.add_request(f"r{i}", p, sp) for i, p in enumerate(prompts)]
+    eng.step()
+    eng.step()
+    assert eng.num_running == 2 and eng.num_waiting == 1
+    real_step = eng.runner.step
+
+    def failing(entries):
+        raise StepError("forced from the test")
+
+    monkeypatch.setattr(eng.runner, "step", failing)
+    with pytest.raises(StepError):
+        eng.step()
+    monkeypatch.setattr(eng.runner, "step", real_step)
+    assert [r.why_done for r in reqs] == ["error", "error", None] and "forced from the test" in reqs[0].error
+    assert eng.num_running == 0 and eng.num_waiting == 1 and eng.cache.num_free_pages == eng.cache.num_pages
+    eng.cache.check_invariants()
+    while eng.has_unfinished():
+        eng.step()
+    assert reqs[2].generated == want and eng.cache.num_free_pages == eng.cache.num_pages
 
 
 def test_the_pool_is_sized_three_ways(model_dirs):

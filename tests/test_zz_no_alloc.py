@@ -41,13 +41,20 @@ def test_static_argmax_matches_the_allocating_one_on_two_calls_in_a_row():
     lib = _lib()
     torch.manual_seed(11)
     dev = torch.device("cuda:0")
-    big = torch.randn(24, 151936, device=dev)
-    big[3, 151935] = 40.0                                  # a maximum in the last, shorter chunk
-    big[5, 4096] = 41.0                                    # ... and at a chunk's first entry
-    big[7, 100] = big[7, 90000] = 42.0                     # a tie: the lower index wins
+    V = 151936
+    big = torch.randn(24, V, device=dev)
+    nb = lib.tm_argmax_work_chunks(c_int(V))
+    chunk = -(-V // nb)                                    # entries of a chunk: 3,999 here, no power of two
+    assert nb > 1 and chunk * (nb - 1) < V <= chunk * nb and chunk % 64
+    big[3, V - 1] = 40.0                                   # a maximum in the last, shorter chunk
+    big[5, 5 * chunk] = 41.0                               # ... at a chunk's first entry
+    big[6, 9 * chunk - 1] = 41.0                           # ... at a chunk's last entry
+    big[7, 100] = big[7, 90000] = 42.0                     # a tie across chunks: the lower index wins
+    big[8, 3 * chunk - 1] = big[8, 3 * chunk] = 43.0       # a tie across a chunk's edge
     got, want = _both(lib, big)
     assert torch.equal(got, want) and torch.equal(got.long(), big.argmax(dim=1).cpu())
-    assert got[3] == 151935 and got[5] == 4096 and got[7] == 100
+    assert got[3] == V - 1 and got[5] == 5 * chunk and got[6] == 9 * chunk - 1 and got[7] == 100
+    assert got[8] == 3 * chunk - 1
     # a second call with a smaller input: fewer rows and fewer chunks; what the first call left in the
     # array beyond them must not be read
     small = torch.randn(5, 20000, device=dev)

@@ -1,0 +1,30 @@
+// The rules by which a step's kernels are chosen, in one place: the row counts up to which each family of
+// matrix-product kernels is preferred, and when the decode attention splits a context over blocks. The step
+// program (step_program.hip) is the only code that applies them; the Python side reads the numbers through
+// tm_rule() where it sizes a buffer or checks an argument, and never decides by them.
+#pragma once
+
+// --- matrix products (bfloat16) ----------------------------------------------------------------------
+// up to this many rows the kernels that stream the matrix once win: the products over packed matrices with
+// the layer's epilogue (bias, rotary + cache write, SiLU*up, residual add), and the ones that start at the norm
+constexpr int TM_SKINNY_ROWS = 16;
+// up to this many rows q|k|v and gate|up keep the normed input in LDS (where it fits) and carry their epilogues
+constexpr int TM_PANEL_ROWS = 48;
+// up to this many rows the products stream the packed matrix once for several row tiles, with their epilogues
+constexpr int TM_STREAM_ROWS = 64;
+// most rows one launch of the skinny product takes at all
+constexpr int TM_SKINNY_MAX_ROWS = 64;
+// most rows the 32-bit matrix-vector product takes
+constexpr int TM_GEMV_F32_ROWS = 16;
+
+// --- decode attention ---------------------------------------------------------------------------------
+constexpr int TM_DECODE_CHUNK = 256;        // keys per block of the split decode attention
+constexpr int TM_DECODE_SPLIT_PAIRS = 192;  // below this many (request, kv head) pairs the split kernels run
+
+inline int tm_decode_chunks(int max_context) { return (max_context + TM_DECODE_CHUNK - 1) / TM_DECODE_CHUNK; }
+
+// Does a decode step of `requests` single tokens split its contexts over blocks (and need the scratch
+// memory for their partial results)?
+inline bool tm_decode_splits(int requests, int kv_heads, int max_context) {
+    return requests * kv_heads < TM_DECODE_SPLIT_PAIRS && tm_decode_chunks(max_context) > 1;
+}

@@ -29,16 +29,17 @@ namespace {
 
 struct PlanKey {
     int M, N, K, lda, ldw, ldc, bias_dtype, out_f32, device;
+    int tuned;      // 1: the plan of callers that ask for timed algorithms; the others never see what timing chose
     bool operator==(const PlanKey& o) const {
         return M == o.M && N == o.N && K == o.K && lda == o.lda && ldw == o.ldw && ldc == o.ldc &&
-               bias_dtype == o.bias_dtype && out_f32 == o.out_f32 && device == o.device;
+               bias_dtype == o.bias_dtype && out_f32 == o.out_f32 && device == o.device && tuned == o.tuned;
     }
 };
 
 struct PlanKeyHash {
     size_t operator()(const PlanKey& k) const {
         size_t h = 1469598103934665603ull;
-        for (int v : {k.M, k.N, k.K, k.lda, k.ldw, k.ldc, k.bias_dtype, k.out_f32, k.device})
+        for (int v : {k.M, k.N, k.K, k.lda, k.ldw, k.ldc, k.bias_dtype, k.out_f32, k.device, k.tuned})
             h = (h ^ (size_t)(uint32_t)v) * 1099511628211ull;
         return h;
     }
@@ -71,18 +72,17 @@ Library& lib() {
     return *l;
 }
 
-// How many of the heuristic's candidates are timed for a shape before the fastest is kept (0 or 1:
-// keep the heuristic's first choice untimed), and at which call of a shape that happens. Steps of a
-// serving run come in hundreds of different numbers of rows, most of them once: timing costs tens
-// of milliseconds per shape, so only a shape that comes back is timed (or one whose caller says
-// that it will be replayed, by asking for the first call).
-// With TOKENMILL_TUNE_LOG set in the environment every timing is printed to stderr.
-int g_tune_candidates = 0;
-int g_tune_after = 3;
+// Timing is the caller's choice, call by call (TmTune, api.h): how many of the heuristic's candidates are
+// timed for a shape before the fastest is kept (0 or 1: keep the heuristic's first choice untimed), and
+// at which call of a shape that happens. Steps of a serving run come in hundreds of different numbers
+// of rows, most of them once: timing costs tens of milliseconds per shape, so only a shape that comes
+// back is timed (or one whose caller says that it will be replayed, by asking for the first call).
 // Beyond the heuristic's candidates, a shape that is timed at its first call (its caller is about to
-// replay it from a graph) also has every algorithm the library holds for the operand types tried:
+// replay it from a graph) can also have every algorithm the library holds for the operand types tried:
 // one quick run each, the fastest few timed like the heuristic's candidates. About a second a shape.
-bool g_tune_every = false;
+// Plans made for callers that time live beside the plans of callers that do not (PlanKey::tuned): an
+// engine that keeps the library's first choice gets the same algorithm whoever else runs in the process.
+// With TOKENMILL_TUNE_LOG set in the environment every timing is printed to stderr.
 constexpr int SHORT_LIST = 12;
 
 struct Operands {
@@ -168,7 +168,7 @@ int candidates(hipblasLtHandle_t handle, const Plan& p, size_t workspace_bytes, 
 }
 
 // Descriptors, layouts and the heuristic's first valid choice: no run, no wait.
-bool make_plan(hipblasLtHandle_t handle, const PlanKey& k, size_t workspace_bytes, Plan& p) {
+bool make_plan(hipblasLtHandle_t handle, const PlanKey& k, size_t workspace_bytes, const TmTune& tune, Plan& p) {
     const hipDataType in_t = HIP_R_16BF, out_t = k.out_f32 ? HIP_R_32F : HIP_R_16BF;
     if (hipblasLtMatmulDescCreate(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F) != HIPBLAS_STATUS_SUCCESS) return false;
     const hipblasOperation_t tr = HIPBLAS_OP_T, no = HIPBLAS_OP_N;
@@ -190,14 +190,14 @@ bool make_plan(hipblasLtHandle_t handle, const PlanKey& k, size_t workspace_byte
     constexpr int UNTIMED_CANDIDATES = 8;
     hipblasLtMatmulHeuristicResult_t found[MAX_CANDIDATES];
     const int n_found = candidates(handle, p, workspace_bytes,
-                                   g_tune_candidates > UNTIMED_CANDIDATES ? g_tune_candidates : UNTIMED_CANDIDATES, found);
+                                   tune.candidates > UNTIMED_CANDIDATES ? tune.candidates : UNTIMED_CANDIDATES, found);
     for (int i = 0; i < n_found && !p.ok; ++i)
         if (found[i].state == HIPBLAS_STATUS_SUCCESS && found[i].workspaceSize <= workspace_bytes) {
             p.algo = found[i].algo;
             p.workspace = found[i].workspaceSize;
             p.ok = true;
         }
-    if (p.ok && n_found > 1 && g_tune_candidates > 1) {
+    if (p.ok && n_found > 1 && tune.candidates > 1) {
         p.found = new hipblasLtMatmulHeuristicResult_t[n_found];
         for (int i = 0; i < n_found; ++i) p.found[i] = found[i];
         p.n_found = n_found;
@@ -292,19 +292,19 @@ bool same_result(hipblasLtHandle_t handle, const PlanKey& k, const Plan& p, cons
     return diff <= allowed;
 }
 
-// Times up to g_tune_candidates of the library's candidates on the caller's own operands and keeps
+// Times up to tune.candidates of the library's candidates on the caller's own operands and keeps
 // the fastest. Needs the stream to run now: never called while it is being captured into a graph.
-void time_plan(hipblasLtHandle_t handle, const PlanKey& k, const Operands& op, Plan& p) {
+void time_plan(hipblasLtHandle_t handle, const PlanKey& k, const Operands& op, const TmTune& tune, Plan& p) {
     std::vector<hipblasLtMatmulHeuristicResult_t> pool;
     if (p.found) {
-        const int n = p.n_found < g_tune_candidates ? p.n_found : g_tune_candidates;
+        const int n = p.n_found < tune.candidates ? p.n_found : tune.candidates;
         pool.assign(p.found, p.found + n);
         delete[] p.found;
         p.found = nullptr;
         p.n_found = 0;
     } else {                                // the plan was made before timing was switched on
         hipblasLtMatmulHeuristicResult_t found[MAX_CANDIDATES];
-        const int n = candidates(handle, p, op.workspace_bytes, g_tune_candidates, found);
+        const int n = candidates(handle, p, op.workspace_bytes, tune.candidates, found);
         pool.assign(found, found + n);
     }
     const size_t named = pool.size();       // the candidates before this index are the heuristic's
@@ -316,7 +316,7 @@ void time_plan(hipblasLtHandle_t handle, const PlanKey& k, const Operands& op, P
     const size_t out_size = k.out_f32 ? 4 : 2;
     const bool cold = (size_t)k.N * k.K * 2 > (size_t)k.M * k.K * 2 + (size_t)k.M * k.N * out_size;
     void* flush = cold ? flush_buffer(k.device) : nullptr;
-    if (g_tune_every && g_tune_after == 1) add_every(handle, k, p, op, flush, pool);
+    if (tune.every && tune.after <= 1) add_every(handle, k, p, op, flush, pool);
     if (pool.size() < 2) return;
     // The heuristic's first choice stays unless another candidate beats it clearly (timings of a
     // few runs scatter by some percent).
@@ -359,34 +359,28 @@ void time_plan(hipblasLtHandle_t handle, const PlanKey& k, const Operands& op, P
 
 }  // namespace
 
-// From now on a shape's candidates (up to n of them) are timed on its own operands when it is
-// called the `after`-th time with the same matrix outside a graph capture, and the fastest is kept; n = 0 keeps the
-// library's first choice (the default). after = 1 times a shape at its first call: for a caller
-// that is about to capture the step into a graph and replay it.
-// every != 0: a shape timed at its first call (after = 1) also tries every algorithm the library holds
-// for the operand types, beyond the heuristic's n (about a second a shape).
-extern "C" int tm_gemm_library_tune(int n, int after, int every) {
-    if (n < 0 || n > MAX_CANDIDATES || after < 1 || (every && n < 2)) return TM_ERR_ARG;
-    std::lock_guard<std::mutex> guard(lib().lock);
-    g_tune_candidates = n;
-    g_tune_after = after;
-    g_tune_every = every != 0;
-    return TM_OK;
-}
-
 // bias_dtype: TM_NONE (no bias), TM_BF16 or TM_F32. out_f32: C is float32 (else bfloat16).
 // workspace: device memory the library may use, the same for every call on a stream.
+// tune: null or candidates < 2 keeps the library's first choice. Else up to `candidates` of the library's
+// candidates are timed on this call's own operands when the shape is called the `after`-th time with the
+// matrix of its first call outside a graph capture, and the fastest is kept (after = 1: at its first call,
+// for a caller that is about to capture the step into a graph and replay it); every != 0: a shape timed at
+// its first call also tries every algorithm the library holds for the operand types (about a second a shape).
 // Returns TM_ERR_ARG for arguments it does not take, TM_ERR_UNSUPPORTED when the library has no
 // algorithm for the product (the caller then uses another path), TM_ERR_LAUNCH when the call fails.
 extern "C" int tm_gemm_library(const void* A, int lda, const void* W, int ldw, const void* bias, int bias_dtype,
                                void* C, int ldc, int out_f32, int M, int N, int K, void* workspace,
-                               size_t workspace_bytes, hipStream_t stream) {
+                               size_t workspace_bytes, const TmTune* tune_or_null, hipStream_t stream) {
     if (M <= 0 || N <= 0 || K <= 0 || lda < K || ldw < K || ldc < N || !A || !W || !C ||
         (bias_dtype != TM_NONE && bias_dtype != TM_BF16 && bias_dtype != TM_F32) || ((bias_dtype != TM_NONE) != (bias != nullptr)))
         return TM_ERR_ARG;
+    TmTune tune{0, 3, 0};
+    if (tune_or_null) tune = *tune_or_null;
+    if (tune.candidates < 0 || tune.candidates > MAX_CANDIDATES || (tune.every && tune.candidates < 2)) return TM_ERR_ARG;
+    if (tune.after < 1) tune.after = 1;
     int device = 0;
     if (hipGetDevice(&device) != hipSuccess) return TM_ERR_LAUNCH;
-    const PlanKey key{M, N, K, lda, ldw, ldc, bias_dtype, out_f32 ? 1 : 0, device};
+    const PlanKey key{M, N, K, lda, ldw, ldc, bias_dtype, out_f32 ? 1 : 0, device, tune.candidates > 1 ? 1 : 0};
     Library& l = lib();
     hipblasLtHandle_t handle;
     Plan plan;
@@ -402,20 +396,20 @@ extern "C" int tm_gemm_library(const void* A, int lda, const void* W, int ldw, c
         auto it = l.plans.find(key);
         if (it == l.plans.end()) {
             Plan made;
-            make_plan(handle, key, workspace_bytes, made);           // a failed plan is kept too: asked once
+            make_plan(handle, key, workspace_bytes, tune, made);           // a failed plan is kept too: asked once
             it = l.plans.emplace(key, made).first;
         }
         Plan& kept = it->second;
-        if (kept.ok && !kept.timed && g_tune_candidates > 1) {
+        if (kept.ok && !kept.timed && tune.candidates > 1) {
             hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
             hipStreamIsCapturing(stream, &capturing);
             // calls with the matrix of the first call are counted: every layer of a step brings the
             // shape once with its own matrix, and a step is not a shape that came back
             if (!kept.first_w) kept.first_w = W;
-            if (capturing == hipStreamCaptureStatusNone && W == kept.first_w && ++kept.calls >= g_tune_after) {
+            if (capturing == hipStreamCaptureStatusNone && W == kept.first_w && ++kept.calls >= tune.after) {
                 kept.timed = true;
                 const Operands op{A, W, bias, C, workspace, workspace_bytes, stream};
-                time_plan(handle, key, op, kept);
+                time_plan(handle, key, op, tune, kept);
             }
         }
         plan = kept;

@@ -45,6 +45,8 @@ class LLMEngine:
             model = load_model(cfg.model, self.dtype, self.device, max_positions=cfg.max_model_len,
                                pack_weights=cfg.pack_weights)
         else:
+            from tokenmill_amd.engine.loading import check_positions
+            check_positions(model.config, cfg.max_model_len)
             self.device, self.dtype = model.device, model.dtype
         self.model = model
         if cfg.tune_gemm:
@@ -72,8 +74,7 @@ class LLMEngine:
 
     # --- requests ---------------------------------------------------------------------------------
 
-    def add_request(self, request_id: str, prompt_ids: list[int], params: SamplingParams,
-                    arrival_time: float | None = None) -> Request:
+    def _check_request(self, request_id: str, prompt_ids: list[int]) -> None:
         vocab, limit = self.runner.vocab, self.cfg.max_model_len
         if request_id in self.requests:
             raise RequestRejected(f"request id {request_id!r} is in use")
@@ -84,9 +85,15 @@ class LLMEngine:
                                   "no room for a generated token")
         if min(prompt_ids) < 0 or max(prompt_ids) >= vocab:
             raise RequestRejected(f"the prompt holds a token outside the vocabulary of {vocab}")
+
+    def add_request(self, request_id: str, prompt_ids: list[int], params: SamplingParams,
+                    arrival_time: float | None = None, expires: bool = True) -> Request:
+        """``expires``: False exempts this request from ``request_timeout`` (``generate`` submits a whole batch
+        at once, and how long the batch takes is no reason to end the prompts that wait their turn)."""
+        self._check_request(request_id, prompt_ids)
         seed = params.seed if params.seed is not None else self._seeds.getrandbits(62)
         req = Request(request_id, prompt_ids, params, seed,
-                      time.monotonic() if arrival_time is None else arrival_time)
+                      time.monotonic() if arrival_time is None else arrival_time, expires=expires)
         self.requests[request_id] = req
         self.scheduler.enqueue(req)
         return req
@@ -123,7 +130,7 @@ class LLMEngine:
             # a request that has been here too long ends before the step is planned, queued or live,
             # and gives its pages back (reference src/infer/engine/engine.py:169-170,213-216)
             too_old = time.monotonic() - self.cfg.request_timeout
-            for req in [r for r in self.requests.values() if r.t_arrived < too_old]:
+            for req in [r for r in self.requests.values() if r.expires and r.t_arrived < too_old]:
                 self._end(req, "timeout", time.monotonic())
                 out.append(RequestOutput(req, []))
         plan = self.scheduler.plan()
@@ -133,10 +140,20 @@ class LLMEngine:
             out.append(RequestOutput(req, []))
         if not plan:
             return out
-        logits = self.runner.step(plan.entries)
         winners = [plan.owners[i] for i in plan.yields]
-        tokens = self.sampler.sample(logits, [r.params for r in winners], [r.stream_seed for r in winners],
-                                     [r.n_generated for r in winners]) if winners else []
+        try:
+            logits = self.runner.step(plan.entries)
+            tokens = self.sampler.sample(logits, [r.params for r in winners], [r.stream_seed for r in winners],
+                                         [r.n_generated for r in winners]) if winners else []
+        except Exception as e:
+            # The step did not run to its end, so what the cache holds for its requests is unknown: they end
+            # here with the error and give their pages back (the reference's loop ends every request in
+            # flight with the error and goes on serving, reference src/infer/engine/engine.py:342-349).
+            # Requests that were not part of the step are untouched.
+            now = time.monotonic()
+            for req in dict.fromkeys(plan.owners):
+                self._end(req, "error", now, f"{type(e).__name__}: {e}")
+            raise
         now = time.monotonic()
         release = self.cache.release_behind_window
         for req, entry in zip(plan.owners, plan.entries):
@@ -186,14 +203,17 @@ class LLMEngine:
         if len(each) != len(prompts):
             raise ValueError(f"{len(prompts)} prompts but {len(each)} sampling parameters")
         self._generate_calls += 1
-        reqs = [self.add_request(f"generate-{self._generate_calls}-{i}", p, sp)
-                for i, (p, sp) in enumerate(zip(prompts, each))]
-        # all of them arrive now and wait their turn: how long the whole batch takes is no reason to end the
-        # ones that come last, so no request times out while this loop runs
-        timeout, self.cfg.request_timeout = self.cfg.request_timeout, None
+        names = [f"generate-{self._generate_calls}-{i}" for i in range(len(prompts))]
+        for name, p in zip(names, prompts):          # all or none: a prompt that is refused leaves nothing queued
+            self._check_request(name, p)
+        # all of them arrive now and wait their turn, so none of them expires; requests that came through
+        # add_request keep their timeout
+        reqs = [self.add_request(name, p, sp, expires=False) for name, p, sp in zip(names, prompts, each)]
         try:
-            while self.scheduler.busy():
+            while any(not r.done for r in reqs):
                 self.step()
-        finally:
-            self.cfg.request_timeout = timeout
+        except BaseException:
+            for r in reqs:                           # what the failed step did not end gives its pages back too
+                self.abort_request(r.id)
+            raise
         return [r.generated for r in reqs]

@@ -25,11 +25,24 @@ def resolve_device(name: str) -> torch.device:
     return torch.device("cuda:0" if name == "auto" else name)
 
 
+def check_positions(model_config, max_positions: int | None) -> None:
+    """Refuses, before anything is loaded, a context the model's position tables do not reach: the reference
+    sizes its rotary table ``min(max_model_len, max_position_embeddings)`` (reference
+    src/infer/model/qwen2.py:34, src/infer/engine/engine.py:94), so a longer context would index beyond it."""
+    from tokenmill_amd.config.model_config import ConfigError
+    most = getattr(model_config, "max_position_embeddings", None)
+    if max_positions is not None and max_positions < 1:
+        raise ConfigError(f"max_model_len must be at least 1, got {max_positions}")
+    if max_positions is not None and most is not None and max_positions > most:
+        raise ConfigError(f"max_model_len {max_positions} exceeds the model's max_position_embeddings {most}")
+
+
 def load_model(model_dir: str | Path, dtype: torch.dtype, device: torch.device, max_positions: int | None = None,
                pack_weights: bool = True):
     """The model that config.json names, with its weights on ``device``. ``pack_weights``: keep a second
     copy of each layer matrix in the order the decode-step kernels read it."""
     arch, cfg = load_config(model_dir)
+    check_positions(cfg, max_positions)
     model = arch.build_model(cfg, max_positions)
     tensors = read_checkpoint(model_dir, model.tensor_specs(), dtype, device, model.ignorable)
     model.load(tensors, dtype, device, pack_weights=pack_weights)
@@ -45,7 +58,9 @@ def load_random_model(config: dict, seed: int, dtype: torch.dtype, device: torch
     from tokenmill_amd.weights.loader import storage_dtype
 
     arch = get_architecture(architecture_name(config))
-    model = arch.build_model(arch.config_from_dict(config, None), max_positions)
+    cfg = arch.config_from_dict(config, None)
+    check_positions(cfg, max_positions)
+    model = arch.build_model(cfg, max_positions)
     g = torch.Generator(device=device).manual_seed(seed)
     tensors = {}
     for name, spec in sorted(model.tensor_specs().items()):

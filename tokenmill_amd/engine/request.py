@@ -25,10 +25,10 @@ class Phase(enum.Enum):
 
 class Request:
     __slots__ = ("id", "tokens", "n_prompt", "params", "stream_seed", "cached", "cache", "phase", "evictions",
-                 "why_done", "error", "t_arrived", "t_first_token", "t_done")
+                 "why_done", "error", "t_arrived", "t_first_token", "t_done", "expires")
 
     def __init__(self, request_id: str, prompt: list[int], params: SamplingParams, stream_seed: int = 0,
-                 t_arrived: float = 0.0):
+                 t_arrived: float = 0.0, expires: bool = True):
         self.id = request_id
         self.tokens: list[int] = list(prompt)
         self.n_prompt = len(self.tokens)
@@ -38,9 +38,10 @@ class Request:
         self.cache: RequestCache | None = None
         self.phase = Phase.QUEUED
         self.evictions = 0
-        self.why_done: str | None = None          # stop | length | abort
+        self.why_done: str | None = None          # stop | length | abort | timeout | error
         self.error: str | None = None
         self.t_arrived = t_arrived
+        self.expires = expires                    # False: the engine's request_timeout does not end it
         self.t_first_token: float | None = None
         self.t_done: float | None = None
 

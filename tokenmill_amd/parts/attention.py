@@ -18,6 +18,9 @@ from tokenmill_amd.parts.base import (KVCacheSpec, KVCacheView, Mixer, NormedInp
 from tokenmill_amd.parts.linear import Linear
 
 
+MAX_HEAD_DIM = 256      # the widest head the generic attention kernel takes (the matrix-unit kernels: 32, 64, 96, 128)
+
+
 class GQAttention(Mixer):
     def __init__(self, hidden: int, num_heads: int, num_kv_heads: int, head_dim: int, scale: float,
                  position: PositionEncoding, qkv_bias: bool = True, o_bias: bool = False,
@@ -25,6 +28,9 @@ class GQAttention(Mixer):
                  names: tuple[str, str, str, str] = ("q_proj", "k_proj", "v_proj", "o_proj")):
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads do not divide into {num_kv_heads} kv heads")
+        if head_dim % 4 or not 0 < head_dim <= MAX_HEAD_DIM:
+            # said where the model is built, not by the first step that reaches a kernel
+            raise ValueError(f"head size {head_dim}: the attention kernels take multiples of 4 up to {MAX_HEAD_DIM}")
         self.hidden, self.num_heads, self.num_kv_heads, self.head_dim = hidden, num_heads, num_kv_heads, head_dim
         self.scale = float(scale)
         self.window = window

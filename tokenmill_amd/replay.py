@@ -30,6 +30,7 @@ class ReplaySession:
                  page_size: int = PAGE_SIZE):
         from tokenmill_amd.cache import CacheManager
         from tokenmill_amd.cache.pool import CachePools
+        from tokenmill_amd.config.registry import load_config
         from tokenmill_amd.engine.loading import load_model, resolve_device, resolve_dtype
         from tokenmill_amd.engine.runner import ModelRunner
         from tokenmill_amd.hip.library import library
@@ -40,14 +41,18 @@ class ReplaySession:
         if page_size < 1:
             raise ValueError("--block-size must be at least 1")
         max_tokens = -(-max_tokens // ROUND_TO) * ROUND_TO
-        self.model = load_model(model_dir, dtype, device, max_positions=max_tokens)
+        # --max-tokens bounds what all live requests hold together; one request can be no longer than that,
+        # nor than the model's own position tables reach
+        _, model_config = load_config(model_dir)
+        max_positions = min(max_tokens, getattr(model_config, "max_position_embeddings", max_tokens))
+        self.model = load_model(model_dir, dtype, device, max_positions=max_positions)
         self.page_size = page_size
         # every request's tokens count rounded up to ROUND_TO; a page that does not divide that may leave
         # one page per request part empty beyond it
         self.num_pages = -(-max_tokens // page_size) + (0 if ROUND_TO % page_size == 0 else max_requests)
         self.pools = CachePools(self.model, self.num_pages, page_size, max_requests, dtype, device)
         self.manager = CacheManager(self.pools.windows, self.num_pages, page_size, max_requests)
-        self.runner = ModelRunner(self.model, self.pools, max_positions=max_tokens)
+        self.runner = ModelRunner(self.model, self.pools, max_positions=max_positions)
         self.lengths: dict[str, int] = {}
 
     def run_step(self, rec: dict):
