@@ -126,7 +126,8 @@ def main() -> int:
         return sum(o.bytes for o in ops), sum(o.flops for o in ops)
 
     def eagerly(eng, fn):
-        """``fn`` with the engine's graph replay switched off: the parts' code runs, so their labels do."""
+        """``fn`` with the engine's graph replay switched off: the same step program runs launch by launch, and
+        the library calls the labels' hook around each operation's launches (a replayed graph calls nothing)."""
         runner = eng.runner
         saved = runner.graphs, runner.step_graphs
         runner.graphs = runner.step_graphs = None
@@ -172,7 +173,8 @@ def main() -> int:
 
     def trace_decode(eng, step_s) -> dict:
         """Kernel time of the replayed step (for "GPU idle"), and per operation the GPU time of the same
-        step launched kernel by kernel, with the share of its floor it reaches."""
+        step program launched kernel by kernel (what the graph is a recording of), with the share of its
+        floor it reaches."""
         with profiling.collect() as replayed:
             for _ in range(PROFILED_STEPS):
                 eng.step()

@@ -159,16 +159,15 @@ def test_same_tokens_under_every_cutting_and_a_starved_pool(model_dirs, plains, 
         assert outs == base
 
 
-def test_steps_of_17_to_48_tokens_take_the_panel_products(model_dirs, plains, monkeypatch):
+def test_steps_of_17_to_48_tokens_take_the_panel_products(model_dirs, plains):
     """24 requests decoding together, and prompt steps of 20 to 40 tokens: the q|k|v and gate|up products
-    that keep the normed input in LDS run (counted, in the library's step program and in the parts' own
-    code), and every token is the plain implementation's."""
+    that keep the normed input in LDS run (counted by the step program), and every token is the plain
+    implementation's."""
     from tokenmill_amd import SamplingParams
-    from tokenmill_amd.hip import ops
     prompts = [random_ids(1 + (7 * i) % 19, 384, 300 + i) for i in range(24)]
     layers = 3
     eng = make_engine(model_dirs["B"], "bfloat16", max_num_batched_tokens=40)
-    assert eng.runner.program is not None
+    assert not eng.runner.program.foreign_parts               # every part of this model is an operation of the library's
     outs = eng.generate(prompts, SamplingParams(max_tokens=10, ignore_eos=True))
     for p, o in zip(prompts, outs):
         assert len(o) == 10
@@ -176,14 +175,6 @@ def test_steps_of_17_to_48_tokens_take_the_panel_products(model_dirs, plains, mo
     took = eng.runner.program.counters()
     assert took["qkv_panel"] >= 9 * layers and took["gate_up_panel"] == took["qkv_panel"]      # the decode steps of 24 tokens at least
     assert eng.cache.num_free_pages == eng.cache.num_pages
-    calls = {"qkv": 0, "gate_up": 0}
-    real_qkv, real_gu = ops.panel_qkv_rope, ops.panel_gate_up_silu
-    monkeypatch.setattr(ops, "panel_qkv_rope", lambda *a, **k: (calls.__setitem__("qkv", calls["qkv"] + 1), real_qkv(*a, **k))[1])
-    monkeypatch.setattr(ops, "panel_gate_up_silu", lambda *a, **k: (calls.__setitem__("gate_up", calls["gate_up"] + 1), real_gu(*a, **k))[1])
-    by_parts = make_engine(model_dirs["B"], "bfloat16", max_num_batched_tokens=40, step_program=False)
-    assert by_parts.runner.program is None
-    assert by_parts.generate(prompts, SamplingParams(max_tokens=10, ignore_eos=True)) == outs
-    assert calls["qkv"] == took["qkv_panel"] and calls["gate_up"] == took["gate_up_panel"]
 
 
 def test_without_the_packed_copy_of_the_matrices(model_dirs, plains):
@@ -576,47 +567,71 @@ def test_generation_with_peaked_attention_at_a_published_head_size(model_dirs, p
 
 
 @pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name,page", [("A", 16), ("B", 8), ("B", 16), ("C", 16), ("D", 16)])
-def test_the_step_program_gives_the_bits_of_the_parts_own_code(model_dirs, name, page, dtype_name):
-    """A step run by the library's step program (one call) and the same step launched kernel by kernel from
-    the parts' Python code choose the same kernels in the same order: equal logits, bit for bit, over whole
-    prompts, portions, single tokens and mixed steps with reused pages."""
+@pytest.mark.parametrize("name,page", [("A", 16), ("B", 8), ("D", 16)])
+def test_operations_run_one_by_one_give_the_bits_of_one_run(model_dirs, name, page, dtype_name):
+    """The step program runs consecutive operations of the library's in one call; a model with a part of
+    another kind runs them in several calls with that part's own code in between. What crosses between two
+    calls (the residual stream and the result still to be added to it) is all the state there is: the same
+    steps run with one call per operation, and with every block's operations called through the parts' own
+    `forward` (each part's one-operation program), give equal logits, bit for bit, over whole prompts,
+    portions, single tokens and mixed steps with reused pages."""
+    from tokenmill_amd.hip.program import _Foreign, _Native
     from tokenmill_amd.replay import ReplaySession
     from test_gpu_replay import make_requests, mixed, portions, prefill_then_decode, run_trace
     reqs = make_requests(name, [37, 64, 21, 90, 48, 33, 75, 18], 14)
     traces = prefill_then_decode(reqs) + portions(reqs) + mixed(reqs, seed=15)
-    program = ReplaySession(model_dirs[name], dtype_name, 4 * 128, page_size=page)
-    parts = ReplaySession(model_dirs[name], dtype_name, 4 * 128, page_size=page)
-    assert program.runner.program is not None
-    parts.runner.program = None
+    whole = ReplaySession(model_dirs[name], dtype_name, 4 * 128, page_size=page)
+    single = ReplaySession(model_dirs[name], dtype_name, 4 * 128, page_size=page)
+    blocks = ReplaySession(model_dirs[name], dtype_name, 4 * 128, page_size=page)
+    program = single.runner.program
+    assert [type(s) for s in program.steps] == [_Native] and program.steps[0].count == 2 + 2 * len(single.model.run)
+    program.steps = [_Native(i, 1) for i in range(program.steps[0].count)]
+    # the third: embedding and head stay operations, every block in between runs through Block.forward
+    model, prog3 = blocks.model, blocks.runner.program
+    n_ops = prog3.steps[0].count
+    steps3 = [_Native(0, 1)]
+    for j, call in enumerate(model.run):
+        def run_block(flow, step, block=model.layers[call.layer], cache=blocks.pools.views[j]):
+            flow.delta = block.forward(flow.resid, flow.delta, step, cache, model.dtype)
+        steps3.append(_Foreign(model.layers[call.layer], run_block))
+    steps3.append(_Native(n_ops - 1, 1))
+    prog3.steps = steps3
     for rec in traces:
-        a, b = program.run_step(rec), parts.run_step(rec)
-        assert (a is None) == (b is None)
+        a, b, c = whole.run_step(rec), single.run_step(rec), blocks.run_step(rec)
+        assert (a is None) == (b is None) == (c is None)
         if a is not None:
-            assert (a == b).all(), f"step {rec['step']} of {len(traces)}"
-    assert program.runner.program.runs == len(traces)
+            assert (a == b).all(), f"step {rec['step']} of {len(traces)}, one call per operation"
+            assert (a == c).all(), f"step {rec['step']} of {len(traces)}, blocks through their own forward"
+    assert whole.runner.program.runs == len(traces)
 
 
-def test_engines_with_different_options_in_one_process(model_dirs):
-    """Three engines (float32 eager; bfloat16 with graphs and chunking; bfloat16 with graphs and no packed
-    matrices) stepped in turn give the tokens each gives alone: no option travels through
-    state that the engines share (the kernel library, its plan cache and workspace, the graphs' pools)."""
+def test_engines_with_different_options_in_one_process(model_dirs, plains):
+    """Four engines (float32 eager; bfloat16 with graphs and chunking; bfloat16 with graphs and no packed
+    matrices; bfloat16 with graphs and the library's algorithms chosen by timing) stepped in turn give the
+    tokens each gives alone: no option travels through state that the engines share (the kernel library, its
+    plan cache and workspace, the graphs' pools). In particular an engine without timing keeps its bits beside
+    one that times the same shapes of the same model (configuration D twice: the timed plans are kept apart)."""
     from tokenmill_amd import SamplingParams
     setups = [("A", "float32", dict(hip_graphs=False)),
               ("B", "bfloat16", dict(hip_graphs=True, enable_chunked_prefill=True, max_num_batched_tokens=64)),
-              ("D", "bfloat16", dict(hip_graphs=True, pack_weights=False))]
+              ("D", "bfloat16", dict(hip_graphs=True, pack_weights=False)),
+              ("D", "bfloat16", dict(hip_graphs=True, pack_weights=False, tune_gemm=True))]
     prompts = {n: [random_ids(k, TINY[n][0]["vocab_size"], 50 + i) for i, k in enumerate((5, 33, 70, 17, 2, 48))] for n in "ABD"}
     sp = SamplingParams(max_tokens=20, ignore_eos=True)
-    alone = {n: make_engine(model_dirs[n], dtype, max_num_seqs=8, **kw).generate(prompts[n], sp) for n, dtype, kw in setups}
+    alone = [make_engine(model_dirs[n], dtype, max_num_seqs=8, **kw).generate(prompts[n], sp) for n, dtype, kw in setups[:3]]
     engines = [(n, make_engine(model_dirs[n], dtype, max_num_seqs=8, **kw)) for n, dtype, kw in setups]
-    reqs = {n: [eng.add_request(f"{n}{i}", p, sp) for i, p in enumerate(prompts[n])] for n, eng in engines}
+    reqs = [[eng.add_request(f"{n}{i}", p, sp) for i, p in enumerate(prompts[n])] for n, eng in engines]
     while any(eng.has_unfinished() for _, eng in engines):
         for _, eng in engines:
             if eng.has_unfinished():
                 eng.step()
-    for n, eng in engines:
-        assert [r.generated for r in reqs[n]] == alone[n], n
+    for k, (n, eng) in enumerate(engines):
+        if k < 3:
+            assert [r.generated for r in reqs[k]] == alone[k], n
         assert eng.cache.num_free_pages == eng.cache.num_pages
+    assert engines[3][1].runner.program.tune and not engines[2][1].runner.program.tune
+    for p, r in zip(prompts["D"], reqs[3]):                     # the timed engine's tokens are right by themselves
+        verify(plains["D"], p, r.generated, torch.bfloat16)
 
 
 def test_the_step_program_refuses_what_its_kernels_do_not_run(model_dirs):
@@ -625,13 +640,12 @@ def test_the_step_program_refuses_what_its_kernels_do_not_run(model_dirs):
     step does not bring and a workspace that is too small are refused before the kernel that would read
     beyond them is launched."""
     import ctypes
-    from tokenmill_amd.engine import program as prog
+    from tokenmill_amd.hip import abi
     from tokenmill_amd.engine.runner import StepEntry
     from tokenmill_amd.hip import ops
     from tokenmill_amd.replay import ReplaySession
     session = ReplaySession(model_dirs["A"], "bfloat16", 64)
     runner, program = session.runner, session.runner.program
-    assert program is not None
     cache = session.manager.allocate("r", 20)
     step, _ = runner.prepare([StepEntry(cache, 0, random_ids(20, 256, 7), [19])])
     want = program.run(step).clone()
@@ -655,12 +669,20 @@ def test_the_step_program_refuses_what_its_kernels_do_not_run(model_dirs):
     step.groups = groups
     # too small a workspace, straight at the entry point
     lib = program._lib
-    s = prog.TmStep()
+    s = abi.TmStep()
     s.T = s.max_context_len = 20
     s.S = s.R = 1
     s.num_groups = 1
-    rc = lib.tm_program_run(program._handle, ctypes.byref(s), None, 16, None, 0, None, None)
+    io = abi.TmStream()
+    small = torch.empty(256, dtype=torch.uint8, device="cuda:0")
+    resid = torch.empty((20, 64), device="cuda:0")
+    io.resid, io.accumulate = resid.data_ptr(), 1
+    rc = lib.tm_program_run(program._handle, 0, len(program.parts), ctypes.byref(s), ctypes.byref(io), small.data_ptr(), 256,
+                            None, 0, None, 0, None)
     assert rc == 1
+    for first, count in ((-1, 1), (0, 0), (1, len(program.parts))):      # operations the program does not have
+        assert lib.tm_program_run(program._handle, first, count, ctypes.byref(s), ctypes.byref(io), small.data_ptr(), 256,
+                                  None, 0, None, 0, None) == 1
     assert torch.equal(program.run(step), want)                            # and nothing of this broke the program
     session.manager.free(cache)
 

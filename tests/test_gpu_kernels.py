@@ -605,15 +605,16 @@ def test_gemm_library(ops, M, N, K, tune, after):
     a strided input, the same bits on the second call (the kept plan); untimed, with the candidates
     timed at the first call, and timed when the shape comes the third time (every call before and
     after gives the product). A shape the library refuses comes back as False and `linear` takes
-    another kernel."""
-    from tokenmill_amd.hip import gemm
+    another kernel. Plans of timed callers live apart from the plans of the others: a call without
+    timing gives the same bits before and after a timed caller has had its algorithm chosen."""
     torch.manual_seed(12)
     dt = torch.bfloat16
     a, w, b = q(torch.randn(M, K), dt), q(torch.randn(N, K) * 0.1, dt), q(torch.randn(N), dt)
     want = a @ w.t()
     da, dw, db = a.to(dt).to(DEV), w.to(dt).to(DEV), b.to(dt).to(DEV)
-    ops.gemm_library_tune(tune, after)
-    try:
+    untimed = torch.full((M, N), 7.0, dtype=dt, device=DEV)
+    taken = ops.gemm_library(da, dw, db, untimed)
+    with ops.tuning(tune, after):
         out = torch.full((M, N), 7.0, dtype=dt, device=DEV)
         if ops.gemm_library(da, dw, db, out):
             torch.testing.assert_close(out.float().cpu(), q(want + b, dt), **tol(dt))
@@ -631,12 +632,13 @@ def test_gemm_library(ops, M, N, K, tune, after):
         out_s = torch.full((M, N), 7.0, dtype=dt, device=DEV)
         if ops.gemm_library(wide[:, :K], dw, None, out_s):
             torch.testing.assert_close(out_s.float().cpu(), q(want, dt), **tol(dt))
-        # whatever the library takes, the policy above it gives the product
+        # whatever the library takes, the rule above it gives the product
         out_l = torch.full((M, N), 7.0, dtype=dt, device=DEV)
-        gemm.linear(da, dw, db, out_l)
+        ops.linear(ops.linear_desc(dw, None, db), da, out_l)
         torch.testing.assert_close(out_l.float().cpu(), q(want + b, dt), **tol(dt))
-    finally:
-        ops.gemm_library_tune(0)
+    if taken:                                               # ... and nothing of the timing reached the untimed plan
+        again = torch.empty_like(untimed)
+        assert ops.gemm_library(da, dw, db, again) and torch.equal(again, untimed)
 
 
 @pytest.mark.parametrize("M,N,K", [(64, 896, 4864), (333, 1152, 896)])
@@ -650,8 +652,7 @@ def test_gemm_library_tries_every_algorithm(ops, M, N, K):
     a, w, b = q(torch.randn(M, K), dt), q(torch.randn(N, K) * 0.1, dt), q(torch.randn(N), dt)
     want = a @ w.t()
     da, dw, db = a.to(dt).to(DEV), w.to(dt).to(DEV), b.to(dt).to(DEV)
-    ops.gemm_library_tune(8, 1, every=True)
-    try:
+    with ops.tuning(8, 1, every=True):
         for bias, add in ((db, b), (None, 0.0)):
             out = torch.full((M, N), 7.0, dtype=dt, device=DEV)
             assert ops.gemm_library(da, dw, bias, out)
@@ -661,10 +662,9 @@ def test_gemm_library_tries_every_algorithm(ops, M, N, K):
         out32 = torch.full((M, N), 7.0, dtype=torch.float32, device=DEV)
         assert ops.gemm_library(da, dw, None, out32)
         torch.testing.assert_close(out32.cpu(), want, rtol=1e-4, atol=1e-4 * K ** 0.5)
-    finally:
-        ops.gemm_library_tune(0)
     with pytest.raises(ops.KernelArgumentError):
-        ops.gemm_library_tune(0, 1, every=True)
+        with ops.tuning(0, 1, every=True):
+            pass
 
 
 def test_gemm_library_takes_a_candidate_whose_workspace_fits(ops):
@@ -677,7 +677,6 @@ def test_gemm_library_takes_a_candidate_whose_workspace_fits(ops):
     da = torch.randn(M, K, device=DEV).to(dt)
     dw = (torch.randn(N, K, device=DEV) * 0.1).to(dt)
     out = torch.full((M, N), 7.0, dtype=dt, device=DEV)
-    ops.gemm_library_tune(0)
     assert ops.gemm_library(da, dw, None, out)
     rows = torch.arange(0, M, 257)
     want = da[rows].float().cpu() @ dw.float().cpu().t()
@@ -704,8 +703,7 @@ def test_gemm_skinny_with_silu_epilogue(ops, M, I, K):
 def test_paged_attention_decode_mfma(ops, monkeypatch, H, KVH, D, page, window, one_block):
     """one_block: the kernel for many requests (one block walks a request's whole context), which the
     dispatcher would only take from 192 (request, kv head) pairs on."""
-    if one_block:
-        monkeypatch.setattr(ops, "DECODE_SPLIT_PAIRS", 0)
+    split = False if one_block else None
     dt = torch.bfloat16
     lens = [1, 2, 16, 17, 255, 256, 257, 700, 64, 1000]
     q_lens = [1] * len(lens)
@@ -722,7 +720,7 @@ def test_paged_attention_decode_mfma(ops, monkeypatch, H, KVH, D, page, window, 
     out = torch.full((S, H * D), 3.0, dtype=dt, device=DEV)
     ctx = torch.tensor(lens, dtype=torch.int32, device=DEV)
     ops.attn_decode_mfma(wide, out, case["kp"].to(DEV), v_layout(case["vp"]).to(DEV), case["tables"].to(DEV), ctx,
-                         H, KVH, D, scale, window, max(lens))
+                         H, KVH, D, scale, window, max(lens), split=split)
     want = paged_truth(case, lens, q_lens, scale, dt, window or None).reshape(S, H * D)
     torch.testing.assert_close(out.float().cpu(), want, **tol(dt))
     if not window:                               # the spiked far key (position 2 of 700) carries its request's output
@@ -735,7 +733,7 @@ def test_paged_attention_decode_mfma(ops, monkeypatch, H, KVH, D, page, window, 
     out2 = torch.empty(2, H * D, dtype=dt, device=DEV)
     ops.attn_decode_mfma(wide[sub].contiguous(), out2, case["kp"].to(DEV), v_layout(case["vp"]).to(DEV),
                          case["tables"][sub].contiguous().to(DEV), ctx[sub].contiguous(), H, KVH, D, scale, window,
-                         max(lens))
+                         max(lens), split=split)
     assert torch.equal(out2, out[sub])
     # block tables wider than any context (the shape a captured graph has), scratch memory full of NaN
     # beyond what the step writes: up to 64 chunks the merge reads ahead of the context length, beyond
@@ -744,7 +742,7 @@ def test_paged_attention_decode_mfma(ops, monkeypatch, H, KVH, D, page, window, 
         width = -(-max_context // page)
         tables = torch.zeros(S, width, dtype=torch.int32)
         tables[:, :case["tables"].shape[1]] = case["tables"]
-        chunks = -(-max_context // ops.DECODE_CHUNK)
+        chunks = -(-max_context // ops.rule("decode_chunk"))
         ws = (torch.full((S, H, chunks, D), float("nan"), device=DEV), torch.full((S, H, chunks, 2), float("nan"), device=DEV))
         out3 = torch.full((S, H * D), 3.0, dtype=dt, device=DEV)
         ops.attn_decode_mfma(wide, out3, case["kp"].to(DEV), v_layout(case["vp"]).to(DEV), tables.to(DEV), ctx,

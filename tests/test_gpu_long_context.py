@@ -84,8 +84,7 @@ def check_far_key(out, case, request, far, row, H, KVH, D, atol):
 @pytest.mark.parametrize("window", [0, 1000])
 def test_decode_attention_at_long_contexts(monkeypatch, H, KVH, D, page, one_block, window):
     from tokenmill_amd.hip import ops
-    if one_block:                                 # the kernel that walks a whole context in one block
-        monkeypatch.setattr(ops, "DECODE_SPLIT_PAIRS", 0)
+    split = False if one_block else None          # False: the kernel that walks a whole context in one block
     dt = torch.bfloat16
     lens = [2048, 4096, 16384, 2047, 4097, 1, 300]
     q_lens = [1] * len(lens)
@@ -98,7 +97,7 @@ def test_decode_attention_at_long_contexts(monkeypatch, H, KVH, D, page, one_blo
     out = torch.full((S, H * D), 3.0, dtype=dt, device=DEV)
     ctx = torch.tensor(lens, dtype=torch.int32, device=DEV)
     kp, vp, tables = case["kp"].to(DEV), v_layout(case["vp"]).to(DEV), case["tables"].to(DEV)
-    ops.attn_decode_mfma(wide, out, kp, vp, tables, ctx, H, KVH, D, scale, window, max(lens))
+    ops.attn_decode_mfma(wide, out, kp, vp, tables, ctx, H, KVH, D, scale, window, max(lens), split=split)
     want = truth_rows(case, lens, q_lens, scale, dt, window or None).reshape(S, H * D)
     got = out.float().cpu()
     torch.testing.assert_close(got, want, **bf16_tol())
@@ -108,7 +107,7 @@ def test_decode_attention_at_long_contexts(monkeypatch, H, KVH, D, page, one_blo
     sub = [2, 0, 4]
     out2 = torch.empty(len(sub), H * D, dtype=dt, device=DEV)
     ops.attn_decode_mfma(wide[sub].contiguous(), out2, kp, vp, tables[sub].contiguous(), ctx[sub].contiguous(),
-                         H, KVH, D, scale, window, max(lens))
+                         H, KVH, D, scale, window, max(lens), split=split)
     assert torch.equal(out2, out[sub])
 
 

@@ -367,7 +367,9 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path, dtype_na
     for mode in ("eager", "graphs", "refused"):
         eng = LLMEngine(EngineConfig(model=str(d), dtype=dtype_name, block_size=8, num_blocks=64, max_model_len=64,
                                      max_num_seqs=4, max_num_batched_tokens=64, watermark=0.0, hip_graphs=mode != "eager"))
-        assert eng.runner.program is None                     # a mixer the library's step program does not know
+        # the mixer with state runs through its own code, between the library's operations: two hops a step, not the model
+        assert [type(p).__name__ for p in eng.runner.program.foreign_parts] == ["DecayedSumMixer"] * 2
+        assert len(eng.runner.program.parts) == 2 + 2 + 4      # embedding, head, two attentions, four feed-forwards
         if mode == "refused":
             for layer in eng.model.layers[::2]:
                 layer.mixer.capturable = False

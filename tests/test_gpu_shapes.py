@@ -116,13 +116,6 @@ def test_every_cut_at_the_layer_sizes_of_the_published_shapes(layer_models, monk
         assert took["qkv_panel"] > 0 or name != "0.5B"        # widths of 3,584 and 5,120 do not fit a block's LDS
     else:
         assert took["qkv_plain"] > 0 and took["qkv_from_norm"] == 0
-    # the same mixed trace launched from the parts' own code: the same bits
-    by_parts = ReplaySession(d, dtype_name, 4 * 128)
-    by_parts.runner.program = None
-    again = run_trace(by_parts, steps)
-    for key, row in run_trace(session, steps).items():
-        assert torch.equal(row, again[key]), f"{name} layers, {dtype_name}: {key}"
-    del by_parts
     del session
     torch.cuda.empty_cache()
 

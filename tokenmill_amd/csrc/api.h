@@ -75,9 +75,15 @@ int tm_attn_prefill_mfma(const void* q, int q_stride, void* out, int out_stride,
 int tm_gemv_f32(const float* A, int lda, const float* W, const float* bias, float* C, int ldc, int M, int N, int K,
                 hipStream_t stream);
 
-int tm_gemm_library_tune(int n, int after, int every);
+// How a caller wants the library's algorithm for a product chosen (tm_gemm_library): see gemm_library.hip.
+struct TmTune {
+    int candidates;     // 0 or 1: the library's first choice, untimed; n: up to n candidates are timed, the fastest kept
+    int after;          // the call of a shape (with the matrix of its first call) at which that happens; 1: at once
+    int every;          // a shape timed at its first call also tries every algorithm the library holds for the types
+};
 int tm_gemm_library(const void* A, int lda, const void* W, int ldw, const void* bias, int bias_dtype, void* C, int ldc,
-                    int out_f32, int M, int N, int K, void* workspace, size_t workspace_bytes, hipStream_t stream);
+                    int out_f32, int M, int N, int K, void* workspace, size_t workspace_bytes, const TmTune* tune,
+                    hipStream_t stream);
 
 int tm_attn_prefill_f32(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
                         const void* v_pool, const int* block_tables, int table_width, const int* tiles, int n_tiles,

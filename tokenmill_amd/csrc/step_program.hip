@@ -1,33 +1,34 @@
-// A model step as one call: the launch sequence of a decoder made of pre-norm attention and pre-norm
-// feed-forward operations, run from a list that the parts filled once at load.
+// A model step as a few calls: the launch sequence of a decoder, run from a list of operations that the
+// model's parts described once at load (embedding, pre-norm attention, pre-norm feed-forward, final norm and
+// output head).
 //
-// The host side of a step that is not a graph replay used to be a few hundred calls from Python into
-// this library (one per kernel, each with its checks and its output allocation). Here the parts
-// describe themselves once (matrices, norms, head sizes, cache pools), and a step is: fill the step's
-// metadata, hand over one workspace, call tm_program_run. Which kernel runs for which row count and
-// type is decided here exactly as the Python parts decide it (tokenmill_amd/parts, hip/gemm.py,
-// hip/attention.py), so both ways launch the same kernels in the same order and give the same bits.
+// This file is the one place where a step's kernels are chosen: which product kernel for which row count
+// and type, which attention kernel for which head size, page and batch (the thresholds stand in choose.h).
+// The Python parts hold no such rule: the engine runs consecutive operations with one tm_program_run call,
+// a part that the library has no operation for runs between two such calls through its own code, and a part
+// that is called by itself (from such code, or a test) runs its own one-operation program through the same
+// entry. tm_linear_run is the product rule alone, for a matrix used outside an operation.
 // (The reference's step is its model's forward pass in torch: src/infer/engine/model_runner.py:76-97,
 // src/infer/model/qwen2.py:43-52.)
 #include "common.h"
 #include "api.h"
+#include "choose.h"
 #include "step_program.h"
 
 #include <stdint.h>
+#include <string.h>
 #include <vector>
 
 namespace {
 
-constexpr int SKINNY_ROWS = 16;         // most rows the skinny and norm-fused kernels are preferred for
-constexpr int PANEL_ROWS = 48;          // most rows the products that keep the normed input in LDS are preferred for
-constexpr int SKINNY_MAX_ROWS = 64;
-constexpr int DECODE_CHUNK = 256;       // keys per block of the split decode attention
-constexpr int DECODE_SPLIT_PAIRS = 192; // below this many (request, kv head) pairs the split kernels run
+enum { OP_EMBED = 0, OP_ATTENTION, OP_FEED_FORWARD, OP_HEAD };
 
 struct Op {
-    int kind;                           // 0 attention, 1 feed-forward
+    int kind;
+    TmEmbedOp embed;
     TmAttentionOp att;
     TmFfnOp ffn;
+    TmFinalOp head;
 };
 
 inline size_t align_up(size_t n) { return (n + 255) & ~(size_t)255; }
@@ -40,12 +41,15 @@ inline int elem_size(int dtype) { return dtype == TM_BF16 ? 2 : 4; }
 struct TmProgram {
     int dtype = TM_BF16;
     int hidden = 0;
-    TmEmbedOp embed{};
-    TmFinalOp final_op{};
-    bool has_embed = false, has_final = false;
     std::vector<Op> ops;
     // the widest of each kind of activation over all operations
-    int max_qkv = 0, max_q = 0, max_gu = 0, max_act = 0, max_heads_d = 0;
+    int max_qkv = 0, max_gu = 0, max_act = 0, max_heads = 0, max_heads_d = 0;
+    // a matrix the checkpoint stores in 32-bit stays 32-bit in a bfloat16 model: its product runs in 32-bit on a
+    // widened copy of the activations; the widest input and output of such products
+    int max_wide_in = 0, max_wide_out = 0;
+    TmHook hook = nullptr;
+    void* hook_user = nullptr;
+    TmTune tune{0, 3, 0};
     // how often each way of computing q|k|v and the activation was taken (for tests and curiosity)
     mutable long long taken[TM_PROGRAM_COUNTERS] = {};
 };
@@ -60,11 +64,12 @@ bool fused_lds_fits(int M, int K) {
 }
 
 bool fused_decode_ok(const float* resid, const TmLinear& L, int M) {
-    return L.packed && M > 0 && M <= SKINNY_ROWS && L.K % 8 == 0 && fused_lds_fits(M, L.K) && aligned(resid, 16);
+    return resid && L.packed && M > 0 && M <= TM_SKINNY_ROWS && L.K % 8 == 0 && fused_lds_fits(M, L.K) && aligned(resid, 16);
 }
 
 bool packed_ok(const TmLinear& L, const void* x, int ldx, int M, int dtype) {
-    return L.packed && M > 0 && M <= SKINNY_ROWS && dtype == TM_BF16 && L.K % 8 == 0 && ldx % 8 == 0 && aligned(x, 16);
+    return L.packed && M > 0 && M <= TM_SKINNY_ROWS && dtype == TM_BF16 && L.dtype == TM_BF16 && L.K % 8 == 0 && ldx % 8 == 0 &&
+           aligned(x, 16);
 }
 
 bool skinny_ok(const TmLinear& L, const void* x, int ldx, int dtype) {
@@ -72,77 +77,124 @@ bool skinny_ok(const TmLinear& L, const void* x, int ldx, int dtype) {
 }
 
 bool panel_ok(const TmLinear& L, const void* x, int ldx, int M, int dtype) {
-    return L.packed && M > SKINNY_ROWS && M <= PANEL_ROWS && dtype == TM_BF16 && ldx % 8 == 0 && aligned(x, 16) &&
+    return L.packed && M > TM_SKINNY_ROWS && M <= TM_PANEL_ROWS && dtype == TM_BF16 && ldx % 8 == 0 && aligned(x, 16) &&
            tm_gemm_panel_fits(M, L.K);
 }
 
-struct Run {
-    const TmProgram* p;
-    const TmStep* s;
+// The product rule. x_dtype: type of x (the model's activations); the matrix has its own (L.dtype).
+struct Products {
     hipStream_t stream;
     void* lib_ws;
     size_t lib_ws_bytes;
-    int dtype;
-    // workspace
-    float* resid;
-    void *x, *qkv, *attn, *gu, *act, *delta_buf, *hnorm;
-    float *part_o, *part_ml;
-    const void* delta = nullptr;        // product output still to be added to the residual stream
+    TmTune tune;
+    float* wide_in = nullptr;           // room for a product's input and output in 32-bit (see TmProgram::max_wide_in)
+    float* wide_out = nullptr;
 
-    int linear(const TmLinear& L, const void* x_, int ldx, int M, void* out, int ldc, int out_dtype) {
+    int library(const TmLinear& L, const void* x, int ldx, int M, void* out, int ldc, int out_dtype) const {
+        return tm_gemm_library(x, ldx, L.w, L.K, L.bias, L.bias_dtype, out, ldc, out_dtype == TM_F32, M, L.N, L.K, lib_ws,
+                               lib_ws_bytes, &tune, stream);
+    }
+
+    int linear(const TmLinear& L, int dtype, const void* x, int ldx, int M, void* out, int ldc, int out_dtype) const {
         if (M == 0) return TM_OK;
-        if (L.packed && L.packed_parts == 1 && packed_ok(L, x_, ldx, M, dtype) && !L.library_first)
-            return tm_gemm_skinny_packed(x_, ldx, L.packed, L.packed_rows, L.bias, L.bias_dtype, out, ldc, M, L.N, L.K,
+        if (L.dtype != dtype) {
+            // a 32-bit matrix under bfloat16 activations: the activations are widened, the product runs in 32-bit,
+            // and the result is rounded to the type asked for
+            if (L.dtype != TM_F32 || dtype != TM_BF16 || !wide_in || !wide_out || ldx != L.K) return TM_ERR_ARG;
+            int rc = tm_convert(x, TM_BF16, wide_in, TM_F32, (long long)M * L.K, stream);
+            if (rc) return rc;
+            if (out_dtype == TM_F32) return linear(L, TM_F32, wide_in, L.K, M, out, ldc, TM_F32);
+            if (ldc != L.N) return TM_ERR_ARG;
+            if ((rc = linear(L, TM_F32, wide_in, L.K, M, wide_out, L.N, TM_F32))) return rc;
+            return tm_convert(wide_out, TM_F32, out, TM_BF16, (long long)M * L.N, stream);
+        }
+        if (L.packed_parts == 1 && packed_ok(L, x, ldx, M, dtype) && !L.library_first)
+            return tm_gemm_skinny_packed(x, ldx, L.packed, L.packed_rows, L.bias, L.bias_dtype, out, ldc, M, L.N, L.K,
                                          out_dtype, 0, nullptr, 0, stream);
         if (dtype != TM_BF16) {
-            const bool gemv = L.dtype == TM_F32 && out_dtype == TM_F32 && (L.bias_dtype == TM_NONE || L.bias_dtype == TM_F32) &&
-                              M <= 16 && L.K % 4 == 0 && ldx % 4 == 0 && aligned(x_, 16) && aligned(L.w, 16);
-            if (gemv) return tm_gemv_f32((const float*)x_, ldx, (const float*)L.w, (const float*)L.bias, (float*)out, ldc, M, L.N, L.K, stream);
-            if (L.dtype == TM_F32 && out_dtype == TM_F32 && (L.bias_dtype == TM_NONE || L.bias_dtype == TM_F32) &&
-                tm_gemm_f32_mfma_fits(x_, ldx, L.w, L.bias, out, ldc, M, L.N, L.K))
-                return tm_gemm_f32_mfma((const float*)x_, ldx, (const float*)L.w, (const float*)L.bias, (float*)out, ldc, M, L.N, L.K, stream);
-            return tm_gemm_nt_tiled(x_, ldx, L.w, L.bias, L.bias_dtype, out, ldc, M, L.N, L.K, dtype, out_dtype, stream);
+            const bool plain32 = out_dtype == TM_F32 && (L.bias_dtype == TM_NONE || L.bias_dtype == TM_F32);
+            if (plain32 && M <= TM_GEMV_F32_ROWS && L.K % 4 == 0 && ldx % 4 == 0 && aligned(x, 16) && aligned(L.w, 16))
+                return tm_gemv_f32((const float*)x, ldx, (const float*)L.w, (const float*)L.bias, (float*)out, ldc, M, L.N, L.K, stream);
+            if (plain32 && tm_gemm_f32_mfma_fits(x, ldx, L.w, L.bias, out, ldc, M, L.N, L.K))
+                return tm_gemm_f32_mfma((const float*)x, ldx, (const float*)L.w, (const float*)L.bias, (float*)out, ldc, M, L.N, L.K, stream);
+            return tm_gemm_nt_tiled(x, ldx, L.w, L.bias, L.bias_dtype, out, ldc, M, L.N, L.K, dtype, out_dtype, stream);
         }
-        const bool skinny = skinny_ok(L, x_, ldx, dtype);
-        const bool library = L.dtype == TM_BF16;
-        if (library && L.library_first) {
-            const int rc = tm_gemm_library(x_, ldx, L.w, L.K, L.bias, L.bias_dtype, out, ldc, out_dtype == TM_F32, M, L.N, L.K,
-                                           lib_ws, lib_ws_bytes, stream);
+        const bool skinny = skinny_ok(L, x, ldx, dtype);
+        if (L.library_first) {
+            const int rc = library(L, x, ldx, M, out, ldc, out_dtype);
             if (rc != TM_ERR_UNSUPPORTED) return rc;
         }
-        if (skinny && M <= SKINNY_ROWS)
-            return tm_gemm_skinny(x_, ldx, L.w, L.bias, L.bias_dtype, out, ldc, M, L.N, L.K, out_dtype, 0, nullptr, 0, stream);
-        if (library) {
-            const int rc = tm_gemm_library(x_, ldx, L.w, L.K, L.bias, L.bias_dtype, out, ldc, out_dtype == TM_F32, M, L.N, L.K,
-                                           lib_ws, lib_ws_bytes, stream);
+        if (skinny && M <= TM_SKINNY_ROWS)
+            return tm_gemm_skinny(x, ldx, L.w, L.bias, L.bias_dtype, out, ldc, M, L.N, L.K, out_dtype, 0, nullptr, 0, stream);
+        {
+            const int rc = library(L, x, ldx, M, out, ldc, out_dtype);
             if (rc != TM_ERR_UNSUPPORTED) return rc;
         }
         if (skinny) {
             const int es = elem_size(dtype), eo = elem_size(out_dtype);
-            for (int r0 = 0; r0 < M; r0 += SKINNY_MAX_ROWS) {
-                const int m = M - r0 < SKINNY_MAX_ROWS ? M - r0 : SKINNY_MAX_ROWS;
-                const int rc = tm_gemm_skinny((const char*)x_ + (size_t)r0 * ldx * es, ldx, L.w, L.bias, L.bias_dtype,
+            for (int r0 = 0; r0 < M; r0 += TM_SKINNY_MAX_ROWS) {
+                const int m = M - r0 < TM_SKINNY_MAX_ROWS ? M - r0 : TM_SKINNY_MAX_ROWS;
+                const int rc = tm_gemm_skinny((const char*)x + (size_t)r0 * ldx * es, ldx, L.w, L.bias, L.bias_dtype,
                                               (char*)out + (size_t)r0 * ldc * eo, ldc, m, L.N, L.K, out_dtype, 0, nullptr, 0, stream);
                 if (rc) return rc;
             }
             return TM_OK;
         }
-        return tm_gemm_nt_tiled(x_, ldx, L.w, L.bias, L.bias_dtype, out, ldc, M, L.N, L.K, dtype, out_dtype, stream);
+        return tm_gemm_nt_tiled(x, ldx, L.w, L.bias, L.bias_dtype, out, ldc, M, L.N, L.K, dtype, out_dtype, stream);
     }
 
-    // resid += round(x W^T + b) in the product's epilogue where a kernel does that; else the product goes to
-    // delta_buf and is added by the next norm.
-    int project_into_residual(const TmLinear& L, const void* x_, int ldx, int M) {
-        if (L.dtype == dtype) {
-            if (L.packed_parts == 1 && packed_ok(L, x_, ldx, M, dtype)) {
-                delta = nullptr;
-                return tm_gemm_skinny_packed(x_, ldx, L.packed, L.packed_rows, L.bias, L.bias_dtype, nullptr, L.N, M, L.N, L.K,
-                                             TM_BF16, 0, resid, L.N, stream);
-            }
-            if (M > 0 && M <= SKINNY_ROWS && skinny_ok(L, x_, ldx, dtype)) {
-                delta = nullptr;
-                return tm_gemm_skinny(x_, ldx, L.w, L.bias, L.bias_dtype, nullptr, L.N, M, L.N, L.K, TM_BF16, 0, resid, L.N, stream);
-            }
+    // Is there a kernel that adds round(x W^T + b) into a 32-bit accumulator in its epilogue?
+    bool accumulates(const TmLinear& L, int dtype, const void* x, int ldx, int M) const {
+        if (L.dtype != dtype || M <= 0) return false;
+        return (L.packed_parts == 1 && packed_ok(L, x, ldx, M, dtype)) || (M <= TM_SKINNY_ROWS && skinny_ok(L, x, ldx, dtype));
+    }
+
+    int accumulate(const TmLinear& L, int dtype, const void* x, int ldx, int M, float* accum, int ldacc) const {
+        if (L.packed_parts == 1 && packed_ok(L, x, ldx, M, dtype))
+            return tm_gemm_skinny_packed(x, ldx, L.packed, L.packed_rows, L.bias, L.bias_dtype, nullptr, L.N, M, L.N, L.K, TM_BF16,
+                                         0, accum, ldacc, stream);
+        return tm_gemm_skinny(x, ldx, L.w, L.bias, L.bias_dtype, nullptr, L.N, M, L.N, L.K, TM_BF16, 0, accum, ldacc, stream);
+    }
+};
+
+struct Run {
+    const TmProgram* p;
+    const TmStep* s;
+    hipStream_t stream;
+    Products products;
+    int dtype;
+    bool labels;
+    // what crosses between operations
+    float* resid;
+    const void* delta;                  // product output still to be added to the residual stream
+    const void* x_in;                   // the next operation's input, already normed
+    const void* qkv_in;                 // the next (attention) operation's q|k|v, already encoded and stored
+    bool accumulate;
+    // workspace
+    void *x, *qkv, *attn, *gu, *act, *delta_buf, *hnorm;
+    float *part_o, *part_ml;
+
+    struct Label {
+        const Run* r;
+        int op, label;
+        Label(const Run* r_, int op_, int label_) : r(r_), op(op_), label(label_) {
+            if (r->labels && r->p->hook) r->p->hook(r->p->hook_user, op, label, 1);
+        }
+        ~Label() {
+            if (r->labels && r->p->hook) r->p->hook(r->p->hook_user, op, label, 0);
+        }
+    };
+
+    int linear(const TmLinear& L, const void* x_, int ldx, int M, void* out, int ldc, int out_dtype) {
+        return products.linear(L, dtype, x_, ldx, M, out, ldc, out_dtype);
+    }
+
+    // resid += round(x W^T + b) in the product's epilogue where a kernel does that and the caller lets it; else the
+    // product goes to delta_buf and is added by the next norm (or handed back).
+    int project(const TmLinear& L, const void* x_, int ldx, int M) {
+        if (accumulate && resid && products.accumulates(L, dtype, x_, ldx, M)) {
+            delta = nullptr;
+            return products.accumulate(L, dtype, x_, ldx, M, resid, L.N);
         }
         delta = delta_buf;
         return linear(L, x_, ldx, M, delta_buf, L.N, dtype);
@@ -150,12 +202,20 @@ struct Run {
 
     // x = norm(resid + delta), resid updated
     int normed(const TmNorm& n) {
+        if (!n.w || !resid) return TM_ERR_ARG;
         const int rc = tm_add_rmsnorm(resid, delta, nullptr, n.w, n.w_dtype, x, dtype, s->T, p->hidden, n.eps, stream);
         delta = nullptr;
         return rc;
     }
 
-    int attention(const TmAttentionOp& a) {
+    int embedding(int op, const TmEmbedOp& e) {
+        Label l(this, op, TM_LABEL_EMBED);
+        if (!resid) return TM_ERR_ARG;
+        delta = nullptr;
+        return tm_embed_gather(e.table, e.dtype, s->token_ids, resid, s->T, p->hidden, e.V, stream);
+    }
+
+    int attention(int op, const TmAttentionOp& a) {
         const int T = s->T, S = s->S, nd = s->num_decode, tp = T - nd, hidden = p->hidden;
         const int HD = a.H * a.D, QKV = (a.H + 2 * a.KVH) * a.D;
         if (a.group < 0 || a.group >= s->num_groups) return TM_ERR_ARG;
@@ -166,113 +226,179 @@ struct Run {
         void* vp = a.write ? a.v_pool : nullptr;
         if (a.rot > 0 && s->max_context_len > a.max_positions) return TM_ERR_ARG;       // beyond the rotary table
         if (!tables || W <= 0 || (long long)W * a.page < s->max_context_len) return TM_ERR_ARG;   // a table that does not reach the newest position
+        if (a.write && !slots) return TM_ERR_ARG;
+        if (!s->positions || !s->context_lens || !s->seq_of_token) return TM_ERR_ARG;
         const bool tables_fusable = a.rot == a.D && a.cos_t && a.sin_t;
         const bool bias_ok = !a.qkv.bias || aligned(a.qkv.bias, 16);
         const void* q = nullptr;
         int q_stride = 0;
         int rc = TM_OK;
-        // 1. the kernel that starts at the norm (at most 16 tokens)
-        if (dtype == TM_BF16 && a.D % 32 == 0 && delta == nullptr && a.norm.w && tables_fusable &&
-            fused_decode_ok(resid, a.qkv, T) && is_pow2(a.page) && bias_ok) {
-            rc = tm_fused_norm_qkv_rope(resid, a.norm.w, a.norm.w_dtype, a.norm.eps, T, hidden, a.qkv.packed, a.qkv.bias,
-                                        a.qkv.bias_dtype, qkv, a.H, a.KVH, a.D, a.cos_t, a.sin_t, s->positions, slots, kp, vp,
-                                        a.page, stream);
-            q = qkv;
-            q_stride = HD;
-            ++p->taken[TM_QKV_FROM_NORM];
+        if (qkv_in) {                       // projected, encoded and stored by the caller
+            q = qkv_in;
+            q_stride = QKV;
+            qkv_in = nullptr;
         } else {
-            if ((rc = normed(a.norm))) return rc;
-            // 2. the normed input kept in LDS (17 to 48 tokens)
-            if (tables_fusable && a.D % 32 == 0 && panel_ok(a.qkv, x, hidden, T, dtype) && is_pow2(a.page) && bias_ok) {
-                rc = tm_panel_qkv_rope(x, hidden, T, hidden, a.qkv.packed, a.qkv.bias, a.qkv.bias_dtype, qkv, a.H, a.KVH, a.D,
-                                       a.cos_t, a.sin_t, s->positions, slots, kp, vp, a.page, stream);
+            Label l(this, op, TM_LABEL_QKV);
+            const bool own_norm = x_in == nullptr;
+            // 1. the kernel that starts at the norm (at most 16 tokens)
+            if (own_norm && dtype == TM_BF16 && a.qkv.dtype == TM_BF16 && a.D % 32 == 0 && delta == nullptr && a.norm.w &&
+                tables_fusable && fused_decode_ok(resid, a.qkv, T) && is_pow2(a.page) && bias_ok) {
+                rc = tm_fused_norm_qkv_rope(resid, a.norm.w, a.norm.w_dtype, a.norm.eps, T, hidden, a.qkv.packed, a.qkv.bias,
+                                            a.qkv.bias_dtype, qkv, a.H, a.KVH, a.D, a.cos_t, a.sin_t, s->positions, slots, kp, vp,
+                                            a.page, stream);
                 q = qkv;
                 q_stride = HD;
-                ++p->taken[TM_QKV_PANEL];
+                ++p->taken[TM_QKV_FROM_NORM];
             } else {
-                // 3. product, then rotation and cache write
-                if ((rc = linear(a.qkv, x, hidden, T, qkv, QKV, dtype))) return rc;
-                if (a.rot > 0 || a.write)
-                    rc = tm_rope_kv_write(qkv, dtype, T, a.H, a.KVH, a.D, a.rot, a.rot > 0 ? a.cos_t : nullptr,
-                                          a.rot > 0 ? a.sin_t : nullptr, a.rot > 0 ? s->positions : nullptr, slots, kp, vp,
-                                          a.write ? a.page : 0, a.write ? 1 : 0, stream);
-                q = qkv;
-                q_stride = QKV;
-                ++p->taken[TM_QKV_PLAIN];
+                const void* xn = x_in;
+                x_in = nullptr;
+                if (own_norm) {
+                    if ((rc = normed(a.norm))) return rc;
+                    xn = x;
+                }
+                // 2. the normed input kept in LDS (17 to 48 tokens)
+                if (tables_fusable && a.D % 32 == 0 && a.qkv.dtype == TM_BF16 && panel_ok(a.qkv, xn, hidden, T, dtype) &&
+                    is_pow2(a.page) && bias_ok) {
+                    rc = tm_panel_qkv_rope(xn, hidden, T, hidden, a.qkv.packed, a.qkv.bias, a.qkv.bias_dtype, qkv, a.H, a.KVH, a.D,
+                                           a.cos_t, a.sin_t, s->positions, slots, kp, vp, a.page, stream);
+                    q = qkv;
+                    q_stride = HD;
+                    ++p->taken[TM_QKV_PANEL];
+                } else {
+                    // 3. product, then rotation and cache write
+                    if ((rc = linear(a.qkv, xn, hidden, T, qkv, QKV, dtype))) return rc;
+                    if (a.rot > 0 || a.write)
+                        rc = tm_rope_kv_write(qkv, dtype, T, a.H, a.KVH, a.D, a.rot, a.rot > 0 ? a.cos_t : nullptr,
+                                              a.rot > 0 ? a.sin_t : nullptr, a.rot > 0 ? s->positions : nullptr, slots, kp, vp,
+                                              a.write ? a.page : 0, a.write ? 1 : 0, stream);
+                    q = qkv;
+                    q_stride = QKV;
+                    ++p->taken[TM_QKV_PLAIN];
+                }
             }
+            if (rc) return rc;
         }
-        if (rc) return rc;
-        // attention over the cache
-        const int es = elem_size(dtype);
-        const bool page_ok = a.page >= 16 && is_pow2(a.page);
-        const bool head_mfma = a.D == 32 || a.D == 64 || a.D == 96 || a.D == 128;
-        bool done_prefill = false, done_decode = false;
-        if (tp && s->n_tiles > 0 && dtype == TM_BF16 && head_mfma && page_ok) {
-            rc = tm_attn_prefill_mfma(q, q_stride, attn, HD, a.k_pool, a.v_pool, tables, W, s->prefill_tiles, s->n_tiles, a.H,
-                                      a.KVH, a.D, a.page, a.scale, a.window, stream);
-            done_prefill = true;
-        } else if (tp && s->n_tiles > 0 && dtype == TM_F32 && a.D % 16 == 0 && a.D >= 16 && a.D <= 128 && page_ok &&
-                   q_stride % 4 == 0) {
-            rc = tm_attn_prefill_f32(q, q_stride, attn, HD, a.k_pool, a.v_pool, tables, W, s->prefill_tiles, s->n_tiles, a.H,
-                                     a.KVH, a.D, a.page, a.scale, a.window, stream);
-            done_prefill = true;
-        }
-        if (rc) return rc;
-        const char* q_dec = (const char*)q + (size_t)tp * q_stride * es;
-        char* out_dec = (char*)attn + (size_t)tp * HD * es;
-        if (nd && dtype == TM_BF16 && head_mfma && page_ok && a.H / a.KVH <= 16) {
-            const int chunks = (s->max_decode_context + DECODE_CHUNK - 1) / DECODE_CHUNK;
-            const bool split = nd * a.KVH < DECODE_SPLIT_PAIRS && chunks > 1;
-            rc = tm_attn_decode_mfma(q_dec, q_stride, out_dec, HD, a.k_pool, a.v_pool, tables + (size_t)(S - nd) * W, W,
-                                     s->context_lens + (S - nd), split ? part_o : nullptr, split ? part_ml : nullptr, chunks, nd,
-                                     a.H, a.KVH, a.D, a.page, a.scale, a.window, stream);
-            done_decode = true;
-        }
-        if (rc) return rc;
-        if (tp && !done_prefill && nd && !done_decode) {
-            rc = tm_attn_paged_generic(q, q_stride, attn, HD, a.k_pool, a.v_pool, tables, W, s->seq_of_token, s->positions, T,
-                                       a.H, a.KVH, a.D, a.page, a.scale, a.window, dtype, stream);
-        } else {
-            if (tp && !done_prefill)
-                rc = tm_attn_paged_generic(q, q_stride, attn, HD, a.k_pool, a.v_pool, tables, W, s->seq_of_token, s->positions, tp,
+        {
+            Label l(this, op, TM_LABEL_ATTENTION);
+            const int es = elem_size(dtype);
+            const bool page_ok = a.page >= 16 && is_pow2(a.page);
+            const bool head_mfma = a.D == 32 || a.D == 64 || a.D == 96 || a.D == 128;
+            const bool q_ok = aligned(q, 16) && q_stride % 8 == 0;
+            bool done_prefill = false, done_decode = false;
+            if (tp && s->n_tiles > 0 && s->prefill_tiles && dtype == TM_BF16 && head_mfma && page_ok && q_ok) {
+                rc = tm_attn_prefill_mfma(q, q_stride, attn, HD, a.k_pool, a.v_pool, tables, W, s->prefill_tiles, s->n_tiles, a.H,
+                                          a.KVH, a.D, a.page, a.scale, a.window, stream);
+                done_prefill = true;
+            } else if (tp && s->n_tiles > 0 && s->prefill_tiles && dtype == TM_F32 && a.D % 16 == 0 && a.D >= 16 &&
+                       a.D <= 128 && page_ok && q_stride % 4 == 0 && aligned(q, 16)) {
+                rc = tm_attn_prefill_f32(q, q_stride, attn, HD, a.k_pool, a.v_pool, tables, W, s->prefill_tiles, s->n_tiles, a.H,
+                                         a.KVH, a.D, a.page, a.scale, a.window, stream);
+                done_prefill = true;
+            }
+            if (rc) return rc;
+            const char* q_dec = (const char*)q + (size_t)tp * q_stride * es;
+            char* out_dec = (char*)attn + (size_t)tp * HD * es;
+            if (nd && dtype == TM_BF16 && head_mfma && page_ok && a.H / a.KVH <= 16 && q_ok) {
+                const bool split = tm_decode_splits(nd, a.KVH, s->max_decode_context);
+                rc = tm_attn_decode_mfma(q_dec, q_stride, out_dec, HD, a.k_pool, a.v_pool, tables + (size_t)(S - nd) * W, W,
+                                         s->context_lens + (S - nd), split ? part_o : nullptr, split ? part_ml : nullptr,
+                                         tm_decode_chunks(s->max_decode_context), nd, a.H, a.KVH, a.D, a.page, a.scale, a.window,
+                                         stream);
+                done_decode = true;
+            }
+            if (rc) return rc;
+            if (tp && !done_prefill && nd && !done_decode) {
+                rc = tm_attn_paged_generic(q, q_stride, attn, HD, a.k_pool, a.v_pool, tables, W, s->seq_of_token, s->positions, T,
                                            a.H, a.KVH, a.D, a.page, a.scale, a.window, dtype, stream);
-            if (!rc && nd && !done_decode)
-                rc = tm_attn_paged_generic(q_dec, q_stride, out_dec, HD, a.k_pool, a.v_pool, tables, W, s->seq_of_token + tp,
-                                           s->positions + tp, nd, a.H, a.KVH, a.D, a.page, a.scale, a.window, dtype, stream);
+            } else {
+                if (tp && !done_prefill)
+                    rc = tm_attn_paged_generic(q, q_stride, attn, HD, a.k_pool, a.v_pool, tables, W, s->seq_of_token, s->positions,
+                                               tp, a.H, a.KVH, a.D, a.page, a.scale, a.window, dtype, stream);
+                if (!rc && nd && !done_decode)
+                    rc = tm_attn_paged_generic(q_dec, q_stride, out_dec, HD, a.k_pool, a.v_pool, tables, W, s->seq_of_token + tp,
+                                               s->positions + tp, nd, a.H, a.KVH, a.D, a.page, a.scale, a.window, dtype, stream);
+            }
+            if (rc) return rc;
         }
-        if (rc) return rc;
-        return project_into_residual(a.o, attn, HD, T);
+        Label l(this, op, TM_LABEL_O_PROJ);
+        return project(a.o, attn, HD, T);
     }
 
-    int feed_forward(const TmFfnOp& f) {
+    int feed_forward(int op, const TmFfnOp& f) {
         const int T = s->T, hidden = p->hidden;
         int rc = TM_OK;
-        const bool plain = f.gate_up.dtype == dtype && f.gate_up.bias == nullptr;
-        if (dtype == TM_BF16 && f.gate_up.bias == nullptr && f.I % 4 == 0 && delta == nullptr && f.norm.w &&
-            f.gate_up.packed_parts == 2 && f.gate_up.packed_rows == 16 && fused_decode_ok(resid, f.gate_up, T)) {
-            rc = tm_fused_norm_gate_up_silu(resid, f.norm.w, f.norm.w_dtype, f.norm.eps, T, hidden, f.gate_up.packed, act, f.I, stream);
-            ++p->taken[TM_GATE_UP_FROM_NORM];
-        } else {
-            if ((rc = normed(f.norm))) return rc;
-            if (plain && f.gate_up.packed_parts == 2 && f.gate_up.packed_rows == 16 && packed_ok(f.gate_up, x, hidden, T, dtype)) {
-                rc = tm_gemm_skinny_packed(x, hidden, f.gate_up.packed, 16, nullptr, TM_NONE, act, f.I, T, f.I, hidden, TM_BF16, 1,
-                                           nullptr, 0, stream);
-            } else if (plain && T <= SKINNY_ROWS && skinny_ok(f.gate_up, x, hidden, dtype)) {
-                rc = tm_gemm_skinny(x, hidden, f.gate_up.w, nullptr, TM_NONE, act, f.I, T, f.I, hidden, TM_BF16, 1, nullptr, 0, stream);
-            } else if (plain && f.gate_up.packed_parts == 2 && f.gate_up.packed_rows == 16 && f.I % 4 == 0 &&
-                       panel_ok(f.gate_up, x, hidden, T, dtype)) {
-                rc = tm_panel_gate_up_silu(x, hidden, T, hidden, f.gate_up.packed, act, f.I, stream);
-                ++p->taken[TM_GATE_UP_PANEL];
+        {
+            Label l(this, op, TM_LABEL_GATE_UP);
+            const bool own_norm = x_in == nullptr;
+            const bool plain = f.gate_up.dtype == dtype && f.gate_up.bias == nullptr;
+            const bool two_parts = f.gate_up.packed_parts == 2 && f.gate_up.packed_rows == 16;
+            if (own_norm && dtype == TM_BF16 && plain && f.I % 4 == 0 && delta == nullptr && f.norm.w && two_parts &&
+                fused_decode_ok(resid, f.gate_up, T)) {
+                rc = tm_fused_norm_gate_up_silu(resid, f.norm.w, f.norm.w_dtype, f.norm.eps, T, hidden, f.gate_up.packed, act, f.I, stream);
+                ++p->taken[TM_GATE_UP_FROM_NORM];
             } else {
-                if ((rc = linear(f.gate_up, x, hidden, T, gu, 2 * f.I, dtype))) return rc;
-                rc = tm_silu_mul(gu, act, dtype, T, f.I, stream);
-                ++p->taken[TM_GATE_UP_PLAIN];
+                const void* xn = x_in;
+                x_in = nullptr;
+                if (own_norm) {
+                    if ((rc = normed(f.norm))) return rc;
+                    xn = x;
+                }
+                if (plain && two_parts && packed_ok(f.gate_up, xn, hidden, T, dtype)) {
+                    rc = tm_gemm_skinny_packed(xn, hidden, f.gate_up.packed, 16, nullptr, TM_NONE, act, f.I, T, f.I, hidden, TM_BF16, 1,
+                                               nullptr, 0, stream);
+                    ++p->taken[TM_GATE_UP_PLAIN];
+                } else if (plain && T <= TM_SKINNY_ROWS && skinny_ok(f.gate_up, xn, hidden, dtype)) {
+                    rc = tm_gemm_skinny(xn, hidden, f.gate_up.w, nullptr, TM_NONE, act, f.I, T, f.I, hidden, TM_BF16, 1, nullptr, 0, stream);
+                    ++p->taken[TM_GATE_UP_PLAIN];
+                } else if (plain && two_parts && f.I % 4 == 0 && panel_ok(f.gate_up, xn, hidden, T, dtype)) {
+                    rc = tm_panel_gate_up_silu(xn, hidden, T, hidden, f.gate_up.packed, act, f.I, stream);
+                    ++p->taken[TM_GATE_UP_PANEL];
+                } else {
+                    if ((rc = linear(f.gate_up, xn, hidden, T, gu, 2 * f.I, dtype))) return rc;
+                    rc = tm_silu_mul(gu, act, dtype, T, f.I, stream);
+                    ++p->taken[TM_GATE_UP_PLAIN];
+                }
             }
+            if (rc) return rc;
         }
-        if (rc) return rc;
-        return project_into_residual(f.down, act, f.I, T);
+        Label l(this, op, TM_LABEL_DOWN);
+        return project(f.down, act, f.I, T);
+    }
+
+    int head(int op, const TmFinalOp& f, float* logits) {
+        const int R = s->R;
+        if (R == 0) return TM_OK;
+        if (!logits || !s->logit_rows) return TM_ERR_ARG;
+        const void* h = x_in;                   // rows already normed (R of them), or the residual's rows to norm
+        x_in = nullptr;
+        if (!h) {
+            Label l(this, op, TM_LABEL_NORM);
+            if (!f.norm.w || !resid) return TM_ERR_ARG;
+            const int rc = tm_add_rmsnorm(resid, delta, s->logit_rows, f.norm.w, f.norm.w_dtype, hnorm, dtype, R, p->hidden,
+                                          f.norm.eps, stream);
+            if (rc) return rc;
+            h = hnorm;
+        }
+        delta = nullptr;
+        Label l(this, op, TM_LABEL_HEAD);
+        return linear(f.head, h, p->hidden, R, logits, f.head.N, TM_F32);
     }
 };
+
+bool linear_valid(const TmLinear& L) {
+    return L.w && L.N > 0 && L.K > 0 && (L.dtype == TM_F32 || L.dtype == TM_BF16) &&
+           (L.packed == nullptr || (L.packed_rows > 0 && L.packed_parts > 0 && L.dtype == TM_BF16));
+}
+
+// A matrix a program of type `dtype` can multiply by: of that type, or 32-bit under bfloat16 activations.
+bool linear_fits(TmProgram* p, const TmLinear& L) {
+    if (!linear_valid(L)) return false;
+    if (L.dtype == p->dtype) return true;
+    if (L.dtype != TM_F32 || p->dtype != TM_BF16) return false;
+    if (L.K > p->max_wide_in) p->max_wide_in = L.K;
+    if (L.N > p->max_wide_out) p->max_wide_out = L.N;
+    return true;
+}
 
 }  // namespace
 
@@ -288,50 +414,62 @@ TmProgram* tm_program_create(int dtype, int hidden) {
 
 void tm_program_destroy(TmProgram* p) { delete p; }
 
-static bool linear_valid(const TmLinear& L, int dtype) {
-    return L.w && L.N > 0 && L.K > 0 && L.dtype == dtype && (L.packed == nullptr || (L.packed_rows > 0 && L.packed_parts > 0));
+void tm_program_set_hook(TmProgram* p, TmHook hook, void* user) {
+    if (!p) return;
+    p->hook = hook;
+    p->hook_user = user;
 }
 
-int tm_program_set_embedding(TmProgram* p, const TmEmbedOp* e) {
-    if (!p || !e || !e->table || e->hidden != p->hidden || e->V <= 0) return TM_ERR_ARG;
-    p->embed = *e;
-    p->has_embed = true;
+int tm_program_set_tune(TmProgram* p, int candidates, int every) {
+    if (!p || candidates < 0 || candidates > 32 || (every && candidates < 2)) return TM_ERR_ARG;
+    p->tune = TmTune{candidates, 3, every ? 1 : 0};
     return TM_OK;
+}
+
+int tm_program_add_embedding(TmProgram* p, const TmEmbedOp* e) {
+    if (!p || !e || !e->table || e->hidden != p->hidden || e->V <= 0) return -1;
+    Op op{};
+    op.kind = OP_EMBED;
+    op.embed = *e;
+    p->ops.push_back(op);
+    return (int)p->ops.size() - 1;
 }
 
 int tm_program_add_attention(TmProgram* p, const TmAttentionOp* a) {
     if (!p || !a || a->H <= 0 || a->KVH <= 0 || a->H % a->KVH || a->D <= 0 || !a->k_pool || !a->v_pool || a->page <= 0 ||
-        !a->norm.w || !linear_valid(a->qkv, p->dtype) || !linear_valid(a->o, p->dtype) || a->qkv.K != p->hidden ||
-        a->qkv.N != (a->H + 2 * a->KVH) * a->D || a->o.K != a->H * a->D || a->o.N != p->hidden || a->window < 0 ||
-        a->rot < 0 || a->rot > a->D || (a->rot > 0 && (!a->cos_t || !a->sin_t)))
-        return TM_ERR_ARG;
+        !linear_fits(p, a->qkv) || !linear_fits(p, a->o) || a->qkv.K != p->hidden || a->qkv.N != (a->H + 2 * a->KVH) * a->D || a->o.K != a->H * a->D || a->o.N != p->hidden ||
+        a->window < 0 || a->rot < 0 || a->rot > a->D || (a->rot > 0 && (!a->cos_t || !a->sin_t)))
+        return -1;
     Op op{};
-    op.kind = 0;
+    op.kind = OP_ATTENTION;
     op.att = *a;
     p->ops.push_back(op);
     if (a->qkv.N > p->max_qkv) p->max_qkv = a->qkv.N;
+    if (a->H > p->max_heads) p->max_heads = a->H;
     if (a->H * a->D > p->max_heads_d) p->max_heads_d = a->H * a->D;
-    return TM_OK;
+    return (int)p->ops.size() - 1;
 }
 
 int tm_program_add_feed_forward(TmProgram* p, const TmFfnOp* f) {
-    if (!p || !f || f->I <= 0 || !f->norm.w || !linear_valid(f->gate_up, p->dtype) || !linear_valid(f->down, p->dtype) ||
-        f->gate_up.K != p->hidden || f->gate_up.N != 2 * f->I || f->down.K != f->I || f->down.N != p->hidden)
-        return TM_ERR_ARG;
+    if (!p || !f || f->I <= 0 || !linear_fits(p, f->gate_up) || !linear_fits(p, f->down) || f->gate_up.K != p->hidden || f->gate_up.N != 2 * f->I || f->down.K != f->I ||
+        f->down.N != p->hidden)
+        return -1;
     Op op{};
-    op.kind = 1;
+    op.kind = OP_FEED_FORWARD;
     op.ffn = *f;
     p->ops.push_back(op);
     if (2 * f->I > p->max_gu) p->max_gu = 2 * f->I;
     if (f->I > p->max_act) p->max_act = f->I;
-    return TM_OK;
+    return (int)p->ops.size() - 1;
 }
 
-int tm_program_set_final(TmProgram* p, const TmFinalOp* f) {
-    if (!p || !f || !f->norm.w || !linear_valid(f->head, p->dtype) || f->head.K != p->hidden) return TM_ERR_ARG;
-    p->final_op = *f;
-    p->has_final = true;
-    return TM_OK;
+int tm_program_add_head(TmProgram* p, const TmFinalOp* f) {
+    if (!p || !f || !linear_fits(p, f->head) || f->head.K != p->hidden) return -1;
+    Op op{};
+    op.kind = OP_HEAD;
+    op.head = *f;
+    p->ops.push_back(op);
+    return (int)p->ops.size() - 1;
 }
 
 void tm_program_counters(const TmProgram* p, long long* out) {
@@ -344,7 +482,6 @@ size_t tm_program_workspace_bytes(const TmProgram* p, int T, int R, int num_deco
     if (!p || T <= 0) return 0;
     const size_t es = elem_size(p->dtype);
     size_t n = 0;
-    n += align_up((size_t)T * p->hidden * 4);                        // residual stream
     n += align_up((size_t)T * p->hidden * es);                       // normed input
     n += align_up((size_t)T * p->max_qkv * es);                      // q|k|v
     n += align_up((size_t)T * p->max_heads_d * es);                  // attention output
@@ -352,25 +489,25 @@ size_t tm_program_workspace_bytes(const TmProgram* p, int T, int R, int num_deco
     n += align_up((size_t)T * p->max_act * es);                      // silu(gate) * up
     n += align_up((size_t)T * p->hidden * es);                       // a product's output still to be added
     n += align_up((size_t)(R > 0 ? R : 1) * p->hidden * es);         // normed rows for the head
-    size_t heads = 0, heads_d = 0;
-    for (const Op& op : p->ops)
-        if (op.kind == 0) {
-            if ((size_t)op.att.H > heads) heads = op.att.H;
-            if ((size_t)op.att.H * op.att.D > heads_d) heads_d = (size_t)op.att.H * op.att.D;
-        }
-    const size_t chunks = (size_t)(max_decode_context + DECODE_CHUNK - 1) / DECODE_CHUNK;
-    n += align_up((size_t)num_decode * heads_d * chunks * 4);        // split decode attention: partial values
-    n += align_up((size_t)num_decode * heads * chunks * 2 * 4);      // ... and their (max, sum)
+    const size_t chunks = (size_t)tm_decode_chunks(max_decode_context > 0 ? max_decode_context : 1);
+    n += align_up((size_t)num_decode * p->max_heads_d * chunks * 4); // split decode attention: partial values
+    n += align_up((size_t)num_decode * p->max_heads * chunks * 2 * 4);   // ... and their (max, sum)
+    const size_t rows = (size_t)(T > R ? T : R);
+    n += align_up(rows * p->max_wide_in * 4);                        // 32-bit copies around the product of a 32-bit matrix
+    n += align_up(rows * p->max_wide_out * 4);
     return n;
 }
 
-int tm_program_run(const TmProgram* p, const TmStep* s, void* workspace, size_t workspace_bytes, void* library_workspace,
-                   size_t library_workspace_bytes, float* logits, hipStream_t stream) {
-    if (!p || !s || !p->has_embed || !p->has_final || s->T <= 0 || s->S <= 0 || s->num_decode < 0 || s->num_decode > s->S ||
-        s->R < 0 || !workspace || !aligned(workspace, 256) || s->num_groups < 0 || s->num_groups > TM_MAX_GROUPS)
+int tm_program_run(const TmProgram* p, int first, int count, const TmStep* s, TmStream* io, void* workspace,
+                   size_t workspace_bytes, void* library_workspace, size_t library_workspace_bytes, float* logits,
+                   int flags, hipStream_t stream) {
+    if (!p || !s || !io || first < 0 || count <= 0 || (size_t)first + (size_t)count > p->ops.size() || s->T <= 0 || s->S < 0 ||
+        s->num_decode < 0 || s->num_decode > s->S || s->num_decode > s->T || s->R < 0 || !workspace || !aligned(workspace, 256) ||
+        s->num_groups < 0 || s->num_groups > TM_MAX_GROUPS)
         return TM_ERR_ARG;
     if (workspace_bytes < tm_program_workspace_bytes(p, s->T, s->R, s->num_decode, s->max_decode_context)) return TM_ERR_ARG;
-    if (s->R > 0 && !logits) return TM_ERR_ARG;
+    if (!io->resid && (io->accumulate || count != 1 || (!io->x && !io->qkv))) return TM_ERR_ARG;
+    if (io->qkv && p->ops[first].kind != OP_ATTENTION) return TM_ERR_ARG;
     const size_t es = elem_size(p->dtype);
     const int T = s->T, R = s->R;
     char* w = (char*)workspace;
@@ -380,8 +517,12 @@ int tm_program_run(const TmProgram* p, const TmStep* s, void* workspace, size_t 
         return (void*)at;
     };
     Run r{};
-    r.p = p; r.s = s; r.stream = stream; r.lib_ws = library_workspace; r.lib_ws_bytes = library_workspace_bytes; r.dtype = p->dtype;
-    r.resid = (float*)take((size_t)T * p->hidden * 4);
+    r.p = p; r.s = s; r.stream = stream; r.dtype = p->dtype;
+    r.products.stream = stream; r.products.lib_ws = library_workspace; r.products.lib_ws_bytes = library_workspace_bytes;
+    r.products.tune = p->tune;
+    if (flags & TM_RUN_TUNE_AT_ONCE) r.products.tune.after = 1;
+    r.labels = (flags & TM_RUN_LABELS) != 0;
+    r.resid = io->resid; r.delta = io->delta; r.x_in = io->x; r.qkv_in = io->qkv; r.accumulate = io->accumulate != 0;
     r.x = take((size_t)T * p->hidden * es);
     r.qkv = take((size_t)T * p->max_qkv * es);
     r.attn = take((size_t)T * p->max_heads_d * es);
@@ -389,27 +530,64 @@ int tm_program_run(const TmProgram* p, const TmStep* s, void* workspace, size_t 
     r.act = take((size_t)T * p->max_act * es);
     r.delta_buf = take((size_t)T * p->hidden * es);
     r.hnorm = take((size_t)(R > 0 ? R : 1) * p->hidden * es);
-    size_t heads = 0, heads_d = 0;
-    for (const Op& op : p->ops)
-        if (op.kind == 0) {
-            if ((size_t)op.att.H > heads) heads = op.att.H;
-            if ((size_t)op.att.H * op.att.D > heads_d) heads_d = (size_t)op.att.H * op.att.D;
+    const size_t chunks = (size_t)tm_decode_chunks(s->max_decode_context > 0 ? s->max_decode_context : 1);
+    r.part_o = (float*)take((size_t)s->num_decode * p->max_heads_d * chunks * 4);
+    r.part_ml = (float*)take((size_t)s->num_decode * p->max_heads * chunks * 2 * 4);
+    const size_t rows = (size_t)(T > R ? T : R);
+    if (p->max_wide_in) r.products.wide_in = (float*)take(rows * p->max_wide_in * 4);
+    if (p->max_wide_out) r.products.wide_out = (float*)take(rows * p->max_wide_out * 4);
+    int rc = TM_OK;
+    for (int i = first; i < first + count && !rc; ++i) {
+        const Op& op = p->ops[i];
+        switch (op.kind) {
+            case OP_EMBED: rc = r.embedding(i, op.embed); break;
+            case OP_ATTENTION: rc = r.attention(i, op.att); break;
+            case OP_FEED_FORWARD: rc = r.feed_forward(i, op.ffn); break;
+            default: rc = r.head(i, op.head, logits); break;
         }
-    const size_t chunks = (size_t)(s->max_decode_context + DECODE_CHUNK - 1) / DECODE_CHUNK;
-    r.part_o = (float*)take((size_t)s->num_decode * heads_d * chunks * 4);
-    r.part_ml = (float*)take((size_t)s->num_decode * heads * chunks * 2 * 4);
-
-    int rc = tm_embed_gather(p->embed.table, p->embed.dtype, s->token_ids, r.resid, T, p->hidden, p->embed.V, stream);
-    if (rc) return rc;
-    for (const Op& op : p->ops) {
-        rc = op.kind == 0 ? r.attention(op.att) : r.feed_forward(op.ffn);
-        if (rc) return rc;
     }
-    if (R == 0) return TM_OK;
-    const TmFinalOp& f = p->final_op;
-    rc = tm_add_rmsnorm(r.resid, r.delta, s->logit_rows, f.norm.w, f.norm.w_dtype, r.hnorm, p->dtype, R, p->hidden, f.norm.eps, stream);
-    if (rc) return rc;
-    return r.linear(f.head, r.hnorm, p->hidden, R, logits, f.head.N, TM_F32);
+    io->delta = r.delta;
+    io->x = nullptr;
+    io->qkv = nullptr;
+    return rc;
+}
+
+int tm_linear_accumulates(const TmLinear* L, int x_dtype, const void* x, int ldx, int M) {
+    if (!L || !linear_valid(*L)) return 0;
+    Products pr{};
+    return pr.accumulates(*L, x_dtype, x, ldx, M) ? 1 : 0;
+}
+
+int tm_linear_run(const TmLinear* L, int x_dtype, const void* x, int ldx, int M, void* out, int ldc, int out_dtype,
+                  float* accum, int ldacc, void* library_workspace, size_t library_workspace_bytes, const TmTune* tune,
+                  hipStream_t stream) {
+    if (!L || !linear_valid(*L) || !x || M < 0 || ldx < L->K || (x_dtype != TM_F32 && x_dtype != TM_BF16)) return TM_ERR_ARG;
+    Products pr{};
+    pr.stream = stream; pr.lib_ws = library_workspace; pr.lib_ws_bytes = library_workspace_bytes;
+    pr.tune = tune ? *tune : TmTune{0, 3, 0};
+    if (accum) {
+        if (ldacc < L->N || !pr.accumulates(*L, x_dtype, x, ldx, M)) return TM_ERR_ARG;
+        return pr.accumulate(*L, x_dtype, x, ldx, M, accum, ldacc);
+    }
+    if (!out || ldc < L->N || (out_dtype != TM_F32 && out_dtype != TM_BF16) || (x_dtype == TM_F32 && out_dtype != TM_F32))
+        return TM_ERR_ARG;
+    return pr.linear(*L, x_dtype, x, ldx, M, out, ldc, out_dtype);
+}
+
+int tm_rule(const char* name) {
+    if (!name) return -1;
+    if (!strcmp(name, "skinny_rows")) return TM_SKINNY_ROWS;
+    if (!strcmp(name, "panel_rows")) return TM_PANEL_ROWS;
+    if (!strcmp(name, "stream_rows")) return TM_STREAM_ROWS;
+    if (!strcmp(name, "skinny_max_rows")) return TM_SKINNY_MAX_ROWS;
+    if (!strcmp(name, "gemv_f32_rows")) return TM_GEMV_F32_ROWS;
+    if (!strcmp(name, "decode_chunk")) return TM_DECODE_CHUNK;
+    if (!strcmp(name, "decode_split_pairs")) return TM_DECODE_SPLIT_PAIRS;
+    return -1;
+}
+
+int tm_decode_split_chunks(int requests, int kv_heads, int max_context) {
+    return tm_decode_splits(requests, kv_heads, max_context) ? tm_decode_chunks(max_context) : 0;
 }
 
 }  // extern "C"

@@ -49,14 +49,13 @@ class LLMEngine:
             check_positions(model.config, cfg.max_model_len)
             self.device, self.dtype = model.device, model.dtype
         self.model = model
-        if cfg.tune_gemm:
-            from tokenmill_amd.hip import ops
-            ops.gemm_library_tune(TUNE_CANDIDATES, every=cfg.tune_gemm_every)
         self.eos_ids = set(getattr(model.config, "eos_token_ids", ()) or ())
         pages = num_cache_pages(cfg, model, self.dtype, self.device)
         self.pools = CachePools(model, pages, cfg.block_size, cfg.max_num_seqs, self.dtype, self.device)
         self.cache = CacheManager(self.pools.windows, pages, cfg.block_size, cfg.max_num_seqs, cfg.watermark)
-        self.runner = ModelRunner(model, self.pools, max_positions=cfg.max_model_len, step_program=cfg.step_program)
+        # timing the library's algorithms is this engine's choice: it travels with the engine's own step program
+        tune = (TUNE_CANDIDATES, cfg.tune_gemm_every) if cfg.tune_gemm else None
+        self.runner = ModelRunner(model, self.pools, max_positions=cfg.max_model_len, tune=tune)
         if cfg.hip_graphs:
             from tokenmill_amd.engine.graphs import DecodeGraphs, StepGraphs
             self.runner.graphs = DecodeGraphs(self.runner, cfg)

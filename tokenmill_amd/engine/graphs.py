@@ -189,8 +189,8 @@ class DecodeGraphs:
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         # a first run outside the graph: lazy set-up happens here, and the library's products are timed now
-        with torch.cuda.stream(side), ops.gemm_library_tune_at_once():
-            runner.forward(step)
+        with torch.cuda.stream(side):
+            runner.forward(step, about_to_be_captured=True)
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
@@ -303,8 +303,8 @@ class StepGraphs:
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         # a first run outside the graph: lazy set-up happens here, and the library's products are timed now
-        with torch.cuda.stream(side), ops.gemm_library_tune_at_once():
-            runner.forward(step)
+        with torch.cuda.stream(side):
+            runner.forward(step, about_to_be_captured=True)
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()

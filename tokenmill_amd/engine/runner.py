@@ -16,7 +16,6 @@ from dataclasses import dataclass, field
 import numpy as np
 import torch
 
-from tokenmill_amd import profiling
 from tokenmill_amd.cache.manager import RELEASED, RequestCache
 from tokenmill_amd.cache.pool import CachePools
 from tokenmill_amd.parts.base import GroupStep, StepContext
@@ -36,14 +35,12 @@ class StepError(ValueError):
 
 
 class ModelRunner:
-    def __init__(self, model, pools: CachePools, max_positions: int, step_program: bool = True):
+    def __init__(self, model, pools: CachePools, max_positions: int, tune: tuple[int, bool] | None = None):
         self.model = model
         self.pools = pools
-        # the model's launch sequence as one call into the kernel library, where every part has an operation there
-        self.program = None
-        if step_program and getattr(model, "run", None) is not None and getattr(model, "dtype", None) is not None:
-            from tokenmill_amd.engine.program import StepProgram
-            self.program = StepProgram.compile(model, pools)
+        # the model's one forward pass: its parts' operations in run order, described once to the kernel library
+        # (``tune``: (candidates, every) if this runner's library products are to be timed)
+        self.program = model.program(pools.views, tune) if hasattr(model, "program") else None
         self.page_size = pools.page_size
         self.max_positions = max_positions
         self.device = model.device
@@ -310,9 +307,6 @@ class ModelRunner:
         ctx, _ = self.prepare(entries)
         return self.forward(ctx)
 
-    def forward(self, step: StepContext) -> torch.Tensor:
-        """The step's float32 logits [R, vocab]: through the library's step program where the model has
-        one, else (and while per-operation times are being collected) through the parts' own code."""
-        if self.program is not None and not profiling.on():
-            return self.program.run(step)
-        return self.model.forward(step, self.pools.views)
+    def forward(self, step: StepContext, about_to_be_captured: bool = False) -> torch.Tensor:
+        """The step's float32 logits [R, vocab], by the model's step program."""
+        return self.program.run(step, at_once=about_to_be_captured)

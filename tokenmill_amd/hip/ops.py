@@ -191,41 +191,59 @@ def library_workspace(device: torch.device) -> torch.Tensor:
 
 
 TUNE_AFTER_CALLS = 3        # a shape's candidates are timed when it is called this often (most shapes of a serving run come once)
-_tune = {"candidates": 0, "after": TUNE_AFTER_CALLS, "every": False}
-
-
-def gemm_library_tune(candidates: int, after: int = TUNE_AFTER_CALLS, every: bool = False) -> None:
-    """From now on a shape that is called the ``after``-th time with the same matrix (outside a graph capture) has up to
-    ``candidates`` of the library's algorithms timed on its own operands, and the fastest is kept
-    (0: the library's first choice, untimed). With ``every`` a shape that is timed at its first call
-    (``after`` = 1, see ``gemm_library_tune_at_once``) also tries every algorithm the library holds for
-    the operand types, not only those its heuristic names: about a second a shape, and an algorithm
-    found that way is kept only if it gives the first choice's result."""
-    _need(0 <= candidates <= 32 and after >= 1, "gemm_library_tune: 0 to 32 candidates, after >= 1 calls")
-    _need(not every or candidates >= 2, "gemm_library_tune: every algorithm is tried beside at least 2 candidates")
-    _check(library().tm_gemm_library_tune(c_int(candidates), c_int(after), c_int(1 if every else 0)), "gemm_library_tune")
-    _tune["candidates"], _tune["after"], _tune["every"] = candidates, after, every
+_tune_now: tuple[int, int, bool] | None = None
 
 
 @contextlib.contextmanager
-def gemm_library_tune_at_once():
-    """Inside, a shape is timed at its first call (if timing is on at all): for the run before a
-    graph capture, whose shapes are about to be replayed many times."""
-    candidates, after, every = _tune["candidates"], _tune["after"], _tune["every"]
-    if candidates < 2:
-        yield
-        return
-    gemm_library_tune(candidates, 1, every)
+def tuning(candidates: int, after: int = TUNE_AFTER_CALLS, every: bool = False):
+    """Inside, the library products that this module's ``linear`` and ``gemm_library`` launch time up to
+    ``candidates`` of the library's algorithms on their own operands when a shape is called the ``after``-th
+    time with the same matrix (outside a graph capture) and keep the fastest (``every``: a shape timed at its
+    first call also tries every algorithm the library holds for the operand types: about a second a shape,
+    and an algorithm found that way is kept only if it gives the first choice's result). Timing is a
+    property of the caller, not of the process: an engine that asks for it wraps its own steps in this, and
+    the plans of timed callers are kept apart from the plans of the others."""
+    global _tune_now
+    _need(0 <= candidates <= 32 and after >= 1, "tuning: 0 to 32 candidates, after >= 1 calls")
+    _need(not every or candidates >= 2, "tuning: every algorithm is tried beside at least 2 candidates")
+    saved, _tune_now = _tune_now, (candidates, after, every)
     try:
         yield
     finally:
-        gemm_library_tune(candidates, after, every)
+        _tune_now = saved
 
 
-def gemm_library(a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, out: torch.Tensor) -> bool:
+def _tune_arg(tune: tuple[int, int, bool] | None):
+    """The TmTune argument of a library product: ``tune`` if given, else what an open ``tuning()`` says, else null."""
+    from tokenmill_amd.hip.abi import TmTune
+    t = tune if tune is not None else _tune_now
+    if t is None or t[0] < 2:
+        return None
+    return ctypes.byref(TmTune(int(t[0]), int(t[1]), 1 if t[2] else 0))
+
+
+def rule(name: str) -> int:
+    """A number of the library's kernel-choosing rules (``csrc/choose.h``), for sizing a buffer or checking an
+    argument: "skinny_rows", "panel_rows", "stream_rows", "skinny_max_rows", "gemv_f32_rows", "decode_chunk",
+    "decode_split_pairs". The rules themselves are applied inside the library only."""
+    value = _rules.get(name)
+    if value is None:
+        from tokenmill_amd.hip.abi import bound
+        value = bound().tm_rule(name.encode())
+        _need(value >= 0, f"the kernel library has no rule named {name!r}")
+        _rules[name] = value
+    return value
+
+
+_rules: dict[str, int] = {}
+
+
+def gemm_library(a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, out: torch.Tensor,
+                 tune: tuple[int, int, bool] | None = None) -> bool:
     """out[M, N] = a[M, K] @ w[N, K]^T (+ bias[N]) by hipBLASLt: bfloat16 inputs, 32-bit sums, out
     bfloat16 or float32. The plan for a shape is made on its first call and kept. Returns False
-    (nothing written) if the library has no algorithm for this product."""
+    (nothing written) if the library has no algorithm for this product. ``tune``: (candidates, after, every)
+    as for ``tuning()``, which it overrides."""
     _gpu(a, w, bias, out)
     M, K = a.shape
     N = w.shape[0]
@@ -243,21 +261,18 @@ def gemm_library(a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, ou
     rc = library().tm_gemm_library(_p(a), c_int(lda), _p(w), c_int(K), _p(bias),
                                    c_int(code(bias.dtype) if bias is not None else -1), _p(out), c_int(ldc),
                                    c_int(1 if out.dtype == torch.float32 else 0), c_int(M), c_int(N), c_int(K),
-                                   _p(ws), ctypes.c_size_t(LIBRARY_WORKSPACE_BYTES), _stream())
+                                   _p(ws), ctypes.c_size_t(LIBRARY_WORKSPACE_BYTES), _tune_arg(tune), _stream())
     if rc == 3:
         return False
     _check(rc, "gemm_library")
     return True
 
 
-GEMV_F32_ROWS = 16          # most rows the 32-bit matrix-vector kernel takes
-
-
 def gemv_f32_ok(a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, out: torch.Tensor) -> bool:
     M, K = a.shape
     lda = a.stride(0) if M > 1 else max(K, a.stride(0))
     return (a.dtype == torch.float32 and w.dtype == torch.float32 and out.dtype == torch.float32
-            and (bias is None or bias.dtype == torch.float32) and 0 < M <= GEMV_F32_ROWS and K % 4 == 0
+            and (bias is None or bias.dtype == torch.float32) and 0 < M <= rule("gemv_f32_rows") and K % 4 == 0
             and lda % 4 == 0 and a.stride(1) == 1 and out.stride(1) == 1 and a.data_ptr() % 16 == 0
             and w.data_ptr() % 16 == 0)
 
@@ -413,6 +428,62 @@ def pack_weight(w: torch.Tensor, rows: int, parts: list[int] | None = None) -> P
     return PackedWeight(data, N, K, rows, tuple(parts))
 
 
+def linear_desc(w: torch.Tensor, packed: "PackedWeight | None", bias: torch.Tensor | None, library_first: bool = False):
+    """A matrix as the library's product rule takes it (a ``TmLinear``; the caller keeps the tensors alive)."""
+    from tokenmill_amd.hip.abi import TmLinear
+    _gpu(w, bias)
+    _need(w.dim() == 2 and w.is_contiguous(), "linear: the matrix must be contiguous [N, K]")
+    if bias is not None:
+        _need(tuple(bias.shape) == (w.shape[0],) and bias.is_contiguous(), "linear: bias must be [N]")
+    if packed is not None:
+        _packed_operand(packed, None, "linear")
+        _need((packed.n, packed.k) == tuple(w.shape), "linear: the packed copy is of another matrix")
+    return TmLinear(w.data_ptr(), packed.data.data_ptr() if packed is not None else None,
+                    bias.data_ptr() if bias is not None else None, packed.rows if packed is not None else 0,
+                    len(packed.parts) if packed is not None else 0, code(bias.dtype) if bias is not None else -1,
+                    w.shape[0], w.shape[1], code(w.dtype), 1 if library_first else 0)
+
+
+def _linear_input(desc, x: torch.Tensor) -> int:
+    _gpu(x)
+    _need(x.dim() == 2 and x.shape[1] == desc.K and x.stride(1) == 1, f"linear: x must be [M, {desc.K}] with unit inner stride")
+    _need(code(x.dtype) == desc.dtype, "linear: x must have the matrix's type (widen it for a 32-bit matrix)")
+    return x.stride(0) if x.shape[0] > 1 else max(desc.K, x.stride(0))
+
+
+def linear_accumulates(desc, x: torch.Tensor) -> bool:
+    """Is there a kernel that adds round(x W^T + b) into a 32-bit tensor in its own epilogue, for these operands?"""
+    from tokenmill_amd.hip.abi import bound
+    ldx = _linear_input(desc, x)
+    return bool(bound().tm_linear_accumulates(ctypes.byref(desc), code(x.dtype), _p(x), ldx, x.shape[0]))
+
+
+def linear(desc, x: torch.Tensor, out: torch.Tensor | None, accum: torch.Tensor | None = None,
+           tune: tuple[int, int, bool] | None = None) -> torch.Tensor:
+    """out[M, N] = x[M, K] W^T (+ bias) by the kernel the library's product rule chooses for the row count and
+    types (``desc``: ``linear_desc``). With ``accum`` (float32 [M, N]; only where ``linear_accumulates``) the
+    result, rounded to the matrix's type, is added there instead and ``out`` stays unwritten."""
+    from tokenmill_amd.hip.abi import bound
+    ldx = _linear_input(desc, x)
+    M = x.shape[0]
+    ws = library_workspace(x.device)
+    if accum is not None:
+        _gpu(accum)
+        _need(accum.dtype == torch.float32 and tuple(accum.shape) == (M, desc.N) and accum.stride(1) == 1,
+              f"linear: accum must be float32 [{M}, {desc.N}]")
+        ldacc = accum.stride(0) if M > 1 else max(desc.N, accum.stride(0))
+        _check(bound().tm_linear_run(ctypes.byref(desc), code(x.dtype), _p(x), ldx, M, None, 0, 0, _p(accum), ldacc, _p(ws),
+                                     LIBRARY_WORKSPACE_BYTES, _tune_arg(tune), _stream()), "linear")
+        return accum
+    _gpu(out)
+    _need(out is not None and tuple(out.shape) == (M, desc.N) and out.stride(1) == 1, f"linear: out must be [{M}, {desc.N}]")
+    _need(not (x.dtype == torch.float32 and out.dtype != torch.float32), "linear: float32 inputs give float32 outputs")
+    ldc = out.stride(0) if M > 1 else max(desc.N, out.stride(0))
+    _check(bound().tm_linear_run(ctypes.byref(desc), code(x.dtype), _p(x), ldx, M, _p(out), ldc, code(out.dtype), None, 0,
+                                 _p(ws), LIBRARY_WORKSPACE_BYTES, _tune_arg(tune), _stream()), "linear")
+    return out
+
+
 def skinny_strip_rows(N: int, K: int) -> int:
     """Rows of a strip the skinny product wants an [N, K] matrix packed in."""
     return int(library().tm_skinny_strip_rows(c_int(N), c_int(K)))
@@ -484,8 +555,8 @@ def _gemm_skinny_packed(a, w: PackedWeight, bias, out, silu: bool, accum) -> tor
     _packed_operand(w, 16 if silu else None, "gemm_skinny")
     M, K = a.shape
     N = w.n // 2 if silu else w.n
-    _need(a.dtype == torch.bfloat16 and a.dim() == 2 and a.stride(1) == 1 and 0 < M <= PACKED_ROWS and K == w.k,
-          f"gemm_skinny: bfloat16 a [M<={PACKED_ROWS}, {w.k}] for a packed matrix")
+    _need(a.dtype == torch.bfloat16 and a.dim() == 2 and a.stride(1) == 1 and 0 < M <= rule("skinny_rows") and K == w.k,
+          f"gemm_skinny: bfloat16 a [M<={rule('skinny_rows')}, {w.k}] for a packed matrix")
     _need(w.parts == ((N, N) if silu else (w.n,)), "gemm_skinny: with silu the matrix is packed as its two halves, else as one part")
     lda = a.stride(0) if M > 1 else max(K, a.stride(0))
     _need(K % 8 == 0 and lda % 8 == 0 and a.data_ptr() % 16 == 0,
@@ -510,12 +581,6 @@ def _gemm_skinny_packed(a, w: PackedWeight, bias, out, silu: bool, accum) -> tor
     return accum if accum is not None else out
 
 
-PACKED_ROWS = 16            # most rows of activations the products over packed matrices take
-
-DECODE_CHUNK = 256          # keys per block of the split decode attention
-DECODE_SPLIT_PAIRS = 192    # below this many (request, kv head) pairs the split kernels (with scratch memory) run
-
-
 def attn_decode_mfma_supported(dtype, H: int, KVH: int, D: int, page: int) -> bool:
     return (dtype == torch.bfloat16 and D in (32, 64, 96, 128) and page >= 16 and page & (page - 1) == 0
             and H % KVH == 0 and H // KVH <= 16)
@@ -523,10 +588,13 @@ def attn_decode_mfma_supported(dtype, H: int, KVH: int, D: int, page: int) -> bo
 
 def attn_decode_mfma(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                      block_tables: torch.Tensor, context_lens: torch.Tensor, H: int, KVH: int, D: int, scale: float,
-                     window: int, max_context: int, workspace: tuple[torch.Tensor, torch.Tensor] | None = None):
+                     window: int, max_context: int, workspace: tuple[torch.Tensor, torch.Tensor] | None = None,
+                     split: bool | None = None):
     """Attention of one new token per request over its cache (the token's own key included).
     q: [S, >= H*D] rows (unit inner stride), out [S, H*D] view; block_tables int32 [S, W];
-    context_lens int32 [S] (new token counted); max_context >= every context length."""
+    context_lens int32 [S] (new token counted); max_context >= every context length. ``split``: None runs
+    the kernel the library's rule names for this many requests (contexts split over blocks and merged, or one
+    block a request and kv head); True / False name it (each kernel alone, in tests)."""
     _gpu(q, out, k_pool, v_pool, block_tables, context_lens)
     S = q.shape[0]
     page = _check_pools(k_pool, v_pool, KVH, D, torch.bfloat16, "attn_decode")
@@ -542,9 +610,12 @@ def attn_decode_mfma(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v
     _need(block_tables.stride(0) == W or S == 1, "attn_decode: block_tables rows must be contiguous")
     _ints(context_lens, S, "context_lens")
     _need(0 < max_context <= W * page, "attn_decode: max_context exceeds what the block tables hold")
-    chunks = -(-max_context // DECODE_CHUNK)
+    from tokenmill_amd.hip.abi import bound
+    chunks = -(-max_context // rule("decode_chunk"))
     part_o = part_ml = None
-    if S * KVH < DECODE_SPLIT_PAIRS and chunks > 1:
+    if split is None:                                             # few (request, kv head) pairs: contexts split over blocks
+        split = bool(bound().tm_decode_split_chunks(S, KVH, max_context))
+    if split and chunks > 1:
         if workspace is None:
             workspace = (torch.empty((S, H, chunks, D), dtype=torch.float32, device=q.device),
                          torch.empty((S, H, chunks, 2), dtype=torch.float32, device=q.device))
@@ -625,9 +696,6 @@ def attn_prefill_f32(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v
     return out
 
 
-FUSED_DECODE_ROWS = 16      # most tokens the norm-fused decode products take
-
-
 def fused_norm_qkv_rope(resid: torch.Tensor, norm_w: torch.Tensor, eps: float, w: PackedWeight,
                         bias: torch.Tensor | None, q_out: torch.Tensor, H: int, KVH: int, D: int, cos: torch.Tensor,
                         sin: torch.Tensor, positions: torch.Tensor, slots: torch.Tensor | None,
@@ -637,7 +705,7 @@ def fused_norm_qkv_rope(resid: torch.Tensor, norm_w: torch.Tensor, eps: float, w
     ``fused_qkv_strip_rows(H, KVH, D, K)`` rows; cos/sin float32 [max_pos, D/2]."""
     _gpu(resid, norm_w, bias, q_out, cos, sin, positions, slots, k_pool, v_pool)
     M, K = resid.shape
-    _need(0 < M <= FUSED_DECODE_ROWS, f"fused qkv: at most {FUSED_DECODE_ROWS} tokens, got {M}")
+    _need(0 < M <= rule("skinny_rows"), f"fused qkv: at most {rule('skinny_rows')} tokens, got {M}")
     _need(resid.dtype == torch.float32 and resid.is_contiguous() and resid.data_ptr() % 16 == 0, "fused qkv: resid float32 [M, K]")
     _need(D % 32 == 0, f"fused qkv: head size {D} must be a multiple of 32")
     _packed_operand(w, fused_qkv_strip_rows(H, KVH, D, K), "fused qkv")
@@ -675,7 +743,7 @@ def fused_norm_gate_up_silu(resid: torch.Tensor, norm_w: torch.Tensor, eps: floa
     _gpu(resid, norm_w, out)
     M, K = resid.shape
     I = out.shape[1]
-    _need(0 < M <= FUSED_DECODE_ROWS, f"fused gate-up: at most {FUSED_DECODE_ROWS} tokens, got {M}")
+    _need(0 < M <= rule("skinny_rows"), f"fused gate-up: at most {rule('skinny_rows')} tokens, got {M}")
     _need(resid.dtype == torch.float32 and resid.is_contiguous() and resid.data_ptr() % 16 == 0, "fused gate-up: resid float32 [M, K]")
     _packed_operand(w, 16, "fused gate-up")
     _need((w.n, w.k) == (2 * I, K) and w.parts == (I, I) and K % 8 == 0 and I % 4 == 0,
@@ -689,9 +757,6 @@ def fused_norm_gate_up_silu(resid: torch.Tensor, norm_w: torch.Tensor, eps: floa
     return out
 
 
-PANEL_ROWS = 64             # most tokens the products that keep the normed input in LDS take
-
-
 def panel_fits(M: int, K: int) -> bool:
     """Do the panel products (q|k|v + rotary + cache write, gate|up + SiLU·up for up to 64 tokens behind a
     norm that ran by itself) take M tokens of width K?"""
@@ -700,8 +765,8 @@ def panel_fits(M: int, K: int) -> bool:
 
 def _panel_input(x: torch.Tensor, who: str) -> int:
     M, K = x.shape
-    _need(x.dtype == torch.bfloat16 and x.stride(1) == 1 and x.data_ptr() % 16 == 0 and 0 < M <= PANEL_ROWS
-          and panel_fits(M, K), f"{who}: x bfloat16 [M<={PANEL_ROWS}, K] with x and the partial sums fitting a block's LDS")
+    _need(x.dtype == torch.bfloat16 and x.stride(1) == 1 and x.data_ptr() % 16 == 0 and M > 0
+          and panel_fits(M, K), f"{who}: x bfloat16 [M, K] with x and the partial sums fitting a block's LDS")
     ldx = x.stride(0) if M > 1 else max(K, x.stride(0))
     _need(ldx % 8 == 0, f"{who}: rows of x must be 16-byte aligned")
     return ldx

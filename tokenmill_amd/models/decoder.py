@@ -74,14 +74,27 @@ class DecoderModel:
 
     # --- one step -----------------------------------------------------------------------------------
 
-    def forward(self, step: StepContext, caches: list) -> torch.Tensor:
-        """Runs the step's tokens through the layers; returns float32 logits [R, vocab] at
-        ``step.logit_rows``. ``caches[j]`` is the cache view of run call j (shared ones resolved)."""
-        resid = self.embedding.forward(step.token_ids)                     # float32 [T, hidden]
-        delta = None
+    def program(self, caches: list, tune: tuple[int, bool] | None = None):
+        """The model's step as a ``StepProgram``: every part describes its operation to it, in the order of the
+        run list; ``caches[j]`` is the cache view of run call j (shared ones resolved). Running the program on
+        a step gives the float32 logits [R, vocab] at ``step.logit_rows``. A part the kernel library has no
+        operation for is called through its own ``forward`` at its place. ``tune``: (candidates, every) if the
+        library's matrix products are to be timed for this model's steps."""
+        from tokenmill_amd.hip.program import StepProgram
+        program = StepProgram(self.dtype, self.embedding.hidden, self.device, tune)
+        emb, head, norm = self.embedding, self.head, self.final_norm
+        if getattr(emb, "emit", lambda p: None)(program) is None:
+            def embed(flow, step):
+                flow.resid, flow.delta = emb.forward(step.token_ids), None
+            program.foreign(emb, embed)
         for j, call in enumerate(self.run):
-            delta = self.layers[call.layer].forward(resid, delta, step, caches[j], self.dtype)
-        if step.num_logit_rows == 0:
-            return torch.empty((0, self.head.vocab), dtype=torch.float32, device=resid.device)
-        h = self.final_norm.add_norm(resid, delta, self.dtype, rows=step.logit_rows)
-        return self.head.forward(h)
+            self.layers[call.layer].emit(program, caches[j])
+        if getattr(head, "emit", lambda p, n: None)(program, norm) is None:
+            def logits(flow, step):
+                if step.num_logit_rows == 0:
+                    flow.logits = torch.empty((0, head.vocab), dtype=torch.float32, device=flow.resid.device)
+                else:
+                    flow.logits = head.forward(norm.add_norm(flow.resid, flow.delta, self.dtype, rows=step.logit_rows))
+                flow.delta = None
+            program.foreign(head, logits)
+        return program

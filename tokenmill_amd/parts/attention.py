@@ -1,19 +1,20 @@
 """Grouped-query attention over the paged cache (reference src/infer/model/layers.py:127-150,
 src/infer/kv/context.py:63-80).
 
-One fused q|k|v projection, position encoding and cache write in one kernel, then attention of
-every token of the step over its own request's cache, then the output projection. Portions of
-prompts and single decoded tokens go through the same call; the kernels read keys and values in
-place through the block tables.
+One fused q|k|v projection, position encoding and cache write, then attention of every token of the
+step over its own request's cache, then the output projection. Portions of prompts and single decoded
+tokens go through the same call; the kernels read keys and values in place through the block tables.
+The part describes all of that to the kernel library as one operation (``emit``); which kernels run
+for a step is decided there.
 """
 from __future__ import annotations
 
 import torch
 
 from tokenmill_amd import profiling
-from tokenmill_amd.hip import attention as attn_kernels
-from tokenmill_amd.hip import gemm, ops
-from tokenmill_amd.parts.base import (KVCacheSpec, KVCacheView, Mixer, NormedInput, PositionEncoding, StepContext,
+from tokenmill_amd.hip import ops
+from tokenmill_amd.hip.program import StepProgram
+from tokenmill_amd.parts.base import (KVCacheSpec, KVCacheView, Mixer, Norm, NormedInput, PositionEncoding, StepContext,
                                       as_tensor)
 from tokenmill_amd.parts.linear import Linear
 
@@ -39,6 +40,7 @@ class GQAttention(Mixer):
         self.q_size, self.kv_size = q, kv
         self.qkv = Linear(hidden, [q, kv, kv], list(names[:3]), bias=qkv_bias)
         self.o = Linear(q, hidden, names[3], bias=o_bias)
+        self._own: dict = {}                    # one-operation programs for calls of ``forward``
 
     def tensor_specs(self, prefix: str):
         return {**self.qkv.tensor_specs(prefix), **self.o.tensor_specs(prefix), **self.position.tensor_specs(prefix)}
@@ -58,66 +60,61 @@ class GQAttention(Mixer):
     def cache_spec(self):
         return KVCacheSpec(self.num_kv_heads, self.head_dim, self.window)
 
-    def _fused_qkv(self, x, step: StepContext, cache: KVCacheView) -> torch.Tensor | None:
-        """q [T, H*D] with k and v already in the cache, by the kernel that starts at the norm; None if
-        that kernel does not take this step."""
-        if not isinstance(x, NormedInput) or x.dtype != torch.bfloat16 or self.head_dim % 32:
-            return None
-        rms = x.fusable_rms()
-        tables = getattr(self.position, "fusable_tables", lambda: None)()
-        page = cache.k.shape[1]
-        bias = self.qkv.bias
-        if (rms is None or tables is None or not gemm.fused_decode_ok(x.resid, self.qkv.packed) or page & (page - 1)
-                or step.max_context_len > self.position.max_positions
-                or (bias is not None and bias.data_ptr() % 16)):
-            return None
-        q = torch.empty((x.num_tokens, self.q_size), dtype=torch.bfloat16, device=x.resid.device)
-        write = cache.write
-        ops.fused_norm_qkv_rope(x.resid, rms[0], rms[1], self.qkv.packed, self.qkv.bias, q, self.num_heads,
-                                self.num_kv_heads, self.head_dim, tables[0], tables[1], step.positions,
-                                step.groups[cache.group].slot_mapping if write else None,
-                                cache.k if write else None, cache.v if write else None)
-        return q
+    # --- the operation ------------------------------------------------------------------------------------
 
-    def _panel_qkv(self, x: torch.Tensor, step: StepContext, cache: KVCacheView) -> torch.Tensor | None:
-        """The same for 17 to 64 tokens, from the normed input; None if that kernel does not take this step."""
-        tables = getattr(self.position, "fusable_tables", lambda: None)()
-        page = cache.k.shape[1]
-        bias = self.qkv.bias
-        if (tables is None or self.head_dim % 32 or not gemm.panel_ok(x, self.qkv.packed) or page & (page - 1)
-                or step.max_context_len > self.position.max_positions
-                or (bias is not None and bias.data_ptr() % 16)):
+    def emit(self, program, norm: Norm | None, cache, encoded_outside: bool = False) -> int | None:
+        """``encoded_outside``: the operation will only ever be handed q|k|v that are already encoded and stored
+        (the way a position encoding the library does not know is run)."""
+        rotation = () if encoded_outside else self.position.rotation()
+        if rotation is None or not isinstance(cache, KVCacheView):
             return None
-        q = torch.empty((x.shape[0], self.q_size), dtype=torch.bfloat16, device=x.device)
-        write = cache.write
-        ops.panel_qkv_rope(x, self.qkv.packed, bias, q, self.num_heads, self.num_kv_heads, self.head_dim, tables[0],
-                           tables[1], step.positions, step.groups[cache.group].slot_mapping if write else None,
-                           cache.k if write else None, cache.v if write else None)
-        return q
+        return program.attention(self, norm, self.qkv, self.o, rotation, cache, self.num_heads, self.num_kv_heads,
+                                 self.head_dim, self.scale, self.window)
 
-    def _attention_cost(self, step: StepContext, elem: int) -> tuple[int, int]:
-        """Every key and value of the step's requests read once, q read and the output written; two
-        products of 2 * head_dim flops per (query, visible key, head)."""
+    def cost(self, label: str, step: StepContext | None, rows: int) -> tuple[int, int]:
+        if label == "qkv":
+            return self.qkv.cost(rows)                  # with norm, rotary and cache write where fused
+        if label == "o_proj":
+            return self.o.cost(rows)
+        # attention: every key and value of the step's requests read once, q read and the output written; two
+        # products of 2 * head_dim flops per (query, visible key, head)
+        elem = self.qkv.weight.element_size()
         keys_read = pairs = 0
         for start, n in zip(step.start_positions, step.q_lens):
             keys_read += min(start + n, self.window + n - 1) if self.window else start + n
-            for i in range(n):
-                pairs += min(start + i + 1, self.window) if self.window else start + i + 1
+            if self.window:
+                pairs += sum(min(start + i + 1, self.window) for i in range(n))
+            else:
+                pairs += n * start + n * (n + 1) // 2
         moved = 2 * keys_read * self.kv_size * elem + 2 * step.num_tokens * self.q_size * elem
         return moved, 4 * pairs * self.num_heads * self.head_dim
 
+    def _alone(self, norm: Norm | None, cache: KVCacheView, dtype, encoded_outside: bool = False):
+        """This mixer's operation as a program of its own, for calls of ``forward``."""
+        key = (id(norm), id(cache.k), cache.write, dtype, encoded_outside)
+        entry = self._own.get(key)
+        if entry is None:
+            program = StepProgram(dtype, self.hidden, cache.k.device)
+            op = self.emit(program, norm, cache, encoded_outside)
+            if op is None:
+                raise ops.KernelArgumentError("the kernel library has no attention operation for these tensors")
+            entry = self._own[key] = (program, op, norm, cache)
+        return entry[0], entry[1]
+
     def forward(self, x, step: StepContext, cache: KVCacheView, residual: torch.Tensor | None = None):
-        with profiling.label("qkv", lambda: self.qkv.cost(step.num_tokens)):       # with norm, rotary and cache write where fused
-            q = self._fused_qkv(x, step, cache)
-            if q is None:
-                x = as_tensor(x)
-                q = self._panel_qkv(x, step, cache)
-            if q is None:
-                q = self.qkv.forward(x)                                    # [T, (H + 2 KVH) D], q first
-                self.position.encode_and_store(q, self.num_heads, self.num_kv_heads, self.head_dim, step, cache)
-        out = torch.empty((q.shape[0], self.q_size), dtype=q.dtype, device=q.device)
-        with profiling.label("attention", lambda: self._attention_cost(step, q.element_size())):
-            attn_kernels.paged_attention(q, out, cache, step, self.num_heads, self.num_kv_heads, self.head_dim,
-                                         self.scale, self.window or 0)
-        with profiling.label("o_proj", lambda: self.o.cost(step.num_tokens)):
-            return self.o.forward(out, accumulate_into=residual)
+        """The same operation called by itself: by a block that is not described to a step program, or a test."""
+        if self.position.rotation() is None:
+            # an encoding the library does not know: project, let it encode and store, attend from there
+            x = as_tensor(x)
+            with profiling.label("qkv", lambda: self.qkv.cost(x.shape[0])):
+                qkv = self.qkv.forward(x)
+                self.position.encode_and_store(qkv, self.num_heads, self.num_kv_heads, self.head_dim, step, cache)
+            program, op = self._alone(None, cache, x.dtype, encoded_outside=True)
+            return program.run_one(op, step, resid=residual, qkv=qkv, accumulate=residual is not None)
+        if isinstance(x, NormedInput) and x.lazy:
+            program, op = self._alone(x.norm, cache, x.dtype)
+            resid, delta = x.take()
+            return program.run_one(op, step, resid=resid, delta=delta, accumulate=residual is resid)
+        x = as_tensor(x)
+        program, op = self._alone(None, cache, x.dtype)
+        return program.run_one(op, step, resid=residual, x=x.contiguous(), accumulate=residual is not None)

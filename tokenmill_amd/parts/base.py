@@ -103,6 +103,12 @@ class Part:
         """Called once after ``load``: make what the kernels want beside the checkpoint's tensors.
         ``pack_weights``: whether second copies of matrices in a kernel's own order may be kept."""
 
+    def cost(self, label: str, step: "StepContext | None", rows: int) -> tuple[int, int]:
+        """(bytes, flops) that the span ``label`` of this part's operation has to move and do for a step of
+        ``rows`` tokens: what a profile prices the span's measured time against. Only parts that describe an
+        operation to the step program are asked."""
+        return 0, 0
+
 
 class Norm(Part):
     def add_norm(self, resid: torch.Tensor, delta: torch.Tensor | None, out_dtype: torch.dtype,
@@ -127,6 +133,7 @@ class NormedInput:
     def __init__(self, norm: Norm, resid: torch.Tensor, delta: torch.Tensor | None, dtype: torch.dtype):
         self.norm, self.resid, self.delta, self.dtype = norm, resid, delta, dtype
         self._tensor: torch.Tensor | None = None
+        self.taken = False                   # a kernel that starts at the norm has taken resid and delta as they are
 
     @property
     def num_tokens(self) -> int:
@@ -144,6 +151,17 @@ class NormedInput:
             return None
         return self.norm.rms_params()
 
+    @property
+    def lazy(self) -> bool:
+        """Still to be computed, by a norm the kernel library computes itself?"""
+        return self._tensor is None and not self.taken and self.norm.rms_params() is not None
+
+    def take(self) -> tuple[torch.Tensor, torch.Tensor | None]:
+        """(resid, delta) for an operation that adds and norms by itself; after this the input counts as computed."""
+        self.taken = True
+        delta, self.delta = self.delta, None
+        return self.resid, delta
+
 
 def as_tensor(x) -> torch.Tensor:
     """The input of a part as a tensor, whether it came lazily or not."""
@@ -151,6 +169,12 @@ def as_tensor(x) -> torch.Tensor:
 
 
 class PositionEncoding(Part):
+    def rotation(self):
+        """What the kernel library's attention operation needs to apply this encoding itself: (cos, sin, rotary
+        width, positions) for a rotation of pairs, () for no encoding at all, None (the default) for an encoding
+        the library does not know: the mixer then projects q|k|v, calls ``encode_and_store`` and goes on from there."""
+        return None
+
     def encode_and_store(self, qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
                          step: StepContext, cache: KVCacheView) -> None:
         """Encode positions into q and k of ``qkv`` in place and store k, v into the cache."""
@@ -158,6 +182,12 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
+    def emit(self, program, norm: Norm, cache) -> int | None:
+        """Describes ``resid += self(norm(resid))`` over ``cache`` to the step program (``hip/program.py``) and
+        returns the operation's index; None (the default) if the kernel library has no operation for this
+        mixer: the program then calls ``forward``."""
+        return None
+
     # Can a step of single tokens through this mixer be recorded into a HIP graph? Yes if ``forward`` works on
     # the step's device tensors alone for such a step (index operations with ``state_slots``, kernels);
     # no if it needs their values on the host (``.tolist()``, ``.item()``) or allocates by them. Only asked
@@ -175,6 +205,28 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
+    def emit(self, program, norm: Norm) -> int | None:
+        """As ``Mixer.emit``, for ``resid += self(norm(resid))``."""
+        return None
+
     def forward(self, x, step: StepContext, residual: torch.Tensor | None = None) -> torch.Tensor | None:
         """Same contract as ``Mixer.forward``, without a cache."""
         raise NotImplementedError
+
+
+class Block(Part):
+    """An arrangement of parts in a layer. ``forward(resid, delta, step, cache, dtype)`` updates the 32-bit
+    residual stream ``resid`` in place, given the not-yet-added result ``delta`` of the block before, and
+    returns its own not-yet-added result (or None). ``emit`` describes the block to a step program; by
+    default as one call of ``forward``, so a block written elsewhere needs nothing more."""
+
+    mixer: Mixer
+
+    def forward(self, resid: torch.Tensor, delta: torch.Tensor | None, step: StepContext, cache,
+                dtype: torch.dtype) -> torch.Tensor | None:
+        raise NotImplementedError
+
+    def emit(self, program, cache) -> None:
+        def run(flow, step):
+            flow.delta = self.forward(flow.resid, flow.delta, step, cache, program.dtype)
+        program.foreign(self, run)

@@ -9,10 +9,10 @@ from __future__ import annotations
 
 import torch
 
-from tokenmill_amd.parts.base import FeedForward, Mixer, Norm, NormedInput, Part, StepContext
+from tokenmill_amd.parts.base import Block, FeedForward, Mixer, Norm, NormedInput, StepContext
 
 
-class PreNormBlock(Part):
+class PreNormBlock(Block):
     def __init__(self, norm_in: Norm, mixer: Mixer, norm_post: Norm, ffn: FeedForward,
                  names: tuple[str, str, str, str] = ("input_layernorm.", "self_attn.",
                                                      "post_attention_layernorm.", "mlp.")):
@@ -35,6 +35,22 @@ class PreNormBlock(Part):
     def prepare(self, pack_weights: bool) -> None:
         for part, _ in self._parts():
             part.prepare(pack_weights)
+
+    def emit(self, program, cache) -> None:
+        """The block as two operations of a step program; a mixer or feed-forward the kernel library has no
+        operation for runs through its own ``forward`` between the library's operations."""
+        if self.mixer.emit(program, self.norm_in, cache) is None:
+            def mix(flow, step):
+                x = NormedInput(self.norm_in, flow.resid, flow.delta, program.dtype)
+                flow.delta = self.mixer.forward(x, step, cache, residual=flow.resid)
+                assert x.delta is None, f"{type(self.mixer).__name__}.forward did not take its input"
+            program.foreign(self.mixer, mix)
+        if self.ffn.emit(program, self.norm_post) is None:
+            def feed(flow, step):
+                x = NormedInput(self.norm_post, flow.resid, flow.delta, program.dtype)
+                flow.delta = self.ffn.forward(x, step, residual=flow.resid)
+                assert x.delta is None, f"{type(self.ffn).__name__}.forward did not take its input"
+            program.foreign(self.ffn, feed)
 
     def forward(self, resid: torch.Tensor, delta: torch.Tensor | None, step: StepContext, cache,
                 dtype: torch.dtype) -> torch.Tensor:

@@ -23,9 +23,15 @@ class TokenEmbedding(Part):
     def load(self, tensors, prefix: str) -> None:
         self.weight = tensors[f"{prefix}{self.name}"]
 
+    def emit(self, program) -> int | None:
+        return program.embedding(self, self.weight)
+
+    def cost(self, label, step, rows):
+        return rows * self.hidden * (self.weight.element_size() + 4), 0
+
     def forward(self, token_ids: torch.Tensor) -> torch.Tensor:
         out = torch.empty((token_ids.numel(), self.hidden), dtype=torch.float32, device=token_ids.device)
-        with profiling.label("embed", lambda: (out.numel() * (self.weight.element_size() + 4), 0)):
+        with profiling.label("embed", lambda: self.cost("embed", None, token_ids.numel())):
             return ops.embed_gather(self.weight, token_ids, out)
 
 
@@ -44,6 +50,17 @@ class OutputHead(Part):
             self.proj.use_weight(self.tied_to.weight)
         else:
             self.proj.load(tensors, prefix)
+
+    def emit(self, program, norm) -> int | None:
+        """logits = proj(norm(resid[logit rows])): the final norm and this head as one operation."""
+        return program.head(self, norm, self.proj, self.vocab)
+
+    def cost(self, label, step, rows):
+        n = step.num_logit_rows if step is not None else rows
+        if label == "norm":
+            e = self.proj.weight.element_size()
+            return n * self.hidden * (4 + e), 0
+        return self.proj.cost(n, out_bytes=4)
 
     def forward(self, h: torch.Tensor) -> torch.Tensor:
         with profiling.label("head", lambda: self.proj.cost(h.shape[0], out_bytes=4)):

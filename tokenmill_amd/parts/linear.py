@@ -26,6 +26,7 @@ class Linear(Part):
         self.weight: torch.Tensor | None = None
         self.bias: torch.Tensor | None = None
         self.packed: ops.PackedWeight | None = None     # the matrix again in the order the decode kernels read
+        self._desc = None                               # the matrix as the library's product rule takes it
 
     def tensor_specs(self, prefix: str) -> dict[str, TensorSpec]:
         specs = {}
@@ -43,6 +44,7 @@ class Linear(Part):
             self.bias = bs[0] if len(bs) == 1 else torch.cat(bs, dim=0).contiguous()
             if self.weight.dtype == torch.float32 and self.bias.dtype != torch.float32:
                 self.bias = self.bias.float()          # a 32-bit product adds a 32-bit bias
+        self._desc = None
 
     def pack(self, rows, parts: list[int] | None = None) -> None:
         """Keep a second copy of a bfloat16 matrix in strip order (``ops.pack_weight``) for the products of
@@ -52,6 +54,15 @@ class Linear(Part):
         w = self.weight
         if w is not None and w.dtype == torch.bfloat16 and w.is_cuda:
             self.packed = ops.pack_weight(w, rows() if callable(rows) else rows, parts)
+            self._desc = None
+
+    def describe(self):
+        """The matrix, its packed copy and its bias as the kernel library takes them (kept until the tensors
+        change); None while there is nothing on a GPU to describe."""
+        if self._desc is None and self.weight is not None and self.weight.is_cuda and self.weight.is_contiguous() \
+                and self.weight.dtype in (torch.float32, torch.bfloat16):
+            self._desc = ops.linear_desc(self.weight, self.packed, self.bias, self.library_first)
+        return self._desc
 
     def cost(self, rows: int, in_bytes: int | None = None, out_bytes: int | None = None) -> tuple[int, int]:
         """(bytes, flops) the product has to move and do for ``rows`` rows: the matrix once, the input and
@@ -66,25 +77,26 @@ class Linear(Part):
     def use_weight(self, weight: torch.Tensor) -> None:
         """Share another part's matrix (a tied output head)."""
         self.weight = weight
+        self._desc = None
 
     def forward(self, x: torch.Tensor, out_dtype: torch.dtype | None = None,
                 accumulate_into: torch.Tensor | None = None) -> torch.Tensor | None:
         """x [M, in] (row-strided views allowed) -> [M, out] in ``out_dtype`` (default: x's type).
         With ``accumulate_into`` (float32 [M, out]) the result may be added there by the product's own
-        epilogue; then None is returned."""
+        epilogue; then None is returned. Which kernel runs is the library's choice (``ops.linear``)."""
         w = self.weight
         out_dtype = out_dtype or x.dtype
-        from tokenmill_amd.hip import gemm
-        if accumulate_into is not None and w.dtype == x.dtype and \
-                gemm.linear_accumulate(x, w, self.bias, accumulate_into, packed=self.packed):
+        desc = self.describe()
+        if accumulate_into is not None and w.dtype == x.dtype and ops.linear_accumulates(desc, x):
+            ops.linear(desc, x, None, accum=accumulate_into)
             return None
         if w.dtype != x.dtype:
             # a matrix the checkpoint stores in 32-bit stays 32-bit: widen the activations for it
             x = ops.convert(x.contiguous(), torch.empty(x.shape, dtype=w.dtype, device=x.device))
         inner_dtype = torch.float32 if x.dtype == torch.float32 else out_dtype
         out = torch.empty((x.shape[0], self.out_features), dtype=inner_dtype, device=x.device)
-        gemm.linear(x, w, self.bias, out, packed=self.packed if x.dtype == w.dtype else None,
-                    library_first=self.library_first)
+        if x.shape[0]:
+            ops.linear(desc, x, out)
         if out.dtype != out_dtype:
             out = ops.convert(out, torch.empty(out.shape, dtype=out_dtype, device=out.device))
         return out

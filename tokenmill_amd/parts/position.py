@@ -46,14 +46,16 @@ class RotaryEmbedding(PositionEncoding):
                           step.groups[cache.group].slot_mapping if write else None,
                           cache.k if write else None, cache.v if write else None)
 
-
-    def fusable_tables(self):
-        """(cos, sin) when the rotation covers the whole head (what the fused q|k|v kernel applies)."""
-        return (self.cos, self.sin) if self.rotary_dim == self.head_dim else None
+    def rotation(self):
+        """(cos, sin, rotary width, positions): what the kernel library's attention operation rotates by."""
+        return (self.cos, self.sin, self.rotary_dim, self.max_positions) if self.cos is not None else None
 
 
 class NoPositionEncoding(PositionEncoding):
     """Stores k and v; q and k stay as they are."""
+
+    def rotation(self):
+        return ()
 
     def encode_and_store(self, qkv, num_heads, num_kv_heads, head_dim, step: StepContext, cache: KVCacheView | None):
         if cache is not None and cache.write:
