@@ -981,6 +981,136 @@ def test_panel_gate_up_silu(ops, M, K, I):
     assert torch.equal(one[0], out[M - 1])
 
 
+@pytest.mark.parametrize("M,K,H,KVH,D,page,rows", [(64, 896, 14, 2, 64, 16, 8), (17, 192, 6, 1, 32, 16, 16), (40, 3584, 4, 4, 128, 32, 16),
+                                                    (33, 120, 3, 1, 96, 64, 4), (5, 1096, 14, 2, 64, 16, 8), (64, 5120, 5, 1, 128, 16, 16)])
+def test_stream_qkv_rope(ops, M, K, H, KVH, D, page, rows):
+    """q|k|v + bias + rotary + cache write for up to 64 tokens at any width (K no multiple of 32 or of the k-steps a
+    wavefront asks for at once; beyond what a block's LDS holds), the matrix streamed from its packed copy whatever
+    the height of its strips."""
+    torch.manual_seed(23)
+    dt = torch.bfloat16
+    theta, max_pos, pages = 1e6, 500, 12
+    n = (H + 2 * KVH) * D
+    x = q(torch.randn(M, K), dt)
+    W, b = q(torch.randn(n, K) * 0.05, dt), q(torch.randn(n) * 0.5, dt)
+    positions = torch.randint(0, max_pos, (M,), dtype=torch.int32)
+    slots = torch.randperm(pages * page)[:M].to(torch.int32)
+    slots[1] = -1
+    qkv = P.linear(x, W, b, dt)
+    cos, sin = P.rope_tables(max_pos, D, theta)
+    qq = P.apply_rope(qkv[:, :H * D].view(M, H, D), cos, sin, positions.long(), dt)
+    kk = P.apply_rope(qkv[:, H * D:(H + KVH) * D].view(M, KVH, D), cos, sin, positions.long(), dt)
+    vv = qkv[:, (H + KVH) * D:].view(M, KVH, D)
+    half = cos[:, :D // 2].contiguous().to(DEV), sin[:, :D // 2].contiguous().to(DEV)
+    kp = torch.full((pages, page, KVH, D), 7.0, dtype=dt, device=DEV)
+    vp = torch.full((pages, KVH, D, page), 7.0, dtype=dt, device=DEV)
+    q_out = torch.empty(M, H * D, dtype=dt, device=DEV)
+    assert ops.stream_fits(M, K) and not ops.stream_fits(65, K) and not ops.stream_fits(M, K + 4)
+    Wp = ops.pack_weight(W.to(dt).to(DEV), rows)
+    wide = torch.zeros(M, K + 16, dtype=dt, device=DEV)                 # a strided input
+    wide[:, :K] = x.to(dt).to(DEV)
+    ops.stream_qkv_rope(wide[:, :K], Wp, b.to(dt).to(DEV), q_out, H, KVH, D, half[0], half[1], positions.to(DEV),
+                        slots.to(DEV), kp, vp)
+    torch.testing.assert_close(q_out.float().cpu().view(M, H, D), qq, **tol(dt))
+    kflat = kp.float().cpu().view(-1, KVH, D)
+    vflat = vp.float().cpu().permute(0, 3, 1, 2).reshape(-1, KVH, D)
+    written = torch.zeros(pages * page, dtype=torch.bool)
+    for t in range(M):
+        if slots[t] >= 0:
+            written[slots[t]] = True
+            torch.testing.assert_close(kflat[slots[t]], kk[t], **tol(dt))
+            torch.testing.assert_close(vflat[slots[t]], vv[t], **tol(dt))
+    assert (kflat[~written] == 7.0).all() and (vflat[~written] == 7.0).all()
+    # a token's result does not depend on the other tokens of the call, nor on the strips' height; a 32-bit bias
+    q_all = torch.empty(M, H * D, dtype=dt, device=DEV)
+    ops.stream_qkv_rope(wide[:, :K], Wp, b.to(DEV), q_all, H, KVH, D, half[0], half[1], positions.to(DEV), None, None, None)
+    assert torch.equal(q_all, q_out)
+    q_one = torch.empty(1, H * D, dtype=dt, device=DEV)
+    ops.stream_qkv_rope(wide[M - 1:, :K], ops.pack_weight(W.to(dt).to(DEV), 16), b.to(dt).to(DEV), q_one, H, KVH, D, half[0],
+                        half[1], positions[M - 1:].to(DEV), None, None, None)
+    assert torch.equal(q_one[0], q_all[M - 1])
+
+
+@pytest.mark.parametrize("M,K,I", [(64, 896, 4864), (17, 64, 128), (48, 3584, 1000), (33, 120, 200), (9, 1048, 100)])
+def test_stream_gate_up_silu(ops, M, K, I):
+    torch.manual_seed(24)
+    dt = torch.bfloat16
+    x, W = q(torch.randn(M, K), dt), q(torch.randn(2 * I, K) * (0.1 if K < 2000 else 0.03), dt)
+    gu = P.linear(x, W, None, dt)
+    want = P.silu_mul(gu[:, :I], gu[:, I:], dt)
+    out = torch.full((M, I), 7.0, dtype=dt, device=DEV)
+    Wp = ops.pack_weight(W.to(dt).to(DEV), 16, [I, I])
+    xd = x.to(dt).to(DEV)
+    ops.stream_gate_up_silu(xd, Wp, out)
+    torch.testing.assert_close(out.float().cpu(), want, rtol=2e-2, atol=2e-2)
+    assert ((out.float().cpu() - want).abs() > 1e-2).float().mean() < 0.01      # a rounding flip of gate or up now and then
+    one = torch.empty(1, I, dtype=dt, device=DEV)
+    ops.stream_gate_up_silu(xd[M - 1:], Wp, one)
+    assert torch.equal(one[0], out[M - 1])
+
+
+@pytest.mark.parametrize("M,N,K,rows", [(64, 896, 4864, 4), (17, 64, 128, 16), (40, 200, 120, 8), (64, 3584, 18944, 16),
+                                        (33, 1001, 1096, 16), (48, 50, 72, 4)])
+def test_stream_linear_stores_or_adds_into_the_residual(ops, M, N, K, rows):
+    """The plain product of 17 to 64 rows over a packed matrix: bfloat16 and float32 out, with and without bias, and
+    the rounded result added into a 32-bit tensor; N no multiple of 32, of 16 or of 4."""
+    torch.manual_seed(25)
+    dt = torch.bfloat16
+    a, w, b = q(torch.randn(M, K), dt), q(torch.randn(N, K) * (0.1 if K < 2000 else 0.02), dt), q(torch.randn(N), dt)
+    want = a @ w.t()
+    da, db = a.to(dt).to(DEV), b.to(dt).to(DEV)
+    Wp = ops.pack_weight(w.to(dt).to(DEV), rows)
+    out = torch.full((M, N), 7.0, dtype=dt, device=DEV)
+    ops.stream_linear(da, Wp, db, out)
+    torch.testing.assert_close(out.float().cpu(), q(want + b, dt), **tol(dt))
+    out32 = torch.full((M, N), 7.0, dtype=torch.float32, device=DEV)
+    ops.stream_linear(da, Wp, None, out32)
+    torch.testing.assert_close(out32.cpu(), want, rtol=1e-4, atol=1e-4 * K ** 0.5)
+    resid = torch.randn(M, N) * 5
+    acc = resid.to(DEV)
+    ops.stream_linear(da, Wp, db, None, accum=acc)
+    assert torch.equal(acc.cpu(), resid + out.float().cpu())            # the rounded product, added in 32-bit
+    one = torch.empty(1, N, dtype=dt, device=DEV)                       # a row does not depend on its batch-mates
+    ops.stream_linear(da[M - 1:], Wp, db, one)
+    assert torch.equal(one[0], out[M - 1])
+    other = torch.empty(M, N, dtype=dt, device=DEV)                     # ... nor on the height of the packed strips
+    ops.stream_linear(da, ops.pack_weight(w.to(dt).to(DEV), 16 if rows != 16 else 8), db, other)
+    assert torch.equal(other, out)
+
+
+@pytest.mark.parametrize("M,N,K,rows", [(64, 896, 4864, 4), (33, 3584, 18944, 16), (20, 200, 120, 8), (48, 1001, 9000, 16)])
+def test_stream_linear_with_k_split_over_blocks_and_the_norm_that_adds_the_parts(ops, M, N, K, rows):
+    """A plain product with few rows of output and a long K splits K over groups of blocks, which leave 32-bit partial
+    sums; the norm that follows adds them up in their order, rounds the sum as the product's own epilogue would have,
+    and goes on as if it had been handed that tensor: the same bits as the two steps one after the other."""
+    torch.manual_seed(26)
+    dt = torch.bfloat16
+    a, w, b = q(torch.randn(M, K), dt), q(torch.randn(N, K) * (0.1 if K < 2000 else 0.02), dt), q(torch.randn(N), dt)
+    want = a @ w.t() + b
+    da, db = a.to(dt).to(DEV), b.to(dt).to(DEV)
+    Wp = ops.pack_weight(w.to(dt).to(DEV), rows)
+    parts = ops.stream_linear_split(da, Wp, db)
+    n_parts = parts.shape[0]
+    assert (n_parts >= 2 if K >= 4000 else n_parts == 1) and tuple(parts.shape[1:]) == (M, N)
+    delta = ops.sum_parts(parts, torch.empty(M, N, dtype=dt, device=DEV))
+    torch.testing.assert_close(delta.float().cpu(), q(want, dt), **tol(dt))
+    assert torch.equal(delta.float().cpu(), q(parts.sum(0).cpu(), dt)) or n_parts > 2   # (two parts: one order only)
+    one = ops.stream_linear_split(da[M - 1:], Wp, db)                   # a row's parts do not depend on its batch-mates
+    assert torch.equal(one[:, 0], parts[:, M - 1])
+    # the norm over the parts = the norm over the rounded sum
+    nw = q(torch.rand(N) + 0.5, dt).to(dt).to(DEV)
+    resid = torch.randn(M, N) * 3
+    r1, r2 = resid.to(DEV), resid.to(DEV)
+    o1 = ops.add_rmsnorm_parts(r1, parts, nw, 1e-6, torch.empty(M, N, dtype=dt, device=DEV))
+    o2 = ops.add_rmsnorm(r2, delta, nw, 1e-6, torch.empty(M, N, dtype=dt, device=DEV))
+    assert torch.equal(o1, o2) and torch.equal(r1, r2)
+    assert torch.equal(r1.cpu(), resid + delta.float().cpu())
+    pick = torch.tensor([M - 1, 0, 3], dtype=torch.int32, device=DEV)    # only some rows (the final norm): resid untouched
+    r3 = resid.to(DEV)
+    o3 = ops.add_rmsnorm_parts(r3, parts, nw, 1e-6, torch.empty(3, N, dtype=dt, device=DEV), rows=pick)
+    assert torch.equal(o3, o1[pick.long()]) and torch.equal(r3.cpu(), resid)
+
+
 @pytest.mark.parametrize("M,N,K", [(8, 896, 4864), (1, 64, 128), (40, 200, 120), (64, 896, 896)])
 def test_gemm_skinny_adds_into_the_residual(ops, M, N, K):
     torch.manual_seed(15)

@@ -12,6 +12,12 @@ int tm_embed_gather(const void* table, int dtype, const int* ids, float* out, in
 int tm_add_rmsnorm(float* resid, const void* delta, const int* rows, const void* weight, int w_dtype, void* out,
                    int dtype, int R, int hidden, float eps, hipStream_t stream);
 
+// The same with what is to be added given as 32-bit partial sums parts[p * stride + i] (p < n_parts) of a product whose
+// K was split over blocks: added in the order of p, rounded to `dtype`, then as above. tm_sum_parts: that rounded sum alone.
+int tm_add_rmsnorm_parts(float* resid, const float* parts, int n_parts, size_t stride, const int* rows, const void* weight,
+                         int w_dtype, void* out, int dtype, int R, int hidden, float eps, hipStream_t stream);
+int tm_sum_parts(const float* parts, int n_parts, size_t stride, void* out, int dtype, size_t n, hipStream_t stream);
+
 int tm_rope_kv_write(void* qkv, int dtype, int T, int H, int KVH, int D, int rot, const float* cos_t,
                      const float* sin_t, const int* positions, const int* slots, void* k_pool, void* v_pool,
                      int page, int write_kv, hipStream_t stream);
@@ -67,6 +73,23 @@ int tm_panel_qkv_rope(const void* X, int ldx, int M, int K, const void* W, const
                       int H, int KVH, int D, const float* cos_t, const float* sin_t, const int* positions,
                       const int* slots, void* k_pool, void* v_pool, int page, hipStream_t stream);
 int tm_panel_gate_up_silu(const void* X, int ldx, int M, int K, const void* W, void* act_out, int I, hipStream_t stream);
+
+// The same products for up to 64 tokens at any width (K a multiple of 8), the matrix streamed once from its packed
+// copy in strips of `rows` rows (16, 8 or 4), and the plain product with bias whose result is stored or, rounded to
+// bfloat16, added into a 32-bit tensor (gemm_stream.hip).
+int tm_gemm_stream_fits(int M, int K);
+int tm_stream_qkv_rope(const void* X, int ldx, int M, int K, const void* W, int rows, const void* bias, int bias_dtype,
+                       void* q_out, int H, int KVH, int D, const float* cos_t, const float* sin_t, const int* positions,
+                       const int* slots, void* k_pool, void* v_pool, int page, hipStream_t stream);
+int tm_stream_gate_up_silu(const void* X, int ldx, int M, int K, const void* W, void* act_out, int I, hipStream_t stream);
+int tm_stream_linear(const void* X, int ldx, int M, int K, const void* W, int rows, int N, const void* bias, int bias_dtype,
+                     void* C, int ldc, int out_f32, float* accum, int ldacc, hipStream_t stream);
+// The plain product with K split over tm_stream_linear_parts(N, K) groups of blocks (a number from the matrix's shape
+// alone; 1: not worth splitting): parts[p][M][N] (float32, M * N elements apart) receives the 32-bit partial sums,
+// the bias in part 0, for tm_add_rmsnorm_parts or tm_sum_parts to add up.
+int tm_stream_linear_parts(int N, int K);
+int tm_stream_linear_split(const void* X, int ldx, int M, int K, const void* W, int rows, int N, const void* bias,
+                           int bias_dtype, float* parts, hipStream_t stream);
 
 int tm_attn_prefill_mfma(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
                          const void* v_pool, const int* block_tables, int table_width, const int* tiles, int n_tiles,

@@ -12,6 +12,8 @@ constexpr int TM_SKINNY_ROWS = 16;
 constexpr int TM_PANEL_ROWS = 48;
 // up to this many rows the products stream the packed matrix once for several row tiles, with their epilogues
 constexpr int TM_STREAM_ROWS = 64;
+// (a plain product of 17 to 64 rows, such as the output and down projections, is streamed where splitting its K over
+// groups of blocks pays: tm_stream_linear_parts in gemm_stream.hip; else it is the library's)
 // most rows one launch of the skinny product takes at all
 constexpr int TM_SKINNY_MAX_ROWS = 64;
 // most rows the 32-bit matrix-vector product takes

@@ -41,20 +41,38 @@ extern "C" int tm_embed_gather(const void* table, int dtype, const int* ids, flo
 // rows == nullptr: row r of the residual is updated in place.
 // rows != nullptr: row rows[r] is read (residual + delta), nothing is written back, out row r.
 // ------------------------------------------------------------------------------------------
+// What is still to be added to the residual stream: a tensor of the model's type, or the partial sums of a product
+// whose K was split over blocks (32-bit, `parts` of them, `stride` elements apart), which are added in their
+// order and rounded to the model's type first, as the product's own epilogue would have stored them.
+template <typename T>
+struct Pending {
+    const T* delta;
+    const float* parts;
+    int n_parts;
+    size_t stride;
+    __device__ __forceinline__ bool any() const { return delta || parts; }
+    __device__ __forceinline__ float at(size_t i) const {
+        if (delta) return Elem<T>::load(delta + i);
+        float s = parts[i];
+        for (int p = 1; p < n_parts; ++p) s += parts[p * stride + i];
+        return Elem<T>::round(s);
+    }
+};
+
 template <typename T, typename WT>
-__global__ void add_rmsnorm_kernel(float* __restrict__ resid, const T* __restrict__ delta,
+__global__ void add_rmsnorm_kernel(float* __restrict__ resid, const Pending<T> pending,
                                    const int* __restrict__ rows, const WT* __restrict__ weight,
                                    T* __restrict__ out, int hidden, float eps) {
     __shared__ float red[4];
     const int r = blockIdx.x;
     const size_t src = rows ? (size_t)rows[r] : (size_t)r;
     float* x = resid + src * hidden;
-    const T* d = delta ? delta + src * hidden : nullptr;
+    const bool d = pending.any();
     T* o = out + (size_t)r * hidden;
     float ss = 0.f;
     for (int c = threadIdx.x; c < hidden; c += 256) {
         float v = x[c];
-        if (d) v += Elem<T>::load(d + c);
+        if (d) v += pending.at(src * hidden + c);
         if (d && !rows) x[c] = v;
         ss += v * v;
     }
@@ -62,7 +80,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const T* __restric
     const float rs = rsqrtf(ss / (float)hidden + eps);
     for (int c = threadIdx.x; c < hidden; c += 256) {
         float v = x[c];
-        if (d && rows) v += Elem<T>::load(d + c);          // in-place rows already hold the sum
+        if (d && rows) v += pending.at(src * hidden + c);   // in-place rows already hold the sum
         const float n = Elem<T>::round(v * rs);            // rounded BEFORE the weight multiplies
         Elem<T>::store(o + c, Elem<WT>::load(weight + c) * n);
     }
@@ -92,7 +110,7 @@ template <> struct Vec4<bf16_t> {
 };
 
 template <typename T, typename WT>
-__global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict__ resid, const T* __restrict__ delta,
+__global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict__ resid, const Pending<T> pending,
                                                               const int* __restrict__ rows,
                                                               const WT* __restrict__ weight, T* __restrict__ out,
                                                               int hidden, float eps) {
@@ -100,7 +118,8 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
     const int r = blockIdx.x;
     const size_t src = rows ? (size_t)rows[r] : (size_t)r;
     float* x = resid + src * hidden;
-    const T* d = delta ? delta + src * hidden : nullptr;
+    const T* d = pending.delta ? pending.delta + src * hidden : nullptr;
+    const float* ps = pending.parts ? pending.parts + src * hidden : nullptr;
     T* o = out + (size_t)r * hidden;
     const int groups = hidden / 4;
     ew_f32x4 v[4];
@@ -113,6 +132,12 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
             v[i] = Vec4<float>::load(x + 4 * gidx);
             if (d) {
                 v[i] += Vec4<T>::load(d + 4 * gidx);
+                if (!rows) Vec4<float>::store(x + 4 * gidx, v[i]);
+            } else if (ps) {
+                ew_f32x4 sum = Vec4<float>::load(ps + 4 * gidx);
+                for (int p = 1; p < pending.n_parts; ++p) sum += Vec4<float>::load(ps + p * pending.stride + 4 * gidx);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) v[i][k] += Elem<T>::round(sum[k]);
                 if (!rows) Vec4<float>::store(x + 4 * gidx, v[i]);
             }
             ss += v[i][0] * v[i][0] + v[i][1] * v[i][1] + v[i][2] * v[i][2] + v[i][3] * v[i][3];
@@ -134,31 +159,70 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
 }
 
 template <typename T, typename WT>
-static void launch_add_rmsnorm(float* resid, const void* delta, const int* rows, const void* weight, void* out, int R,
-                               int hidden, float eps, hipStream_t stream) {
+static void launch_add_rmsnorm(float* resid, const void* delta, const float* parts, int n_parts, size_t stride,
+                               const int* rows, const void* weight, void* out, int R, int hidden, float eps,
+                               hipStream_t stream) {
     const bool vec = hidden % 4 == 0 && hidden <= 4096 && ((uintptr_t)resid % 16) == 0 && ((uintptr_t)weight % 16) == 0 &&
-                     ((uintptr_t)out % 16) == 0 && (!delta || ((uintptr_t)delta % 16) == 0);
+                     ((uintptr_t)out % 16) == 0 && (!delta || ((uintptr_t)delta % 16) == 0) &&
+                     (!parts || (((uintptr_t)parts % 16) == 0 && stride % 4 == 0));
+    const Pending<T> pending{(const T*)delta, parts, n_parts, stride};
     if (vec)
-        add_rmsnorm_vec_kernel<T, WT><<<R, 256, 0, stream>>>(resid, (const T*)delta, rows, (const WT*)weight, (T*)out,
-                                                             hidden, eps);
+        add_rmsnorm_vec_kernel<T, WT><<<R, 256, 0, stream>>>(resid, pending, rows, (const WT*)weight, (T*)out, hidden, eps);
     else
-        add_rmsnorm_kernel<T, WT><<<R, 256, 0, stream>>>(resid, (const T*)delta, rows, (const WT*)weight, (T*)out,
-                                                         hidden, eps);
+        add_rmsnorm_kernel<T, WT><<<R, 256, 0, stream>>>(resid, pending, rows, (const WT*)weight, (T*)out, hidden, eps);
+}
+
+static int add_rmsnorm_any(float* resid, const void* delta, const float* parts, int n_parts, size_t stride, const int* rows,
+                           const void* weight, int w_dtype, void* out, int dtype, int R, int hidden, float eps,
+                           hipStream_t stream) {
+    if (R <= 0) return TM_OK;
+    if (hidden <= 0 || !(eps > 0.f)) return TM_ERR_ARG;
+    if (dtype == TM_F32 && w_dtype == TM_F32)
+        launch_add_rmsnorm<float, float>(resid, delta, parts, n_parts, stride, rows, weight, out, R, hidden, eps, stream);
+    else if (dtype == TM_BF16 && w_dtype == TM_BF16)
+        launch_add_rmsnorm<bf16_t, bf16_t>(resid, delta, parts, n_parts, stride, rows, weight, out, R, hidden, eps, stream);
+    else if (dtype == TM_BF16 && w_dtype == TM_F32)
+        launch_add_rmsnorm<bf16_t, float>(resid, delta, parts, n_parts, stride, rows, weight, out, R, hidden, eps, stream);
+    else
+        return TM_ERR_ARG;
+    TM_CHECK_LAUNCH();
+    return TM_OK;
 }
 
 extern "C" int tm_add_rmsnorm(float* resid, const void* delta, const int* rows, const void* weight,
                               int w_dtype, void* out, int dtype, int R, int hidden, float eps,
                               hipStream_t stream) {
-    if (R <= 0) return TM_OK;
-    if (hidden <= 0 || !(eps > 0.f)) return TM_ERR_ARG;
-    if (dtype == TM_F32 && w_dtype == TM_F32)
-        launch_add_rmsnorm<float, float>(resid, delta, rows, weight, out, R, hidden, eps, stream);
-    else if (dtype == TM_BF16 && w_dtype == TM_BF16)
-        launch_add_rmsnorm<bf16_t, bf16_t>(resid, delta, rows, weight, out, R, hidden, eps, stream);
-    else if (dtype == TM_BF16 && w_dtype == TM_F32)
-        launch_add_rmsnorm<bf16_t, float>(resid, delta, rows, weight, out, R, hidden, eps, stream);
-    else
-        return TM_ERR_ARG;
+    return add_rmsnorm_any(resid, delta, nullptr, 0, 0, rows, weight, w_dtype, out, dtype, R, hidden, eps, stream);
+}
+
+// The same, with what is to be added given as the 32-bit partial sums of a product whose K was split over blocks:
+// parts[p * stride + i], p < n_parts, added in the order of p and rounded to `dtype` before they meet the residual.
+extern "C" int tm_add_rmsnorm_parts(float* resid, const float* parts, int n_parts, size_t stride, const int* rows,
+                                    const void* weight, int w_dtype, void* out, int dtype, int R, int hidden, float eps,
+                                    hipStream_t stream) {
+    if (!parts || n_parts < 1 || n_parts > 16) return TM_ERR_ARG;
+    return add_rmsnorm_any(resid, nullptr, parts, n_parts, stride, rows, weight, w_dtype, out, dtype, R, hidden, eps, stream);
+}
+
+// out[i] = round(sum over p of parts[p * stride + i]) in `dtype`: the partial sums as the tensor the product would
+// have stored.
+template <typename T>
+__global__ void sum_parts_kernel(const float* __restrict__ parts, int n_parts, size_t stride, T* __restrict__ out, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    float s = parts[i];
+    for (int p = 1; p < n_parts; ++p) s += parts[p * stride + i];
+    Elem<T>::store(out + i, s);
+}
+
+extern "C" int tm_sum_parts(const float* parts, int n_parts, size_t stride, void* out, int dtype, size_t n,
+                            hipStream_t stream) {
+    if (n == 0) return TM_OK;
+    if (!parts || n_parts < 1 || !out) return TM_ERR_ARG;
+    const unsigned blocks = (unsigned)((n + 255) / 256);
+    if (dtype == TM_BF16) sum_parts_kernel<bf16_t><<<blocks, 256, 0, stream>>>(parts, n_parts, stride, (bf16_t*)out, n);
+    else if (dtype == TM_F32) sum_parts_kernel<float><<<blocks, 256, 0, stream>>>(parts, n_parts, stride, (float*)out, n);
+    else return TM_ERR_ARG;
     TM_CHECK_LAUNCH();
     return TM_OK;
 }

@@ -22,6 +22,7 @@
 namespace {
 
 enum { OP_EMBED = 0, OP_ATTENTION, OP_FEED_FORWARD, OP_HEAD };
+constexpr int TM_MAX_SUMS = 8;          // most groups of blocks a product's K is split over (tm_stream_linear_parts)
 
 struct Op {
     int kind;
@@ -79,6 +80,12 @@ bool skinny_ok(const TmLinear& L, const void* x, int ldx, int dtype) {
 bool panel_ok(const TmLinear& L, const void* x, int ldx, int M, int dtype) {
     return L.packed && M > TM_SKINNY_ROWS && M <= TM_PANEL_ROWS && dtype == TM_BF16 && ldx % 8 == 0 && aligned(x, 16) &&
            tm_gemm_panel_fits(M, L.K);
+}
+
+// the products that stream a packed matrix once for up to 64 tokens (gemm_stream.hip)
+bool stream_ok(const TmLinear& L, const void* x, int ldx, int M, int dtype) {
+    return L.packed && M > TM_SKINNY_ROWS && M <= TM_STREAM_ROWS && dtype == TM_BF16 && L.dtype == TM_BF16 && ldx % 8 == 0 &&
+           aligned(x, 16) && tm_gemm_stream_fits(M, L.K);
 }
 
 // The product rule. x_dtype: type of x (the model's activations); the matrix has its own (L.dtype).
@@ -146,7 +153,8 @@ struct Products {
     // Is there a kernel that adds round(x W^T + b) into a 32-bit accumulator in its epilogue?
     bool accumulates(const TmLinear& L, int dtype, const void* x, int ldx, int M) const {
         if (L.dtype != dtype || M <= 0) return false;
-        return (L.packed_parts == 1 && packed_ok(L, x, ldx, M, dtype)) || (M <= TM_SKINNY_ROWS && skinny_ok(L, x, ldx, dtype));
+        return (L.packed_parts == 1 && packed_ok(L, x, ldx, M, dtype)) ||
+               (M <= TM_SKINNY_ROWS && skinny_ok(L, x, ldx, dtype));
     }
 
     int accumulate(const TmLinear& L, int dtype, const void* x, int ldx, int M, float* accum, int ldacc) const {
@@ -173,6 +181,8 @@ struct Run {
     // workspace
     void *x, *qkv, *attn, *gu, *act, *delta_buf, *hnorm;
     float *part_o, *part_ml;
+    float* sums;                        // room for the partial sums of a product whose K is split over blocks, or null
+    int pending_sums = 0;               // that many partial sums [T, hidden] in `sums` are still to be added to the residual
 
     struct Label {
         const Run* r;
@@ -192,6 +202,17 @@ struct Run {
     // resid += round(x W^T + b) in the product's epilogue where a kernel does that and the caller lets it; else the
     // product goes to delta_buf and is added by the next norm (or handed back).
     int project(const TmLinear& L, const void* x_, int ldx, int M) {
+        // 17 to 64 rows over a matrix with few rows of output: K split over groups of blocks, whose partial sums the
+        // next norm adds up (or, where the caller wants the result itself, a small kernel)
+        const int groups = (sums && L.N == p->hidden && L.packed_parts == 1 && stream_ok(L, x_, ldx, M, dtype))
+                               ? tm_stream_linear_parts(L.N, L.K) : 1;
+        if (groups >= 2 && groups <= TM_MAX_SUMS) {
+            const int rc = tm_stream_linear_split(x_, ldx, M, L.K, L.packed, L.packed_rows, L.N, L.bias, L.bias_dtype, sums, stream);
+            if (rc) return rc;
+            delta = nullptr;
+            pending_sums = groups;
+            return accumulate && resid ? TM_OK : settle();
+        }
         if (accumulate && resid && products.accumulates(L, dtype, x_, ldx, M)) {
             delta = nullptr;
             return products.accumulate(L, dtype, x_, ldx, M, resid, L.N);
@@ -200,18 +221,38 @@ struct Run {
         return linear(L, x_, ldx, M, delta_buf, L.N, dtype);
     }
 
-    // x = norm(resid + delta), resid updated
-    int normed(const TmNorm& n) {
-        if (!n.w || !resid) return TM_ERR_ARG;
-        const int rc = tm_add_rmsnorm(resid, delta, nullptr, n.w, n.w_dtype, x, dtype, s->T, p->hidden, n.eps, stream);
-        delta = nullptr;
+    // The partial sums become the tensor the product would have stored: delta.
+    int settle() {
+        if (!pending_sums) return TM_OK;
+        const size_t n = (size_t)s->T * p->hidden;
+        const int rc = tm_sum_parts(sums, pending_sums, n, delta_buf, dtype, n, stream);
+        pending_sums = 0;
+        delta = delta_buf;
         return rc;
     }
+
+    // out = norm(resid + what is pending), for all rows (resid updated) or the rows named
+    int add_norm(const TmNorm& n, const int* rows, void* out, int R) {
+        if (!n.w || !resid) return TM_ERR_ARG;
+        int rc;
+        if (pending_sums)
+            rc = tm_add_rmsnorm_parts(resid, sums, pending_sums, (size_t)s->T * p->hidden, rows, n.w, n.w_dtype, out, dtype, R,
+                                      p->hidden, n.eps, stream);
+        else
+            rc = tm_add_rmsnorm(resid, delta, rows, n.w, n.w_dtype, out, dtype, R, p->hidden, n.eps, stream);
+        delta = nullptr;
+        pending_sums = 0;
+        return rc;
+    }
+
+    // x = norm(resid + delta), resid updated
+    int normed(const TmNorm& n) { return add_norm(n, nullptr, x, s->T); }
 
     int embedding(int op, const TmEmbedOp& e) {
         Label l(this, op, TM_LABEL_EMBED);
         if (!resid) return TM_ERR_ARG;
         delta = nullptr;
+        pending_sums = 0;
         return tm_embed_gather(e.table, e.dtype, s->token_ids, resid, s->T, p->hidden, e.V, stream);
     }
 
@@ -241,7 +282,7 @@ struct Run {
             Label l(this, op, TM_LABEL_QKV);
             const bool own_norm = x_in == nullptr;
             // 1. the kernel that starts at the norm (at most 16 tokens)
-            if (own_norm && dtype == TM_BF16 && a.qkv.dtype == TM_BF16 && a.D % 32 == 0 && delta == nullptr && a.norm.w &&
+            if (own_norm && dtype == TM_BF16 && a.qkv.dtype == TM_BF16 && a.D % 32 == 0 && delta == nullptr && !pending_sums && a.norm.w &&
                 tables_fusable && fused_decode_ok(resid, a.qkv, T) && is_pow2(a.page) && bias_ok) {
                 rc = tm_fused_norm_qkv_rope(resid, a.norm.w, a.norm.w_dtype, a.norm.eps, T, hidden, a.qkv.packed, a.qkv.bias,
                                             a.qkv.bias_dtype, qkv, a.H, a.KVH, a.D, a.cos_t, a.sin_t, s->positions, slots, kp, vp,
@@ -264,8 +305,16 @@ struct Run {
                     q = qkv;
                     q_stride = HD;
                     ++p->taken[TM_QKV_PANEL];
+                } else if (tables_fusable && a.D % 32 == 0 && a.qkv.packed_parts == 1 && stream_ok(a.qkv, xn, hidden, T, dtype) &&
+                           is_pow2(a.page)) {
+                    // 3. the packed matrix streamed once for up to 64 tokens
+                    rc = tm_stream_qkv_rope(xn, hidden, T, hidden, a.qkv.packed, a.qkv.packed_rows, a.qkv.bias, a.qkv.bias_dtype,
+                                            qkv, a.H, a.KVH, a.D, a.cos_t, a.sin_t, s->positions, slots, kp, vp, a.page, stream);
+                    q = qkv;
+                    q_stride = HD;
+                    ++p->taken[TM_QKV_STREAM];
                 } else {
-                    // 3. product, then rotation and cache write
+                    // 4. product, then rotation and cache write
                     if ((rc = linear(a.qkv, xn, hidden, T, qkv, QKV, dtype))) return rc;
                     if (a.rot > 0 || a.write)
                         rc = tm_rope_kv_write(qkv, dtype, T, a.H, a.KVH, a.D, a.rot, a.rot > 0 ? a.cos_t : nullptr,
@@ -332,7 +381,7 @@ struct Run {
             const bool own_norm = x_in == nullptr;
             const bool plain = f.gate_up.dtype == dtype && f.gate_up.bias == nullptr;
             const bool two_parts = f.gate_up.packed_parts == 2 && f.gate_up.packed_rows == 16;
-            if (own_norm && dtype == TM_BF16 && plain && f.I % 4 == 0 && delta == nullptr && f.norm.w && two_parts &&
+            if (own_norm && dtype == TM_BF16 && plain && f.I % 4 == 0 && delta == nullptr && !pending_sums && f.norm.w && two_parts &&
                 fused_decode_ok(resid, f.gate_up, T)) {
                 rc = tm_fused_norm_gate_up_silu(resid, f.norm.w, f.norm.w_dtype, f.norm.eps, T, hidden, f.gate_up.packed, act, f.I, stream);
                 ++p->taken[TM_GATE_UP_FROM_NORM];
@@ -353,6 +402,9 @@ struct Run {
                 } else if (plain && two_parts && f.I % 4 == 0 && panel_ok(f.gate_up, xn, hidden, T, dtype)) {
                     rc = tm_panel_gate_up_silu(xn, hidden, T, hidden, f.gate_up.packed, act, f.I, stream);
                     ++p->taken[TM_GATE_UP_PANEL];
+                } else if (plain && two_parts && f.I % 4 == 0 && stream_ok(f.gate_up, xn, hidden, T, dtype)) {
+                    rc = tm_stream_gate_up_silu(xn, hidden, T, hidden, f.gate_up.packed, act, f.I, stream);
+                    ++p->taken[TM_GATE_UP_STREAM];
                 } else {
                     if ((rc = linear(f.gate_up, xn, hidden, T, gu, 2 * f.I, dtype))) return rc;
                     rc = tm_silu_mul(gu, act, dtype, T, f.I, stream);
@@ -373,13 +425,12 @@ struct Run {
         x_in = nullptr;
         if (!h) {
             Label l(this, op, TM_LABEL_NORM);
-            if (!f.norm.w || !resid) return TM_ERR_ARG;
-            const int rc = tm_add_rmsnorm(resid, delta, s->logit_rows, f.norm.w, f.norm.w_dtype, hnorm, dtype, R, p->hidden,
-                                          f.norm.eps, stream);
+            const int rc = add_norm(f.norm, s->logit_rows, hnorm, R);
             if (rc) return rc;
             h = hnorm;
         }
         delta = nullptr;
+        pending_sums = 0;
         Label l(this, op, TM_LABEL_HEAD);
         return linear(f.head, h, p->hidden, R, logits, f.head.N, TM_F32);
     }
@@ -492,6 +543,8 @@ size_t tm_program_workspace_bytes(const TmProgram* p, int T, int R, int num_deco
     const size_t chunks = (size_t)tm_decode_chunks(max_decode_context > 0 ? max_decode_context : 1);
     n += align_up((size_t)num_decode * p->max_heads_d * chunks * 4); // split decode attention: partial values
     n += align_up((size_t)num_decode * p->max_heads * chunks * 2 * 4);   // ... and their (max, sum)
+    if (T <= TM_STREAM_ROWS && p->dtype == TM_BF16)
+        n += align_up((size_t)TM_MAX_SUMS * T * p->hidden * 4);      // partial sums of a product whose K is split over blocks
     const size_t rows = (size_t)(T > R ? T : R);
     n += align_up(rows * p->max_wide_in * 4);                        // 32-bit copies around the product of a 32-bit matrix
     n += align_up(rows * p->max_wide_out * 4);
@@ -533,6 +586,7 @@ int tm_program_run(const TmProgram* p, int first, int count, const TmStep* s, Tm
     const size_t chunks = (size_t)tm_decode_chunks(s->max_decode_context > 0 ? s->max_decode_context : 1);
     r.part_o = (float*)take((size_t)s->num_decode * p->max_heads_d * chunks * 4);
     r.part_ml = (float*)take((size_t)s->num_decode * p->max_heads * chunks * 2 * 4);
+    r.sums = (T <= TM_STREAM_ROWS && p->dtype == TM_BF16) ? (float*)take((size_t)TM_MAX_SUMS * T * p->hidden * 4) : nullptr;
     const size_t rows = (size_t)(T > R ? T : R);
     if (p->max_wide_in) r.products.wide_in = (float*)take(rows * p->max_wide_in * 4);
     if (p->max_wide_out) r.products.wide_out = (float*)take(rows * p->max_wide_out * 4);
@@ -546,6 +600,7 @@ int tm_program_run(const TmProgram* p, int first, int count, const TmStep* s, Tm
             default: rc = r.head(i, op.head, logits); break;
         }
     }
+    if (!rc) rc = r.settle();                   // partial sums do not cross to the caller: it gets the tensor
     io->delta = r.delta;
     io->x = nullptr;
     io->qkv = nullptr;

@@ -822,6 +822,150 @@ def panel_gate_up_silu(x: torch.Tensor, w: PackedWeight, out: torch.Tensor) -> t
     return out
 
 
+def stream_fits(M: int, K: int) -> bool:
+    """Do the products that stream a packed matrix once for up to 64 tokens take M tokens of width K?"""
+    return bool(library().tm_gemm_stream_fits(c_int(M), c_int(K)))
+
+
+def _stream_input(x: torch.Tensor, w: PackedWeight, who: str) -> int:
+    M, K = x.shape
+    _need(x.dtype == torch.bfloat16 and x.stride(1) == 1 and x.data_ptr() % 16 == 0 and stream_fits(M, K) and K == w.k,
+          f"{who}: x bfloat16 [M<=64, {w.k}], 16-byte aligned")
+    ldx = x.stride(0) if M > 1 else max(K, x.stride(0))
+    _need(ldx % 8 == 0, f"{who}: rows of x must be 16-byte aligned")
+    return ldx
+
+
+def stream_qkv_rope(x: torch.Tensor, w: PackedWeight, bias: torch.Tensor | None, q_out: torch.Tensor, H: int, KVH: int,
+                    D: int, cos: torch.Tensor, sin: torch.Tensor, positions: torch.Tensor, slots: torch.Tensor | None,
+                    k_pool: torch.Tensor | None, v_pool: torch.Tensor | None) -> torch.Tensor:
+    """q_out[M, H*D] and the cache <- rope(x @ w^T + bias) for up to 64 tokens of any width; x bfloat16 [M, K] is the
+    normed input, w the [(H + 2 KVH) D, K] matrix packed in strips of 16, 8 or 4 rows; the rest as for
+    ``fused_norm_qkv_rope``."""
+    _gpu(x, bias, q_out, cos, sin, positions, slots, k_pool, v_pool)
+    M, K = x.shape
+    _packed_operand(w, None, "stream qkv")
+    ldx = _stream_input(x, w, "stream qkv")
+    _need(D % 32 == 0, f"stream qkv: head size {D} must be a multiple of 32")
+    _need((w.n, w.k) == ((H + 2 * KVH) * D, K) and len(w.parts) == 1, "stream qkv: w must be the packed [(H+2KVH)D, K] matrix")
+    _need(cos.dtype == torch.float32 and sin.dtype == torch.float32 and cos.is_contiguous() and sin.is_contiguous()
+          and cos.shape == sin.shape and cos.dim() == 2 and cos.shape[1] * 2 == D and cos.data_ptr() % 16 == 0
+          and sin.data_ptr() % 16 == 0, "stream qkv: cos/sin must be float32 [max_pos, D/2] (rotation over the whole head)")
+    _need(q_out.dtype == torch.bfloat16 and q_out.is_contiguous() and tuple(q_out.shape) == (M, H * D), "stream qkv: q_out [M, H*D]")
+    _ints(positions, M, "positions")
+    page = 16
+    if slots is not None:
+        _need(k_pool is not None and v_pool is not None, "stream qkv: slots need the cache pools")
+        page = _check_pools(k_pool, v_pool, KVH, D, torch.bfloat16, "stream qkv")
+        _need(page & (page - 1) == 0, "stream qkv: the page size must be a power of two")
+        _ints(slots, M, "slots")
+    if bias is not None:
+        _need(tuple(bias.shape) == (w.n,) and bias.is_contiguous(), "stream qkv: bias [rows]")
+    _check(library().tm_stream_qkv_rope(_p(x), c_int(ldx), c_int(M), c_int(K), _p(w.data), c_int(w.rows), _p(bias),
+                                        c_int(code(bias.dtype) if bias is not None else -1), _p(q_out), c_int(H),
+                                        c_int(KVH), c_int(D), _p(cos), _p(sin), _p(positions), _p(slots),
+                                        _p(k_pool if slots is not None else None),
+                                        _p(v_pool if slots is not None else None), c_int(page), _stream()),
+           "stream_qkv_rope")
+    return q_out
+
+
+def stream_gate_up_silu(x: torch.Tensor, w: PackedWeight, out: torch.Tensor) -> torch.Tensor:
+    """out[M, I] <- silu(x Wg^T) * (x Wu^T) for up to 64 tokens of any width; w as for ``fused_norm_gate_up_silu``."""
+    _gpu(x, out)
+    M, K = x.shape
+    I = out.shape[1]
+    _packed_operand(w, 16, "stream gate-up")
+    ldx = _stream_input(x, w, "stream gate-up")
+    _need((w.n, w.k) == (2 * I, K) and w.parts == (I, I) and I % 4 == 0,
+          "stream gate-up: w must be the packed [2I, K] matrix in two parts of I rows; I % 4 == 0")
+    _need(out.dtype == torch.bfloat16 and out.is_contiguous() and out.shape[0] == M, "stream gate-up: out bfloat16 [M, I]")
+    _check(library().tm_stream_gate_up_silu(_p(x), c_int(ldx), c_int(M), c_int(K), _p(w.data), _p(out), c_int(I),
+                                            _stream()), "stream_gate_up_silu")
+    return out
+
+
+def stream_linear(x: torch.Tensor, w: PackedWeight, bias: torch.Tensor | None, out: torch.Tensor | None,
+                  accum: torch.Tensor | None = None) -> torch.Tensor:
+    """out[M, N] = x @ w^T (+ bias) for up to 64 tokens of any width, out bfloat16 or float32; or with ``accum``
+    (float32 [M, N]) the result, rounded to bfloat16, is added there and out stays unwritten. w: the [N, K]
+    matrix packed as one part in strips of 16, 8 or 4 rows."""
+    _gpu(x, bias, out, accum)
+    M, K = x.shape
+    _packed_operand(w, None, "stream linear")
+    ldx = _stream_input(x, w, "stream linear")
+    N = w.n
+    _need(len(w.parts) == 1, "stream linear: the matrix is packed as one part")
+    if bias is not None:
+        _need(tuple(bias.shape) == (N,) and bias.is_contiguous(), "stream linear: bias must be [N]")
+    if accum is not None:
+        _need(out is None and accum.dtype == torch.float32 and tuple(accum.shape) == (M, N) and accum.stride(1) == 1,
+              "stream linear: accum must be float32 [M, N], and excludes out")
+        ldacc = accum.stride(0) if M > 1 else max(N, accum.stride(0))
+        c, ldc, f32 = None, N, 0
+    else:
+        _need(out is not None and tuple(out.shape) == (M, N) and out.stride(1) == 1
+              and out.dtype in (torch.bfloat16, torch.float32), "stream linear: out [M, N] bfloat16 or float32")
+        ldacc = 0
+        c, ldc, f32 = out, (out.stride(0) if M > 1 else max(N, out.stride(0))), 1 if out.dtype == torch.float32 else 0
+    _check(library().tm_stream_linear(_p(x), c_int(ldx), c_int(M), c_int(K), _p(w.data), c_int(w.rows), c_int(N), _p(bias),
+                                      c_int(code(bias.dtype) if bias is not None else -1), _p(c), c_int(ldc), c_int(f32),
+                                      _p(accum), c_int(ldacc), _stream()), "stream_linear")
+    return accum if accum is not None else out
+
+
+def stream_linear_split(x: torch.Tensor, w: PackedWeight, bias: torch.Tensor | None) -> torch.Tensor:
+    """The plain product of up to 64 rows with K split over groups of blocks: returns float32 [parts, M, N], the
+    partial sums (bias in part 0) that ``add_rmsnorm_parts`` or ``sum_parts`` add up. The number of parts follows
+    from the matrix's shape alone."""
+    _gpu(x, bias)
+    M, K = x.shape
+    _packed_operand(w, None, "stream linear")
+    ldx = _stream_input(x, w, "stream linear")
+    N = w.n
+    _need(len(w.parts) == 1, "stream linear: the matrix is packed as one part")
+    if bias is not None:
+        _need(tuple(bias.shape) == (N,) and bias.is_contiguous(), "stream linear: bias must be [N]")
+    n_parts = library().tm_stream_linear_parts(c_int(N), c_int(K))
+    parts = torch.empty((n_parts, M, N), dtype=torch.float32, device=x.device)
+    _check(library().tm_stream_linear_split(_p(x), c_int(ldx), c_int(M), c_int(K), _p(w.data), c_int(w.rows), c_int(N),
+                                            _p(bias), c_int(code(bias.dtype) if bias is not None else -1), _p(parts),
+                                            _stream()), "stream_linear_split")
+    return parts
+
+
+def sum_parts(parts: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out = round(parts[0] + parts[1] + ...) in out's type; parts float32 [P, ...]."""
+    _gpu(parts, out)
+    _need(parts.dtype == torch.float32 and parts.is_contiguous() and out.is_contiguous()
+          and tuple(parts.shape[1:]) == tuple(out.shape), "sum_parts: parts float32 [P, *out.shape]")
+    _check(library().tm_sum_parts(_p(parts), c_int(parts.shape[0]), ctypes.c_size_t(out.numel()), _p(out), code(out.dtype),
+                                  ctypes.c_size_t(out.numel()), _stream()), "sum_parts")
+    return out
+
+
+def add_rmsnorm_parts(resid: torch.Tensor, parts: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor,
+                      rows: torch.Tensor | None = None) -> torch.Tensor:
+    """``add_rmsnorm`` with what is to be added given as float32 partial sums [P, T, hidden]: added in their order and
+    rounded to out's type before they meet the residual."""
+    _gpu(resid, parts, weight, out, rows)
+    T, hidden = resid.shape
+    R = T if rows is None else rows.numel()
+    _need(resid.dtype == torch.float32 and resid.is_contiguous(), "add_rmsnorm: the residual stream is contiguous float32")
+    _need(tuple(out.shape) == (R, hidden) and out.is_contiguous(), f"add_rmsnorm: out must be [{R}, {hidden}]")
+    _need(parts.dtype == torch.float32 and parts.is_contiguous() and parts.dim() == 3 and tuple(parts.shape[1:]) == (T, hidden)
+          and 1 <= parts.shape[0] <= 16, "add_rmsnorm: parts must be float32 [P <= 16, T, hidden]")
+    _need(tuple(weight.shape) == (hidden,) and weight.is_contiguous(), "add_rmsnorm: weight must be [hidden]")
+    _need(out.dtype == torch.bfloat16 or weight.dtype == torch.float32, "add_rmsnorm: a float32 output needs float32 weights")
+    if rows is not None:
+        _ints(rows, R, "rows")
+    _need(eps > 0, "add_rmsnorm: eps must be positive")
+    _check(library().tm_add_rmsnorm_parts(_p(resid), _p(parts), c_int(parts.shape[0]), ctypes.c_size_t(T * hidden), _p(rows),
+                                          _p(weight), code(weight.dtype), _p(out), code(out.dtype), c_int(R), c_int(hidden),
+                                          c_float(eps), _stream()), "add_rmsnorm_parts")
+    return out
+
+
 def fused_lds_fits(M: int, K: int) -> bool:
     """Does the normed input of M tokens (4, 8 or 16 rows of K + 8 bfloat16), beside the partial sums of
     the block's 4 (K < 2048) or 8 wavefronts, fit the 160 KB of LDS a block of the norm-fused products may use?"""
