@@ -109,6 +109,8 @@ template <> struct Vec4<bf16_t> {
     }
 };
 
+#define ADD_NORM_MAX_PARTS 8       // most partial sums the vector kernel adds (more: the plain kernel)
+
 template <typename T, typename WT>
 __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict__ resid, const Pending<T> pending,
                                                               const int* __restrict__ rows,
@@ -134,8 +136,15 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
                 v[i] += Vec4<T>::load(d + 4 * gidx);
                 if (!rows) Vec4<float>::store(x + 4 * gidx, v[i]);
             } else if (ps) {
-                ew_f32x4 sum = Vec4<float>::load(ps + 4 * gidx);
-                for (int p = 1; p < pending.n_parts; ++p) sum += Vec4<float>::load(ps + p * pending.stride + 4 * gidx);
+                // all parts asked for at once (a part that does not exist: part 0 again, not counted), then added in order
+                ew_f32x4 part[ADD_NORM_MAX_PARTS];
+#pragma unroll
+                for (int p = 0; p < ADD_NORM_MAX_PARTS; ++p)
+                    part[p] = Vec4<float>::load(ps + (size_t)(p < pending.n_parts ? p : 0) * pending.stride + 4 * gidx);
+                ew_f32x4 sum = part[0];
+#pragma unroll
+                for (int p = 1; p < ADD_NORM_MAX_PARTS; ++p)
+                    if (p < pending.n_parts) sum += part[p];
 #pragma unroll
                 for (int k = 0; k < 4; ++k) v[i][k] += Elem<T>::round(sum[k]);
                 if (!rows) Vec4<float>::store(x + 4 * gidx, v[i]);
@@ -164,7 +173,7 @@ static void launch_add_rmsnorm(float* resid, const void* delta, const float* par
                                hipStream_t stream) {
     const bool vec = hidden % 4 == 0 && hidden <= 4096 && ((uintptr_t)resid % 16) == 0 && ((uintptr_t)weight % 16) == 0 &&
                      ((uintptr_t)out % 16) == 0 && (!delta || ((uintptr_t)delta % 16) == 0) &&
-                     (!parts || (((uintptr_t)parts % 16) == 0 && stride % 4 == 0));
+                     (!parts || (((uintptr_t)parts % 16) == 0 && stride % 4 == 0 && n_parts <= ADD_NORM_MAX_PARTS));
     const Pending<T> pending{(const T*)delta, parts, n_parts, stride};
     if (vec)
         add_rmsnorm_vec_kernel<T, WT><<<R, 256, 0, stream>>>(resid, pending, rows, (const WT*)weight, (T*)out, hidden, eps);

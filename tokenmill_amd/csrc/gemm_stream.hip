@@ -170,6 +170,26 @@ __global__ __launch_bounds__(64 * KS * US) void gemm_stream_kernel(const StreamA
         accB[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     }
     const int rounds = (per + ST_KCH - 1) / ST_KCH;                  // the same for every wavefront of the block
+    // What the q|k|v epilogue needs from memory, where a wavefront owns one token tile (tile kw): the token's position,
+    // cache slot and the bias are asked for before anything else (loads come back in the order they were issued, so
+    // these are not behind the matrix), the rotary row, whose address hangs on the position, after the first round.
+    constexpr bool PRE = EPI == ST_EPI_QKV && NT <= KS;
+    int pre_pos = 0, pre_slot = -1;
+    float pre_bA[4] = {0.f, 0.f, 0.f, 0.f}, pre_bB[4] = {0.f, 0.f, 0.f, 0.f};
+    f32x4_t pre_cs = {0.f, 0.f, 0.f, 0.f}, pre_sn = {0.f, 0.f, 0.f, 0.f};
+    if constexpr (PRE) {
+        const int tok = 16 * kw + r < M ? 16 * kw + r : M - 1;       // (tile kw may not exist: a token that does)
+        pre_pos = f.positions[tok];
+        pre_slot = f.slots ? f.slots[tok] : -1;
+        if (f.bias) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int ia = cu.nA + 4 * g + i, ib = cu.nB + 4 * g + i;
+                pre_bA[i] = f.bias_f32 ? ((const float*)f.bias)[ia] : bf16_to_f32(((const bf16_t*)f.bias)[ia]);
+                pre_bB[i] = f.bias_f32 ? ((const float*)f.bias)[ib] : bf16_to_f32(((const bf16_t*)f.bias)[ib]);
+            }
+        }
+    }
     // The matrix runs ST_WD k-steps ahead of the products, in registers: the activations of a k-step need to be in
     // LDS only when it is multiplied, so how much of the matrix a wavefront has in flight is not bound by LDS.
     FFrag fa[ST_WD], fb[ST_WD];
@@ -188,6 +208,13 @@ __global__ __launch_bounds__(64 * KS * US) void gemm_stream_kernel(const StreamA
                 store_x(round);
                 __syncthreads();
                 if (round + 1 < rounds) load_x(round + 1);            // on their way while this round multiplies
+                if constexpr (PRE) {
+                    if (round == 0 && cu.head < f.H + f.KVH) {        // the position has arrived with the first activations
+                        const size_t at = (size_t)pre_pos * (f.D / 2) + 16 * cu.jt + 4 * g;
+                        pre_cs = *(const f32x4_t*)(f.cos_t + at);
+                        pre_sn = *(const f32x4_t*)(f.sin_t + at);
+                    }
+                }
                 const int base = ks0 + round * ST_KCH;
 #pragma unroll
                 for (int j = 0; j < ST_KCH; ++j) {
@@ -258,8 +285,8 @@ __global__ __launch_bounds__(64 * KS * US) void gemm_stream_kernel(const StreamA
             float xA[4], xB[4];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                float bA = 0.f, bB = 0.f;
-                if (f.bias) {
+                float bA = pre_bA[i], bB = pre_bB[i];
+                if (!PRE && f.bias) {
                     const int ia = cu.nA + 4 * g + i, ib = cu.nB + 4 * g + i;
                     bA = f.bias_f32 ? ((const float*)f.bias)[ia] : bf16_to_f32(((const bf16_t*)f.bias)[ia]);
                     bB = f.bias_f32 ? ((const float*)f.bias)[ib] : bf16_to_f32(((const bf16_t*)f.bias)[ib]);
@@ -267,12 +294,16 @@ __global__ __launch_bounds__(64 * KS * US) void gemm_stream_kernel(const StreamA
                 xA[i] = fd_round(sA[i] + bA);
                 xB[i] = fd_round(sB[i] + bB);
             }
-            const int slot = f.slots ? f.slots[tok] : -1;
+            const int slot = PRE ? pre_slot : (f.slots ? f.slots[tok] : -1);
             if (cu.head < f.H + f.KVH) {
                 const int half = f.D / 2;
                 const int j0 = 16 * cu.jt + 4 * g;                                   // pair index of element 0
-                const size_t at = (size_t)f.positions[tok] * half + j0;
-                const f32x4_t cs = *(const f32x4_t*)(f.cos_t + at), sn = *(const f32x4_t*)(f.sin_t + at);
+                f32x4_t cs = pre_cs, sn = pre_sn;
+                if (!PRE) {
+                    const size_t at = (size_t)f.positions[tok] * half + j0;
+                    cs = *(const f32x4_t*)(f.cos_t + at);
+                    sn = *(const f32x4_t*)(f.sin_t + at);
+                }
                 float y1[4], y2[4];
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
