@@ -4,10 +4,12 @@ weights, synthetic token ids, on one MI355X.
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype bfloat16|float32] [--layers L]
                     [--config CONFIG.json|NAME]      another shape of the architecture (7b, 32b, a file)
                     [--part all|decode|prefill|offline|mixed7b|preempt32b]
+                    [--part decode --contexts 8192,32768 --batches 8,64]     decode steps over long contexts
 
 A "step" is one decode step of the engine (scheduling, metadata upload, the forward pass and greedy
 sampling) with a batch of 8 requests, each holding a 2,048-token prompt. One JSON line is printed:
-the decode rate, the step-time histogram, the prefill, decoding at batch 1 and 64, the step's
+the decode rate, the step-time histogram, the prefill, decoding at batch 1 and 64 and, at the headline
+batch, over contexts of 8,192 and 32,768 tokens (each with the fraction of the HBM peak its step reaches), the step's
 roofline fraction, and per operation its GPU time and the share of its own floor it reaches, with
 "GPU idle" = wall time - kernel time (what the reference's profiler reports, reference
 bench/profile_decode.py:73-82). Bytes and flops come from the model's parts (they state what each
@@ -68,6 +70,10 @@ def main() -> int:
     ap.add_argument("--offline-gen", type=int, default=128)
     ap.add_argument("--offline-seqs", type=int, default=128, help="requests running at a time in the offline run")
     ap.add_argument("--chunked", action="store_true", help="offline run: portions of prompts beside decoding requests")
+    ap.add_argument("--contexts", default=None,
+                    help="with --part decode: instead of one batch, a sweep of decode steps over these context lengths (e.g. 8192,32768) "
+                         "and the --batches, each with its roofline fraction")
+    ap.add_argument("--batches", default="8,64", help="batch sizes of the --contexts sweep")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -79,6 +85,10 @@ def main() -> int:
     prompt_len = args.prompt_len
     long_context = args.part in ("mixed7b", "preempt32b")
     max_model_len = 8192 if long_context else max(MAX_MODEL_LEN, prompt_len + args.steps + args.warmup + HISTOGRAM_STEPS + 128)
+    # context lengths beyond the headline's, decoded at the headline batch: two more entries of `points` (or, with
+    # --contexts, a sweep of its own)
+    LONG_POINTS = (8192, 32768)
+    sweep = [int(c) for c in args.contexts.split(",")] if args.contexts else []
 
     import torch
 
@@ -95,7 +105,10 @@ def main() -> int:
     layers_full = shape["num_hidden_layers"]
     if args.layers:
         shape["num_hidden_layers"] = args.layers
-    model = load_random_model(shape, seed=0, dtype=dtype, device=device, max_positions=max_model_len)
+    # the position tables reach the longest context any engine of this run allows (each engine has its own limit)
+    most_positions = max([max_model_len] + sweep + ([] if args.skip_points or args.part != "all" else list(LONG_POINTS)))
+    most_positions = min(most_positions, shape.get("max_position_embeddings", most_positions))
+    model = load_random_model(shape, seed=0, dtype=dtype, device=device, max_positions=most_positions)
     gen = torch.Generator().manual_seed(0)
     vocab = shape["vocab_size"]
 
@@ -110,7 +123,7 @@ def main() -> int:
                 "head_dim": getattr(model.config, "head_dim", None), "intermediate": shape.get("intermediate_size"),
                 "vocab": shape.get("vocab_size"), "tied": bool(shape.get("tie_word_embeddings", False))}
 
-    def engine_for(batch, extra_steps=0):
+    def engine_for(batch, extra_steps=0, prompt_len=prompt_len, max_model_len=max_model_len):
         pages = batch * (-(-(prompt_len + args.steps + args.warmup + extra_steps + 64) // BLOCK_SIZE)) + 8
         cfg = EngineConfig(dtype=args.dtype, block_size=BLOCK_SIZE, num_blocks=pages, max_model_len=max_model_len,
                            max_num_seqs=max(batch, 1), max_num_batched_tokens=max(prompt_len, batch),
@@ -136,13 +149,19 @@ def main() -> int:
         finally:
             runner.graphs, runner.step_graphs = saved
 
-    def time_decode(batch, steps, warmup, detail=False):
+    def time_decode(batch, steps, warmup, detail=False, context=None):
         """ms per step over exactly ``steps`` steps; with ``detail`` also the histogram over at least
-        HISTOGRAM_STEPS steps, the step's bytes, and the kernel trace."""
+        HISTOGRAM_STEPS steps, the step's bytes, and the kernel trace. ``context``: the requests' length when the
+        timed steps end (prompts that much shorter than it), in an engine whose limit is that context; with it the
+        step's bytes come back too."""
         extra = (max(0, HISTOGRAM_STEPS - steps) + 2 * PROFILED_STEPS + 4) if detail else 0
-        eng = engine_for(batch, extra)
+        if context is None:
+            eng, prompt_tokens = engine_for(batch, extra), prompt_len
+        else:
+            prompt_tokens = context - steps - warmup - 16
+            eng = engine_for(batch, 16, prompt_len=prompt_tokens, max_model_len=context)
         sp = SamplingParams(max_tokens=steps + warmup + extra + 8, ignore_eos=True)
-        for i, p in enumerate(prompts(batch)):
+        for i, p in enumerate(prompts(batch, prompt_tokens)):
             eng.add_request(f"d{i}", p, sp)
         while eng.scheduler.queue or any(r.pending > 1 for r in eng.scheduler.live):
             eng.step()                                   # prefills (one prompt a step: budget = 2,048 tokens)
@@ -156,7 +175,9 @@ def main() -> int:
             assert len(outs) == batch
         torch.cuda.synchronize()
         step_s = (time.perf_counter() - t0) / steps
-        out = {"step_s": step_s, "context": prompt_len + warmup + steps // 2}
+        out = {"step_s": step_s, "context": prompt_tokens + warmup + steps // 2}
+        if context is not None:
+            out["bytes"], _ = account(lambda: eagerly(eng, eng.step))
         if detail:
             for _ in range(max(0, HISTOGRAM_STEPS - steps)):
                 eng.step()
@@ -310,6 +331,18 @@ def main() -> int:
                                       "frac": round(pre["flops"] / pre["s"] / profiling.PEAK_FLOPS_S[args.dtype], 4),
                                       "kernel_ms": pre.get("kernel_ms"), "kernels": pre.get("kernels")}}))
         return 0
+    if args.part == "decode" and sweep:
+        rows = {}
+        for ctx in sweep:
+            for b in [int(v) for v in args.batches.split(",")]:
+                d = time_decode(b, args.steps, args.warmup, context=ctx)
+                rows[f"b{b}_ctx{ctx}"] = {"tok_s": round(b / d["step_s"], 1), "ms_per_step": round(d["step_s"] * 1e3, 4),
+                                          "GB_per_step": round(d["bytes"] / 1e9, 3),
+                                          "hbm_frac": round(d["bytes"] / d["step_s"] / profiling.PEAK_HBM_BYTES_S, 4)}
+                print(f"b{b}_ctx{ctx}: {rows[f'b{b}_ctx{ctx}']}", file=sys.stderr, flush=True)
+        print(json.dumps({"metric": f"decode steps over long contexts ({shape_name})", "dtype": args.dtype, "steps": args.steps,
+                          "warmup": args.warmup, "rows": rows}))
+        return 0
     dec = time_decode(args.batch, args.steps, args.warmup, detail=True)
     step_s = dec["step_s"]
     value = args.batch / step_s
@@ -319,11 +352,17 @@ def main() -> int:
                           "gpu_idle_ms": dec.get("gpu_idle_ms"), "kernels": dec.get("kernels")}))
         return 0
     pre = time_prefill(detail=True)
-    points = {}
+    points, long_frac = {}, {}
     if not args.skip_points:
         for b in (1, 64):
             d = time_decode(b, max(16, args.steps // 2), max(4, args.warmup // 2))
             points[f"decode_b{b}"] = round(b / d["step_s"], 1)
+        for ctx in LONG_POINTS:                          # the headline batch over longer contexts, each against its own roofline
+            if ctx > most_positions:
+                continue
+            d = time_decode(args.batch, 16, 4, context=ctx)
+            points[f"decode_b{args.batch}_ctx{ctx}"] = round(args.batch / d["step_s"], 1)
+            long_frac[f"ctx{ctx}"] = round(d["bytes"] / d["step_s"] / profiling.PEAK_HBM_BYTES_S, 4)
     achieved = dec["bytes"] / step_s / 1e9
     peak_gbs = profiling.PEAK_HBM_BYTES_S / 1e9
     line = {
@@ -339,6 +378,7 @@ def main() -> int:
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": peak_gbs, "unit": "GB/s",
                      "frac": round(achieved / peak_gbs, 4)},
         "points": points,
+        "long_context_hbm_frac": long_frac,
         "step_ms": dec["step_ms"],
         "decode_kernel_ms": dec.get("kernel_ms"), "decode_gpu_idle_ms": dec.get("gpu_idle_ms"),
         "decode_kernels": dec.get("kernels"),

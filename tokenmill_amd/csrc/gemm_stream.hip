@@ -391,9 +391,11 @@ static void stream_config(int n_units, int ksteps, int tiles, int* ks, int* us) 
         return;
     }
     // From the matrix alone (KS fixes the order of a token's sums). Measured on an MI355X at the 0.5B and 7B layer
-    // sizes, 32 and 64 tokens: gate|up 7B (1,184 units) 2 x 2: 55 / 71 us (2 x 4: 62 / 75, 4 x 2: 56 / 79, 8 x 1: 72 / 111);
-    // gate|up 0.5B (304 units) 4 x 2: 9 / 12 us; q|k|v 7B (144 units) 8 x 1: 17 / 25 us (4 x 2: 20 / 27).
-    if (n_units >= 1024) { *ks = 2; *us = 2; }
+    // sizes, 32 / 48 / 64 tokens: gate|up 7B (1,184 units) 1 x 4: 60 / 67 / 68 us (2 x 2: 57 / 68 / 76, 2 x 4: 63 / 65 / 79,
+    // 4 x 2: 56 / 74 / 81, 8 x 1: 72 / - / 111), gate|up 32B (1,728 units) 1 x 4: 96 / 103 / 109 us = 5.9 / 5.5 / 5.2 TB/s
+    // (2 x 2: 110 / 117 / 130); gate|up 0.5B (304 units) 4 x 2: 9 / - / 12 us; q|k|v 7B (144 units) 8 x 1: 17 / - / 25 us
+    // (4 x 2: 20 / - / 27).
+    if (n_units >= 1024) { *ks = 1; *us = 4; }
     else if (n_units >= 256) { *ks = 4; *us = 2; }
     else { *ks = 8; *us = 1; }
     (void)ksteps;

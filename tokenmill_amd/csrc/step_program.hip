@@ -77,8 +77,8 @@ bool skinny_ok(const TmLinear& L, const void* x, int ldx, int dtype) {
     return dtype == TM_BF16 && L.dtype == TM_BF16 && L.K % 8 == 0 && ldx % 8 == 0 && aligned(x, 16) && aligned(L.w, 16);
 }
 
-bool panel_ok(const TmLinear& L, const void* x, int ldx, int M, int dtype) {
-    return L.packed && M > TM_SKINNY_ROWS && M <= TM_PANEL_ROWS && dtype == TM_BF16 && ldx % 8 == 0 && aligned(x, 16) &&
+bool panel_ok(const TmLinear& L, const void* x, int ldx, int M, int dtype, int most_rows = TM_PANEL_ROWS) {
+    return L.packed && M > TM_SKINNY_ROWS && M <= most_rows && dtype == TM_BF16 && ldx % 8 == 0 && aligned(x, 16) &&
            tm_gemm_panel_fits(M, L.K);
 }
 
@@ -298,7 +298,7 @@ struct Run {
                     xn = x;
                 }
                 // 2. the normed input kept in LDS (17 to 48 tokens)
-                if (tables_fusable && a.D % 32 == 0 && a.qkv.dtype == TM_BF16 && panel_ok(a.qkv, xn, hidden, T, dtype) &&
+                if (tables_fusable && a.D % 32 == 0 && a.qkv.dtype == TM_BF16 && panel_ok(a.qkv, xn, hidden, T, dtype, TM_PANEL_QKV_ROWS) &&
                     is_pow2(a.page) && bias_ok) {
                     rc = tm_panel_qkv_rope(xn, hidden, T, hidden, a.qkv.packed, a.qkv.bias, a.qkv.bias_dtype, qkv, a.H, a.KVH, a.D,
                                            a.cos_t, a.sin_t, s->positions, slots, kp, vp, a.page, stream);
