@@ -49,12 +49,23 @@ union Bf16x8Bits {
 };
 
 // The keys and values of 64 positions [wbase, wbase + 64) of one kv head as a wavefront holds them
-// between asking for them and using them: four 16-key tiles of MFMA operands.
+// between asking for them and using them: four tiles of 16 keys as MFMA operands.
+//
+// Which 16 keys make a tile is chosen for the loads of the values. A lane of the second product needs, for
+// 32 keys at a time, 8 keys of one row d of V^T, and it must be the 8 keys whose probabilities the lane got
+// from the first product's accumulators: 4 from each tile of a pair. With tiles of consecutive keys those are
+// 4 + 4 keys 16 apart: two 8-byte loads, and an instruction of the wavefront touches 32 bytes of each of 16
+// rows, which reads the pool at 3.9 TB/s at best. So the tiles of a pair (2b, 2b + 1) split their 32 keys in
+// runs of four: row rho of tile t is key 32 (t / 2) + 8 (rho / 4) + 4 (t % 2) + rho % 4. The lane that holds
+// rows 4g..4g+3 of both tiles then has the keys 32b + 8g .. + 7: one 16-byte load, 64 bytes of a row an
+// instruction (4.7 TB/s), and half as many loads. The keys are whole rows of the pool either way.
+__device__ __forceinline__ int tile_key(int t, int rho) { return 32 * (t / 2) + 8 * (rho / 4) + 4 * (t % 2) + rho % 4; }
+
 template <int D>
 struct Keys64 {
-    int tile_page[4];                       // page of each tile, -1 if no query may see it (wave-uniform)
-    Bf16x8Bits k[4][D / 32];
-    u32x2_t v[D / 16][4];
+    int group_page[4];                      // page of the 16 positions [wbase + 16 q, + 16), -1 if no query may see them (wave-uniform)
+    Bf16x8Bits k[4][D / 32];                // [tile][32 d]
+    u32x4_t v[D / 16][2];                   // [16 d][32 keys]: keys 32 b + 8 g .. + 7 of row d = 16 dt + r
 };
 
 // The block-table entries of the four 16-key tiles of [wbase, wbase + 64), read without a test at an
@@ -77,25 +88,32 @@ __device__ __forceinline__ void load_keys64(Keys64<D>& kv, const bf16_t* __restr
     constexpr int NDC = D / 32, NDT = D / 16;
     const int page_mask = (1 << page_shift) - 1;
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
-        const int tile0 = wbase + 16 * t;
-        kv.tile_page[t] = (tile0 < ctx && tile0 + 16 > lo) ? entry[t] : -1;                         // wave-uniform
+    for (int q = 0; q < 4; ++q) {
+        const int first = wbase + 16 * q;
+        kv.group_page[q] = (first < ctx && first + 16 > lo) ? entry[q] : -1;                        // wave-uniform
     }
     // Every load is unconditional, so that none of them has to be waited for before the next is
-    // issued: a tile nobody may see reads page 0 instead, and keys beyond the context read the rest of
+    // issued: positions nobody may see read page 0 instead, and keys beyond the context read the rest of
     // their page. What such loads bring is never used: their scores are replaced by -inf and their
     // values are masked bit by bit.
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-        const int tile0 = wbase + 16 * t;
-        const int in_page = tile0 & page_mask;
-        const size_t pg = kv.tile_page[t] >= 0 ? (size_t)kv.tile_page[t] : 0;
-        const bf16_t* kr = k_pool + (((pg << page_shift) + in_page + r) * KVH + kvh) * D + 8 * g;
-        const bf16_t* vr = v_pool + (((pg * KVH + kvh) * D + r) << page_shift) + in_page + 4 * g;
+        // the 16 positions of a row's key: the pair's first 16 for rows 0..7, its second 16 for rows 8..15
+        const int key = wbase + tile_key(t, r);
+        const int page = r < 8 ? kv.group_page[2 * (t / 2)] : kv.group_page[2 * (t / 2) + 1];
+        const size_t pg = page >= 0 ? (size_t)page : 0;
+        const bf16_t* kr = k_pool + (((pg << page_shift) + (key & page_mask)) * KVH + kvh) * D + 8 * g;
 #pragma unroll
         for (int c = 0; c < NDC; ++c) kv.k[t][c].u = *(const u32x4_t*)(kr + 32 * c);
+    }
 #pragma unroll
-        for (int dt = 0; dt < NDT; ++dt) kv.v[dt][t] = *(const u32x2_t*)(vr + ((size_t)(16 * dt) << page_shift));
+    for (int b = 0; b < 2; ++b) {
+        const int key = wbase + 32 * b + 8 * g;                      // this lane's 8 keys of the pair
+        const int page = g < 2 ? kv.group_page[2 * b] : kv.group_page[2 * b + 1];
+        const size_t pg = page >= 0 ? (size_t)page : 0;
+        const bf16_t* vr = v_pool + (((pg * KVH + kvh) * D + r) << page_shift) + (key & page_mask);
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt) kv.v[dt][b] = *(const u32x4_t*)(vr + ((size_t)(16 * dt) << page_shift));
     }
     // nothing that uses the keys may be scheduled above the loads of the values: both are on their
     // way before the first wait
@@ -109,7 +127,7 @@ __device__ __forceinline__ void attend_keys64(const Keys64<D>& kv, const Bf16x8B
                                               int lo, float scale_log2, int g, float& m, float& l,
                                               f32x4_t (&o)[D / 16]) {
     constexpr int NDC = D / 32, NDT = D / 16;
-    float sc[4][4];                                                 // [16-key tile][key 4g+i] for head r
+    float sc[4][4];                                                 // [tile][row 4g+i of the tile] for head r
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
         f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
@@ -118,7 +136,7 @@ __device__ __forceinline__ void attend_keys64(const Keys64<D>& kv, const Bf16x8B
             acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kv.k[t][c].b, qreg[c].b, acc, 0, 0, 0);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const int kj = wbase + 16 * t + 4 * g + i;
+            const int kj = wbase + tile_key(t, 4 * g + i);
             sc[t][i] = (kj < ctx && kj >= lo) ? acc[i] * scale_log2 : -INFINITY;
         }
     }
@@ -149,22 +167,18 @@ __device__ __forceinline__ void attend_keys64(const Keys64<D>& kv, const Bf16x8B
         Bf16x8Bits pt;
         pt.u = u32x4_t{pack_bf16(pr[2 * b][0], pr[2 * b][1]), pack_bf16(pr[2 * b][2], pr[2 * b][3]),
                        pack_bf16(pr[2 * b + 1][0], pr[2 * b + 1][1]), pack_bf16(pr[2 * b + 1][2], pr[2 * b + 1][3])};
-        // which of this lane's 4 + 4 keys exist (a value beyond the context may hold anything)
+        // which of this lane's 8 keys exist (a value beyond the context may hold anything)
         uint32_t keep[4];
 #pragma unroll
-        for (int half = 0; half < 2; ++half) {
-            const int k0 = wbase + 16 * (2 * b + half) + 4 * g;
-#pragma unroll
-            for (int w2 = 0; w2 < 2; ++w2) {
-                const int ka = k0 + 2 * w2, kb = ka + 1;
-                keep[half * 2 + w2] = ((ka < ctx && ka >= lo) ? 0x0000ffffu : 0u) | ((kb < ctx && kb >= lo) ? 0xffff0000u : 0u);
-            }
+        for (int w2 = 0; w2 < 4; ++w2) {
+            const int ka = wbase + 32 * b + 8 * g + 2 * w2, kb = ka + 1;
+            keep[w2] = ((ka < ctx && ka >= lo) ? 0x0000ffffu : 0u) | ((kb < ctx && kb >= lo) ? 0xffff0000u : 0u);
         }
 #pragma unroll
         for (int dt = 0; dt < NDT; ++dt) {
             Bf16x8Bits vf;
-            vf.u = u32x4_t{kv.v[dt][2 * b][0] & keep[0], kv.v[dt][2 * b][1] & keep[1],
-                           kv.v[dt][2 * b + 1][0] & keep[2], kv.v[dt][2 * b + 1][1] & keep[3]};
+            vf.u = u32x4_t{kv.v[dt][b][0] & keep[0], kv.v[dt][b][1] & keep[1], kv.v[dt][b][2] & keep[2],
+                           kv.v[dt][b][3] & keep[3]};
             o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.b, pt.b, o[dt], 0, 0, 0);
         }
     }
