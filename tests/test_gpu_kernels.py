@@ -761,10 +761,16 @@ def tiles_for(lens, q_lens):
     return torch.tensor(tiles, dtype=torch.int32)
 
 
-@pytest.mark.parametrize("H,KVH,D,page", [(14, 2, 64, 16), (6, 1, 32, 16), (5, 5, 128, 32), (20, 1, 64, 16),
-                                           (8, 2, 96, 16), (4, 2, 64, 64)])
+# the two kernels: wavefronts that split a tile's key blocks (any group), and a tile's keys and values staged through
+# LDS for all heads of a kv head (groups up to 16: 2, 4 or 8 wavefronts a block, the last with a copy loop whose
+# trip count does not divide at head size 96)
+@pytest.mark.parametrize("H,KVH,D,page,shared", [
+    (14, 2, 64, 16, False), (6, 1, 32, 16, False), (5, 5, 128, 32, False), (20, 1, 64, 16, False), (8, 2, 96, 16, False),
+    (4, 2, 64, 64, False),
+    (14, 2, 128, 16, True), (10, 2, 128, 32, True), (24, 2, 96, 16, True), (12, 1, 128, 64, True), (14, 2, 64, 16, True),
+    (6, 1, 32, 16, True), (4, 2, 64, 64, True), (3, 3, 96, 32, True)])
 @pytest.mark.parametrize("window", [0, 40])
-def test_paged_attention_prefill_mfma(ops, H, KVH, D, page, window):
+def test_paged_attention_prefill_mfma(ops, H, KVH, D, page, shared, window):
     dt = torch.bfloat16
     lens = [2, 37, 130, 64, 5, 300, 33, 200]
     q_lens = [2, 37, 2, 64, 3, 45, 17, 200]      # whole prompts and portions that start and end mid-page
@@ -780,7 +786,7 @@ def test_paged_attention_prefill_mfma(ops, H, KVH, D, page, window):
     wide[:, :H * D] = case["q"].reshape(T, H * D).to(DEV)
     out = torch.full((T, H * D), 3.0, dtype=dt, device=DEV)
     ops.attn_prefill_mfma(wide, out, case["kp"].to(DEV), v_layout(case["vp"]).to(DEV), case["tables"].to(DEV),
-                          tiles_for(lens, q_lens).to(DEV), H, KVH, D, scale, window)
+                          tiles_for(lens, q_lens).to(DEV), H, KVH, D, scale, window, shared=shared)
     want = paged_truth(case, lens, q_lens, scale, dt, window or None).reshape(T, H * D)
     torch.testing.assert_close(out.float().cpu(), want, **tol(dt))
     if not window:                               # the last query of request 5 is carried by its far key 3
@@ -796,7 +802,8 @@ def test_paged_attention_prefill_mfma(ops, H, KVH, D, page, window):
     out2 = torch.empty(T, H * D, dtype=dt, device=DEV)
     t2 = torch.tensor([(s, first + j, min(16, 77 - j), j) for j in range(0, 77, 16)] +
                       [(s, first + 77 + j, min(16, 123 - j), 77 + j) for j in range(0, 123, 16)], dtype=torch.int32)
-    ops.attn_prefill_mfma(wide, out2, k_dev, v_dev, case["tables"].to(DEV), t2.to(DEV), H, KVH, D, scale, window)
+    ops.attn_prefill_mfma(wide, out2, k_dev, v_dev, case["tables"].to(DEV), t2.to(DEV), H, KVH, D, scale, window,
+                          shared=shared)
     assert torch.equal(out2[first:first + 200], out[first:first + 200])
 
 

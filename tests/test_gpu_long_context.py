@@ -111,9 +111,11 @@ def test_decode_attention_at_long_contexts(monkeypatch, H, KVH, D, page, one_blo
     assert torch.equal(out2, out[sub])
 
 
-@pytest.mark.parametrize("H,KVH,D,page", SHAPES)
+@pytest.mark.parametrize("H,KVH,D,page,shared", [shape + (False,) for shape in SHAPES] +
+                         [(7, 1, 128, 16, True), (10, 2, 128, 64, True), (9, 1, 96, 32, True), (14, 2, 64, 16, True)])
 @pytest.mark.parametrize("window", [0, 1000])
-def test_prefill_attention_at_long_contexts(H, KVH, D, page, window):
+def test_prefill_attention_at_long_contexts(H, KVH, D, page, shared, window):
+    """Both kernels (``shared``: the one that stages keys and values through LDS for the heads of a kv head)."""
     from tokenmill_amd.hip import ops
     dt = torch.bfloat16
     lens = [2048, 4096, 16384, 2050]
@@ -126,7 +128,8 @@ def test_prefill_attention_at_long_contexts(H, KVH, D, page, window):
     wide[:, :H * D] = case["q"].reshape(T, H * D).to(DEV)
     out = torch.full((T, H * D), 3.0, dtype=dt, device=DEV)
     kp, vp, tables = case["kp"].to(DEV), v_layout(case["vp"]).to(DEV), case["tables"].to(DEV)
-    ops.attn_prefill_mfma(wide, out, kp, vp, tables, tiles_for(lens, q_lens).to(DEV), H, KVH, D, scale, window)
+    ops.attn_prefill_mfma(wide, out, kp, vp, tables, tiles_for(lens, q_lens).to(DEV), H, KVH, D, scale, window,
+                          shared=shared)
     want = truth_rows(case, lens, q_lens, scale, dt, window or None).reshape(T, H * D)
     got = out.float().cpu()
     torch.testing.assert_close(got, want, **bf16_tol())
@@ -136,7 +139,7 @@ def test_prefill_attention_at_long_contexts(H, KVH, D, page, window):
     out2 = torch.empty(T, H * D, dtype=dt, device=DEV)
     t2 = torch.tensor([(0, j, min(16, 1000 - j), j) for j in range(0, 1000, 16)] +
                       [(0, 1000 + j, min(16, 1048 - j), 1000 + j) for j in range(0, 1048, 16)], dtype=torch.int32)
-    ops.attn_prefill_mfma(wide, out2, kp, vp, tables, t2.to(DEV), H, KVH, D, scale, window)
+    ops.attn_prefill_mfma(wide, out2, kp, vp, tables, t2.to(DEV), H, KVH, D, scale, window, shared=shared)
     assert torch.equal(out2[:2048], out[:2048])
 
 

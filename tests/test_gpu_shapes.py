@@ -157,6 +157,10 @@ def test_the_measured_configuration_against_the_plain_implementation(layer_model
             assert (48 if n_requests == 40 else 8) in eng.runner.graphs.buckets
         eng.cache.check_invariants()
         assert eng.cache.num_free_pages == eng.cache.num_pages
+        took = eng.runner.program.counters()
+        if "chunked" not in what:                 # whole prompts of 2,100 and more tokens: the attention that shares a
+            # tile's keys among the seven heads of a kv head at head size 128, the one that splits them at 64
+            assert (took["prefill_shared_keys"] > 0) == (name == "7B") and (took["prefill_split_keys"] > 0) == (name != "7B")
         del eng
         torch.cuda.empty_cache()
     # Up to 16 rows every kernel fixes its order of additions by the sizes alone: padding a step to its bucket

@@ -95,6 +95,13 @@ int tm_attn_prefill_mfma(const void* q, int q_stride, void* out, int out_stride,
                          const void* v_pool, const int* block_tables, int table_width, const int* tiles, int n_tiles,
                          int H, int KVH, int D, int page, float scale, int window, hipStream_t stream);
 
+// The same attention with the keys and values of a tile staged through LDS once for all query heads of a kv
+// head (attention_prefill_shared.hip); same operands, out rows 8-byte aligned.
+int tm_attn_prefill_shared(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
+                           const void* v_pool, const int* block_tables, int table_width, const int* tiles, int n_tiles,
+                           int H, int KVH, int D, int page, float scale, int window, hipStream_t stream);
+int tm_attn_prefill_shared_takes(int H, int KVH, int D);
+
 int tm_gemv_f32(const float* A, int lda, const float* W, const float* bias, float* C, int ldc, int M, int N, int K,
                 hipStream_t stream);
 

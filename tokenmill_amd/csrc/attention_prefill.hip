@@ -17,27 +17,7 @@
 //                    B = P^T   [32 keys x 16 tokens] straight from the S^T accumulators
 #include "common.h"
 #include "api.h"
-
-#define PF_SLACK 8.f        // how far (log2 units) a score may exceed the running reference before it moves
-
-typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
-typedef float f32x4_t __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
-
-union PFrag {
-    u32x4_t u;
-    bf16x8_t b;
-};
-
-typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-typedef float f32x2_t __attribute__((ext_vector_type(2)));
-
-// two floats -> packed bfloat16 (round to nearest even, one instruction on gfx950)
-__device__ __forceinline__ uint32_t pk_bf16(float a, float b) {
-    const bf16x2_t v = __builtin_convertvector(f32x2_t{a, b}, bf16x2_t);
-    return *(const uint32_t*)&v;
-}
+#include "attention_prefill_common.h"
 
 template <int D>
 struct KVBlock {
@@ -93,39 +73,6 @@ __device__ __forceinline__ void load_kv_block(KVBlock<D>& blk, int2 pages, int s
     }
 }
 
-// max(a, b, c) in the nesting the compiler turns into one three-operand maximum. A two-operand
-// maximum of values whose origin it cannot see (matrix-unit results, lane swaps) costs it an extra
-// instruction per operand (it first makes signalling NaNs quiet); the three-operand form does not,
-// so the reductions below are chains of these, started from a constant.
-__device__ __forceinline__ float max3(float a, float b, float c) { return fmaxf(fmaxf(a, b), c); }
-
-// maximum over the four lanes (r, 0..3) that hold one query column
-__device__ __forceinline__ float column_max(float v) {
-    const uint32_t u = __float_as_uint(v);
-    const auto a = __builtin_amdgcn_permlane32_swap(u, u, false, false);     // lanes l and l ^ 32
-    const float m32 = max3(-INFINITY, __uint_as_float(a[0]), __uint_as_float(a[1]));
-    const uint32_t w = __float_as_uint(m32);
-    const auto b = __builtin_amdgcn_permlane16_swap(w, w, false, false);     // lanes l and l ^ 16
-    return max3(-INFINITY, __uint_as_float(b[0]), __uint_as_float(b[1]));
-}
-
-// Running softmax state of the query heads a wavefront works on.
-//   m: running maximum of (score * scale * log2 e) of this lane's column; l: this lane's share of
-//   the running sum (its 8 keys of every block), reduced over the lanes of a column at the end
-template <int D, int HPW>
-struct HeadState {
-    float m[HPW], l[HPW];
-    f32x4_t o[HPW][D / 16];
-};
-
-// What a wavefront knows about the tile it works on (all wave-uniform but my_pos and my_lo).
-struct TileView {
-    int pos0;               // position of the tile's first query
-    int last_key;           // newest key any query of the tile sees
-    int last_lo;            // oldest key the tile's last query sees (0 without a window)
-    int my_pos, my_lo;      // this lane's query column: its position and the oldest key it sees
-};
-
 // One block of 32 keys against the wavefront's heads.
 template <int D, int HPW>
 __device__ __forceinline__ void attend_block(KVBlock<D>& blk, HeadState<D, HPW>& st, const PFrag (&qf)[HPW][D / 32],
@@ -174,19 +121,22 @@ __device__ __forceinline__ void attend_block(KVBlock<D>& blk, HeadState<D, HPW>&
                     if (kj > tv.my_pos || kj < tv.my_lo) sc[hh][t][i] = -INFINITY;
                 }
         }
-        float bm = max3(-INFINITY, sc[hh][0][0], sc[hh][0][1]);
-        bm = max3(bm, sc[hh][0][2], sc[hh][0][3]);
-        bm = max3(bm, sc[hh][1][0], sc[hh][1][1]);
-        bm = max3(bm, sc[hh][1][2], sc[hh][1][3]);
-        bm = column_max(bm) * scale_log2;                        // scale > 0: the maximum commutes with it
+        // this lane's largest score of the block (scale > 0: the maximum commutes with it)
+        float lm = max3(-INFINITY, sc[hh][0][0], sc[hh][0][1]);
+        lm = max3(lm, sc[hh][0][2], sc[hh][0][3]);
+        lm = max3(lm, sc[hh][1][0], sc[hh][1][1]);
+        lm = max3(lm, sc[hh][1][2], sc[hh][1][3]);
         // The running reference m of a column moves only when the block's maximum exceeds it by more
         // than PF_SLACK (in units of log2): until then the weights are exp2(s - m) <= 2^PF_SLACK instead of
         // <= 1, which changes nothing but their common scale (it cancels against the sum), and the
         // rescaling of the accumulators, the expensive part of a block on the vector unit, becomes rare.
         // Each column decides for itself and one that stays multiplies by exactly 1, so a query's result
-        // does not depend on the other queries of its tile.
-        const bool grow = bm > st.m[hh] + PF_SLACK;              // (true for a column that has seen no key: m = -inf)
-        if (__any(grow)) {
+        // does not depend on the other queries of its tile. Whether any column moves is asked of the lanes'
+        // own maxima first (a column's maximum exceeds the limit exactly when one of its four lanes' does), so
+        // the exchange between the lanes of a column is as rare as the rescaling.
+        if (__any(lm * scale_log2 > st.m[hh] + PF_SLACK)) {          // (true for a column that has seen no key: m = -inf)
+            const float bm = column_max(lm) * scale_log2;
+            const bool grow = bm > st.m[hh] + PF_SLACK;
             const float m_new = grow ? bm : st.m[hh];
             const float corr = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(st.m[hh] - m_new);
             st.m[hh] = m_new;

@@ -33,3 +33,14 @@ inline int tm_decode_chunks(int max_context) { return (max_context + TM_DECODE_C
 inline bool tm_decode_splits(int requests, int kv_heads, int max_context) {
     return requests * kv_heads < TM_DECODE_SPLIT_PAIRS && tm_decode_chunks(max_context) > 1;
 }
+
+// --- prefill attention (bfloat16) ---------------------------------------------------------------------
+// Two kernels: one whose wavefronts each load their own key blocks and split a tile's keys among them (many
+// short chains: best for short prompts and for small head sizes), and one that stages a tile's keys and values
+// through LDS once for all query heads of a kv head (twice the rate at head sizes above 64 from about a thousand
+// tokens on, where the first is held back by one wavefront a SIMD). The second needs at least three wavefronts'
+// worth of heads (two heads a wavefront) to fill a CU, and a launch of at least a block a CU.
+inline bool tm_prefill_shares_keys(int D, int H, int KVH, int n_tiles) {
+    const int G = H / KVH;
+    return D > 64 && G >= 5 && G <= 16 && (long long)n_tiles * KVH >= 256;
+}

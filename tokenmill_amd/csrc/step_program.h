@@ -97,13 +97,15 @@ struct TmProgram;
 // how an operation was computed, counted per program (tm_program_counters fills TM_PROGRAM_COUNTERS numbers)
 enum {
     TM_QKV_FROM_NORM = 0,       // q|k|v by the kernel that starts at the norm (at most 16 tokens)
-    TM_QKV_PANEL,               // ... by the kernel that keeps the normed input in LDS (17 to 48 tokens)
+    TM_QKV_PANEL,               // ... by the kernel that keeps the normed input in LDS (17 to 64 tokens)
     TM_QKV_STREAM,              // ... by the kernel that streams the packed matrix for up to 64 tokens
     TM_QKV_PLAIN,               // ... by a product, then rotation and cache write
     TM_GATE_UP_FROM_NORM,
     TM_GATE_UP_PANEL,
     TM_GATE_UP_STREAM,
     TM_GATE_UP_PLAIN,           // a product with the SiLU*up epilogue, or a product and then SiLU*up
+    TM_PREFILL_SPLIT_KEYS,      // bfloat16 attention of prompt portions: wavefronts split a tile's key blocks
+    TM_PREFILL_SHARED_KEYS,     // ... a tile's keys and values staged through LDS for all heads of a kv head
     TM_PROGRAM_COUNTERS
 };
 void tm_program_counters(const TmProgram* p, long long* out);

@@ -335,8 +335,16 @@ struct Run {
             const bool q_ok = aligned(q, 16) && q_stride % 8 == 0;
             bool done_prefill = false, done_decode = false;
             if (tp && s->n_tiles > 0 && s->prefill_tiles && dtype == TM_BF16 && head_mfma && page_ok && q_ok) {
-                rc = tm_attn_prefill_mfma(q, q_stride, attn, HD, a.k_pool, a.v_pool, tables, W, s->prefill_tiles, s->n_tiles, a.H,
-                                          a.KVH, a.D, a.page, a.scale, a.window, stream);
+                if (tm_prefill_shares_keys(a.D, a.H, a.KVH, s->n_tiles) && tm_attn_prefill_shared_takes(a.H, a.KVH, a.D) &&
+                    HD % 4 == 0 && aligned(attn, 8)) {
+                    ++p->taken[TM_PREFILL_SHARED_KEYS];
+                    rc = tm_attn_prefill_shared(q, q_stride, attn, HD, a.k_pool, a.v_pool, tables, W, s->prefill_tiles,
+                                                s->n_tiles, a.H, a.KVH, a.D, a.page, a.scale, a.window, stream);
+                } else {
+                    ++p->taken[TM_PREFILL_SPLIT_KEYS];
+                    rc = tm_attn_prefill_mfma(q, q_stride, attn, HD, a.k_pool, a.v_pool, tables, W, s->prefill_tiles,
+                                              s->n_tiles, a.H, a.KVH, a.D, a.page, a.scale, a.window, stream);
+                }
                 done_prefill = true;
             } else if (tp && s->n_tiles > 0 && s->prefill_tiles && dtype == TM_F32 && a.D % 16 == 0 && a.D >= 16 &&
                        a.D <= 128 && page_ok && q_stride % 4 == 0 && aligned(q, 16)) {

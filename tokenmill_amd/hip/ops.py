@@ -640,10 +640,12 @@ def attn_prefill_mfma_supported(dtype, H: int, KVH: int, D: int, page: int) -> b
 
 def attn_prefill_mfma(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                       block_tables: torch.Tensor, tiles: torch.Tensor, H: int, KVH: int, D: int, scale: float,
-                      window: int) -> torch.Tensor:
+                      window: int, shared: bool = False) -> torch.Tensor:
     """Attention of prompt portions over the cache. q: [T, >= H*D] rows, out [T, H*D]; tiles int32
     [n, 4] = (request index, first row, tokens (1..16), position of the first token) cover the rows
-    to compute; every row of a tile belongs to one request at consecutive positions."""
+    to compute; every row of a tile belongs to one request at consecutive positions. ``shared``: the kernel
+    that stages a tile's keys and values through LDS for all heads of a kv head, instead of the one whose
+    wavefronts split the key blocks (each kernel alone, in tests; a step's choice is the library's)."""
     _gpu(q, out, k_pool, v_pool, block_tables, tiles)
     T = q.shape[0]
     page = _check_pools(k_pool, v_pool, KVH, D, torch.bfloat16, "attn_prefill")
@@ -658,10 +660,15 @@ def attn_prefill_mfma(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, 
           "attn_prefill: block_tables must be contiguous int32 [S, W]")
     _need(tiles.dtype == torch.int32 and tiles.dim() == 2 and tiles.shape[1] == 4 and tiles.is_contiguous(),
           "attn_prefill: tiles must be contiguous int32 [n, 4]")
-    _check(library().tm_attn_prefill_mfma(_p(q), c_int(q_stride), _p(out), c_int(out_stride), _p(k_pool), _p(v_pool),
-                                          _p(block_tables), c_int(block_tables.shape[1]), _p(tiles),
-                                          c_int(tiles.shape[0]), c_int(H), c_int(KVH), c_int(D), c_int(page),
-                                          c_float(scale), c_int(window), _stream()), "attn_prefill_mfma")
+    if shared:
+        _need(bool(library().tm_attn_prefill_shared_takes(c_int(H), c_int(KVH), c_int(D))) and out_stride % 4 == 0
+              and out.data_ptr() % 8 == 0, "attn_prefill: the shared-keys kernel takes up to 16 query heads a kv head "
+              "and out rows aligned to 8 bytes")
+    entry = library().tm_attn_prefill_shared if shared else library().tm_attn_prefill_mfma
+    _check(entry(_p(q), c_int(q_stride), _p(out), c_int(out_stride), _p(k_pool), _p(v_pool),
+                 _p(block_tables), c_int(block_tables.shape[1]), _p(tiles),
+                 c_int(tiles.shape[0]), c_int(H), c_int(KVH), c_int(D), c_int(page),
+                 c_float(scale), c_int(window), _stream()), "attn_prefill_shared" if shared else "attn_prefill_mfma")
     return out
 
 
