@@ -97,7 +97,10 @@ struct StageCopy {
         }
     }
 
-    __device__ __forceinline__ void store(unsigned char* stage, int tid) const {
+    // Store what was loaded into a stage of LDS. `keys` of the stage's 64 positions exist: the values of the
+    // others (beyond the newest key; they can hold anything) are cleared here, once for all wavefronts, so that
+    // the products need no mask (their weights are zero, but zero times anything is not).
+    __device__ __forceinline__ void store(unsigned char* stage, int tid, int keys) const {
 #pragma unroll
         for (int i = 0; i < ITERS; ++i) {
             const int idx = tid + i * THREADS;
@@ -105,7 +108,14 @@ struct StageCopy {
             const int kk = idx / (D / 8), pc = idx % (D / 8);
             *(u32x4_t*)(stage + stage_row(kk) * SharedShape<D>::K_STRIDE + pc * 16) = k[i];
             const int j = idx / (2 * D), d = (idx % (2 * D)) / 2, half = idx & 1;
-            *(u32x4_t*)(stage + SharedShape<D>::K_BYTES + d * SharedShape<D>::V_STRIDE + j * 32 + half * 16) = v[i];
+            u32x4_t val = v[i];
+            if (keys < PS_KEYS) {                                    // block-uniform: a tile's last stage only
+                const int first = 16 * j + 8 * half;
+#pragma unroll
+                for (int w = 0; w < 4; ++w)
+                    val[w] &= ((first + 2 * w < keys) ? 0x0000ffffu : 0u) | ((first + 2 * w + 1 < keys) ? 0xffff0000u : 0u);
+            }
+            *(u32x4_t*)(stage + SharedShape<D>::K_BYTES + d * SharedShape<D>::V_STRIDE + j * 32 + half * 16) = val;
         }
     }
 };
@@ -113,7 +123,7 @@ struct StageCopy {
 // 32 keys [key0, key0 + 32) of the stage in LDS against the wavefront's heads.
 template <int D, int HPW>
 __device__ __forceinline__ void attend_shared(const unsigned char* stage, int sub, HeadState<D, HPW>& st,
-                                              const PFrag (&qf)[HPW][D / 32], int key0, int nh, const TileView& tv,
+                                              const PFrag (&qf)[HPW][D / 32], int key0, const TileView& tv,
                                               int r, int g, float scale_log2) {
     constexpr int NDC = D / 32, NDT = D / 16;
     constexpr int KS = SharedShape<D>::K_STRIDE, VS = SharedShape<D>::V_STRIDE;
@@ -128,7 +138,6 @@ __device__ __forceinline__ void attend_shared(const unsigned char* stage, int su
     PFrag pt[HPW];
 #pragma unroll
     for (int hh = 0; hh < HPW; ++hh) {
-        if (hh >= nh) continue;                                  // wave-uniform
         f32x4_t sc[2];
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
@@ -183,24 +192,12 @@ __device__ __forceinline__ void attend_shared(const unsigned char* stage, int su
         pt[hh].u = u32x4_t{pk_bf16(pr[0][0], pr[0][1]), pk_bf16(pr[0][2], pr[0][3]), pk_bf16(pr[1][0], pr[1][1]),
                            pk_bf16(pr[1][2], pr[1][3])};
     }
-    // values of keys nobody may see (beyond the newest key) can hold anything: clear them
-    const bool tail = key0 + 31 > tv.last_key;
-    uint32_t keep[4] = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};
-    if (tail) {
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-            const int ka = key0 + 8 * g + 2 * w;
-            keep[w] = ((ka <= tv.last_key) ? 0x0000ffffu : 0u) | ((ka + 1 <= tv.last_key) ? 0xffff0000u : 0u);
-        }
-    }
 #pragma unroll
     for (int dt = 0; dt < NDT; ++dt) {
         PFrag vf;
         vf.u = *(const u32x4_t*)(stage + SharedShape<D>::K_BYTES + (16 * dt + r) * VS + 64 * sub + 16 * g);
-        if (tail) vf.u = u32x4_t{vf.u[0] & keep[0], vf.u[1] & keep[1], vf.u[2] & keep[2], vf.u[3] & keep[3]};
 #pragma unroll
         for (int hh = 0; hh < HPW; ++hh) {
-            if (hh >= nh) continue;                              // wave-uniform
             st.o[hh][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.b, pt[hh].b, st.o[hh][dt], 0, 0, 0);
         }
     }
@@ -272,7 +269,7 @@ __global__ __launch_bounds__(64 * WAVES, SharedPlan<D>::WAVES_PER_SIMD) void att
         TilePlaces places = lane_places(base, lane, first_tile, last_tile, table, page_shift, kvh, KVH, D);
         StageCopy<D, THREADS> copy;
         copy.load(places, 0, kp, vp, KVH, page_shift, tid);
-        copy.store(stages, tid);
+        copy.store(stages, tid, tv.last_key + 1 - sb0 * PS_KEYS);
         __syncthreads();
         for (int sb = sb0; sb <= sb1; ++sb) {
             const int cur = (sb - sb0) & 1;
@@ -287,10 +284,10 @@ __global__ __launch_bounds__(64 * WAVES, SharedPlan<D>::WAVES_PER_SIMD) void att
                 for (int sub = 0; sub < 2; ++sub) {
                     const int key0 = sb * PS_KEYS + 32 * sub;
                     if (key0 > tv.last_key || key0 + 31 < first_key) continue;     // block-uniform: nothing of it is visible
-                    attend_shared<D, HPW>(stages + cur * STAGE, sub, st, qf, key0, nh, tv, r, g, scale_log2);
+                    attend_shared<D, HPW>(stages + cur * STAGE, sub, st, qf, key0, tv, r, g, scale_log2);
                 }
             }
-            copy.store(stages + (cur ^ 1) * STAGE, tid);
+            copy.store(stages + (cur ^ 1) * STAGE, tid, tv.last_key + 1 - next * PS_KEYS);
             __syncthreads();
         }
 
