@@ -127,10 +127,11 @@ def _long_prompts(n_requests: int, seed: int) -> list[list[int]]:
     return [random_ids(n, 1000, seed + i) for i, n in enumerate(lengths)]
 
 
-@pytest.mark.parametrize("name,n_requests,n_checked", [("0.5B", 8, 8), ("0.5B", 40, 6), ("7B", 8, 2), ("7B", 40, 3)])
+@pytest.mark.parametrize("name,n_requests,n_checked", [("0.5B", 8, 8), ("0.5B", 40, 6), ("7B", 8, 2), ("7B", 40, 3),
+                                                       ("32B", 8, 2)])
 def test_the_measured_configuration_against_the_plain_implementation(layer_models, name, n_requests, n_checked):
     """What the headline benchmark runs (reference tests/test_gpu.py:132-149 compares its graph path with its eager
-    one at the real model): bfloat16 engines at the layer sizes of the 0.5B and 7B shapes with max_model_len 4,096,
+    one at the real model): bfloat16 engines at the layer sizes of the 0.5B, 7B and 32B shapes with max_model_len 4,096,
     decode steps replayed from HIP graphs over contexts above 2,048 keys (the split attention inside the graph at
     8 requests, the one-block attention and the 48-row bucket's products at 40), once with the library's
     algorithms chosen by timing and the prompts cut into portions. Tokens are checked against the plain
@@ -159,8 +160,8 @@ def test_the_measured_configuration_against_the_plain_implementation(layer_model
         assert eng.cache.num_free_pages == eng.cache.num_pages
         took = eng.runner.program.counters()
         if "chunked" not in what:                 # whole prompts of 2,100 and more tokens: the attention that shares a
-            # tile's keys among the seven heads of a kv head at head size 128, the one that splits them at 64
-            assert (took["prefill_shared_keys"] > 0) == (name == "7B") and (took["prefill_split_keys"] > 0) == (name != "7B")
+            # tile's keys among the seven (five) heads of a kv head at head size 128, the one that splits them at 64
+            assert (took["prefill_shared_keys"] > 0) == (name != "0.5B") and (took["prefill_split_keys"] > 0) == (name == "0.5B")
         del eng
         torch.cuda.empty_cache()
     # Up to 16 rows every kernel fixes its order of additions by the sizes alone: padding a step to its bucket
