@@ -805,6 +805,12 @@ def test_paged_attention_prefill_mfma(ops, H, KVH, D, page, shared, window):
     ops.attn_prefill_mfma(wide, out2, k_dev, v_dev, case["tables"].to(DEV), t2.to(DEV), H, KVH, D, scale, window,
                           shared=shared)
     assert torch.equal(out2[first:first + 200], out[first:first + 200])
+    # a launch of many tiles (the same ones again and again, as a padded step's table holds them): at head sizes up to
+    # 64 a wavefront of the split-keys kernel then takes four heads instead of two, and a head's bits stay
+    out3 = torch.empty(T, H * D, dtype=dt, device=DEV)
+    ops.attn_prefill_mfma(wide, out3, k_dev, v_dev, case["tables"].to(DEV), t2.repeat(40, 1).to(DEV), H, KVH, D, scale,
+                          window, shared=shared)
+    assert torch.equal(out3[first:first + 200], out2[first:first + 200])
 
 
 @pytest.mark.parametrize("H,KVH,D,page", [(14, 2, 64, 16), (6, 1, 32, 16), (5, 5, 128, 32), (3, 1, 48, 16), (8, 2, 80, 64),

@@ -18,6 +18,7 @@
 #include "common.h"
 #include "api.h"
 #include "attention_prefill_common.h"
+#include "choose.h"
 
 template <int D>
 struct KVBlock {
@@ -300,8 +301,25 @@ __global__ __launch_bounds__(64 * KS) void attn_prefill_mfma_kernel(
     }
 }
 
-// heads a wavefront takes and wavefronts a block has, by head size (registers decide)
+// Heads a wavefront takes and wavefronts a block has, by head size (registers decide). Up to head size 64 a
+// wavefront can hold four heads, which quarters the loads of a long prompt's keys; a short step, whose blocks of
+// two heads a wavefront still fit the chip in one round, takes those instead: twice the blocks, half as long
+// (512 tokens at the 0.5B shape: 13.4 to 9.8 us; a head's arithmetic is the same either way, so its bits are).
 template <int D> struct PrefillShape { static constexpr int HPW = D <= 64 ? 4 : 2, KS = D <= 64 ? 8 : 4; };
+
+template <int D, int HPW>
+static void launch_split_keys(const void* q, int q_stride, void* out, int out_stride, const void* k_pool, const void* v_pool,
+                              const int* block_tables, int table_width, const int* tiles, int n_tiles, int H, int KVH,
+                              int page_shift, float scale_log2, int window, hipStream_t stream) {
+    constexpr int KS = PrefillShape<D>::KS;
+    const int splits = (H / KVH + HPW - 1) / HPW;
+    // fold the table in two once the folded launch still gives every CU a block
+    const int pair = (long long)(n_tiles / 2) * KVH * splits >= 256 ? 1 : 0;
+    dim3 grid(pair ? (n_tiles + 1) / 2 : n_tiles, KVH * splits);
+    attn_prefill_mfma_kernel<D, HPW, KS><<<grid, 64 * KS, 0, stream>>>(
+        (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, block_tables,
+        table_width, tiles, n_tiles, pair, H, KVH, page_shift, scale_log2, window);
+}
 
 extern "C" int tm_attn_prefill_mfma(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
                                     const void* v_pool, const int* block_tables, int table_width, const int* tiles,
@@ -316,17 +334,16 @@ extern "C" int tm_attn_prefill_mfma(const void* q, int q_stride, void* out, int 
     int page_shift = 0;
     while ((1 << page_shift) < page) ++page_shift;
     const float scale_log2 = scale * 1.4426950408889634f;
+    if ((long long)KVH * ((G + 1) / 2) > 65535) return TM_ERR_ARG;
+#define TM_SPLIT_ARGS q, q_stride, out, out_stride, k_pool, v_pool, block_tables, table_width, tiles, n_tiles, H, KVH, \
+                      page_shift, scale_log2, window, stream
 #define TM_PREFILL_CASE(DD)                                                                                       \
     case DD: {                                                                                                    \
-        constexpr int HPW = PrefillShape<DD>::HPW, KS = PrefillShape<DD>::KS;                                     \
-        const int splits = (G + HPW - 1) / HPW;                                                                   \
-        if ((long long)KVH * splits > 65535) return TM_ERR_ARG;                                                   \
-        /* fold the table in two once the folded launch still gives every CU a block */                          \
-        const int pair = (long long)(n_tiles / 2) * KVH * splits >= 256 ? 1 : 0;                                  \
-        dim3 grid(pair ? (n_tiles + 1) / 2 : n_tiles, KVH * splits);                                              \
-        attn_prefill_mfma_kernel<DD, HPW, KS><<<grid, 64 * KS, 0, stream>>>(                                      \
-            (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool,   \
-            block_tables, table_width, tiles, n_tiles, pair, H, KVH, page_shift, scale_log2, window);             \
+        constexpr int HPW = PrefillShape<DD>::HPW;                                                                \
+        if (HPW > 2 && G > 2 && (long long)n_tiles * KVH * ((G + 1) / 2) <= TM_PREFILL_ONE_ROUND)                 \
+            launch_split_keys<DD, 2>(TM_SPLIT_ARGS);                                                              \
+        else                                                                                                      \
+            launch_split_keys<DD, HPW>(TM_SPLIT_ARGS);                                                            \
         break;                                                                                                    \
     }
     switch (D) {
@@ -338,6 +355,7 @@ extern "C" int tm_attn_prefill_mfma(const void* q, int q_stride, void* out, int 
             return TM_ERR_ARG;
     }
 #undef TM_PREFILL_CASE
+#undef TM_SPLIT_ARGS
     TM_CHECK_LAUNCH();
     return TM_OK;
 }

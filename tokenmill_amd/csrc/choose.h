@@ -44,3 +44,7 @@ inline bool tm_prefill_shares_keys(int D, int H, int KVH, int n_tiles) {
     const int G = H / KVH;
     return D > 64 && G >= 5 && G <= 16 && (long long)n_tiles * KVH >= 256;
 }
+
+// The split-keys kernel at head sizes up to 64 takes two heads a wavefront instead of four while the blocks that
+// gives are no more than the chip runs at once (one a CU).
+constexpr int TM_PREFILL_ONE_ROUND = 256;

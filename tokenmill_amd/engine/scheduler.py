@@ -180,6 +180,8 @@ class Scheduler:
             if set_aside_prompts and req.pending > 1:
                 partway.append(req)
                 continue
+            # outside mixed steps a live request has run its whole prompt (a step that fails ends its requests)
+            assert req.pending == 1, f"request {req.id} is live with {req.pending} tokens pending"
             grown = self.cache.try_append(req.cache, req.n_tokens)
             while not grown:
                 unserved_end -= 1                       # live[unserved_end] is the newest not yet served
