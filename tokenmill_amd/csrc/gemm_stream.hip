@@ -382,14 +382,7 @@ __global__ __launch_bounds__(64 * KS * US) void gemm_stream_kernel(const StreamA
 // the matrix's shape alone (never from the number of tokens: that keeps a token's sums in one order). Many units
 // (gate|up): the units share, K is split little; few units over a long K (the down projection): K is split over
 // the whole block, so that the chip still has a few thousand wavefronts streaming.
-static int g_stream_force_ks = 0, g_stream_force_us = 0;            // set by tm_stream_force, for measurements
-
 static void stream_config(int n_units, int ksteps, int tiles, int* ks, int* us) {
-    if (g_stream_force_ks) {
-        *ks = g_stream_force_ks;
-        *us = g_stream_force_us;
-        return;
-    }
     // From the matrix alone (KS fixes the order of a token's sums). Measured on an MI355X at the 0.5B and 7B layer
     // sizes, 32 / 48 / 64 tokens: gate|up 7B (1,184 units) 1 x 4: 60 / 67 / 68 us (2 x 2: 57 / 68 / 76, 2 x 4: 63 / 65 / 79,
     // 4 x 2: 56 / 74 / 81, 8 x 1: 72 / - / 111), gate|up 32B (1,728 units) 1 x 4: 96 / 103 / 109 us = 5.9 / 5.5 / 5.2 TB/s
@@ -400,16 +393,6 @@ static void stream_config(int n_units, int ksteps, int tiles, int* ks, int* us) 
     else { *ks = 8; *us = 1; }
     (void)ksteps;
     (void)tiles;
-}
-
-// For measurements: every later stream product runs with ks x us wavefronts a block (0, 0: the rule again).
-extern "C" int tm_stream_force(int ks, int us) {
-    const bool known = (ks == 0 && us == 0) || (ks == 2 && us == 4) || (ks == 4 && us == 2) || (ks == 8 && us == 1) ||
-                       (ks == 4 && us == 1) || (ks == 2 && us == 2) || (ks == 1 && us == 4);
-    if (!known) return TM_ERR_ARG;
-    g_stream_force_ks = ks;
-    g_stream_force_us = us;
-    return TM_OK;
 }
 
 template <int EPI, int NT, int KS, int US>
@@ -431,12 +414,9 @@ template <int EPI, int NT>
 static int launch_stream_tiles(const StreamArgs& a, int n_units, int kparts, hipStream_t stream) {
     int ks = 0, us = 0;
     stream_config(n_units * kparts, (a.f.K + 31) / 32 / kparts, NT, &ks, &us);
-    switch (ks * 16 + us) {
-        case 2 * 16 + 4: return launch_stream_config<EPI, NT, 2, 4>(a, n_units, kparts, stream);
+    switch (ks * 16 + us) {                     // the shapes stream_config names
         case 4 * 16 + 2: return launch_stream_config<EPI, NT, 4, 2>(a, n_units, kparts, stream);
         case 8 * 16 + 1: return launch_stream_config<EPI, NT, 8, 1>(a, n_units, kparts, stream);
-        case 4 * 16 + 1: return launch_stream_config<EPI, NT, 4, 1>(a, n_units, kparts, stream);
-        case 2 * 16 + 2: return launch_stream_config<EPI, NT, 2, 2>(a, n_units, kparts, stream);
         default: return launch_stream_config<EPI, NT, 1, 4>(a, n_units, kparts, stream);
     }
 }
@@ -519,15 +499,7 @@ extern "C" int tm_stream_linear(const void* X, int ldx, int M, int K, const void
 
 // Groups of blocks a plain product's K is split over: enough that a matrix with few rows still has a few thousand
 // wavefronts streaming it, each with a few rounds of k-steps to itself. From the matrix's shape alone.
-static int g_stream_force_parts = 0;                                // set by tm_stream_force_parts, for measurements
-extern "C" int tm_stream_force_parts(int parts) {
-    if (parts < 0 || parts > 8) return TM_ERR_ARG;
-    g_stream_force_parts = parts;
-    return TM_OK;
-}
-
 extern "C" int tm_stream_linear_parts(int N, int K) {
-    if (g_stream_force_parts) return g_stream_force_parts;
     // The fewest groups (a power of two, at most 8) that give the matrix about 400 blocks, as long as a wavefront (of
     // the four that split a block's share of K) keeps four k-steps to itself. Measured on an MI355X, 32 and 64 rows:
     // 7B down (112 units, K 18,944) 4 groups: 30 / 39 us against 56 / 81 us unsplit and 52 / 69 us for the library's
