@@ -23,11 +23,14 @@ __global__ __launch_bounds__(256) void gemm_nt_tiled_kernel(const TA* __restrict
     const int tid = threadIdx.x;
     const int tx = tid % 16, ty = tid / 16;
     const int m0 = blockIdx.y * GT_BM, n0 = blockIdx.x * GT_BN;
-    float acc[4][4];
+    // the sum over K in blocks of 128: a block's sum is taken by itself and then joins the total (one chain of
+    // additions over all of K loses sqrt(K) roundings' worth of accuracy, blocks lose the chain of a block and then
+    // the chain of the blocks); where the blocks end depends on K alone
+    float acc[4][4], total[4][4];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+        for (int j = 0; j < 4; ++j) acc[i][j] = total[i][j] = 0.f;
 
     for (int k0 = 0; k0 < K; k0 += GT_BK) {
 #pragma unroll
@@ -56,6 +59,15 @@ __global__ __launch_bounds__(256) void gemm_nt_tiled_kernel(const TA* __restrict
 #pragma unroll
                 for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], w[j], acc[i][j]);
         }
+        if ((k0 / GT_BK + 1) % 8 == 0 || k0 + GT_BK >= K) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    total[i][j] += acc[i][j];
+                    acc[i][j] = 0.f;
+                }
+        }
         __syncthreads();
     }
 #pragma unroll
@@ -66,7 +78,7 @@ __global__ __launch_bounds__(256) void gemm_nt_tiled_kernel(const TA* __restrict
         for (int j = 0; j < 4; ++j) {
             const int n = n0 + tx * 4 + j;
             if (n >= N) continue;
-            float v = acc[i][j];
+            float v = total[i][j];
             if (bias) v += Elem<TB>::load(bias + n);
             Elem<TC>::store(C + (size_t)m * ldc + n, v);
         }
