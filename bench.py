@@ -57,6 +57,8 @@ def main() -> int:
                     help="tokens of every prompt: the prefill's length and the context the decode steps start from")
     ap.add_argument("--config", default=None, help="a config.json or a shipped shape's name (7b, 32b): run it instead of the 0.5B shape")
     ap.add_argument("--no-graphs", action="store_true", help="launch decode steps kernel by kernel")
+    ap.add_argument("--no-pipeline", action="store_true",
+                    help="read a decode step's tokens before the next step is queued (as without --pipeline-decode)")
     ap.add_argument("--no-tune", action="store_true", help="keep the library's first choice of matrix-product algorithm")
     ap.add_argument("--tune-every", action="store_true",
                     help="captured shapes also try every algorithm the library holds, not only its heuristic's candidates")
@@ -78,6 +80,7 @@ def main() -> int:
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+    pipelined = not args.no_pipeline and not args.no_graphs
     if args.part == "mixed7b":
         args.config = args.config or "7b"
     if args.part == "preempt32b":
@@ -127,8 +130,15 @@ def main() -> int:
         pages = batch * (-(-(prompt_len + args.steps + args.warmup + extra_steps + 64) // BLOCK_SIZE)) + 8
         cfg = EngineConfig(dtype=args.dtype, block_size=BLOCK_SIZE, num_blocks=pages, max_model_len=max_model_len,
                            max_num_seqs=max(batch, 1), max_num_batched_tokens=max(prompt_len, batch),
-                           watermark=0.0, hip_graphs=not args.no_graphs, tune_gemm=not args.no_tune, tune_gemm_every=args.tune_every and not args.no_tune)
+                           watermark=0.0, hip_graphs=not args.no_graphs, tune_gemm=not args.no_tune, tune_gemm_every=args.tune_every and not args.no_tune,
+                           pipeline_decode=pipelined)
         return LLMEngine(cfg, model=model)
+
+    def settle(eng):
+        """From here on the engine's steps run one at a time: the step in flight is finished and none is queued
+        ahead any more (what is measured after this is a single step by itself)."""
+        eng.cfg.pipeline_decode = False
+        eng.flush()
 
     def account(fn) -> tuple[float, float]:
         """(bytes, flops) the parts say the device work of ``fn`` has to move and do."""
@@ -177,6 +187,7 @@ def main() -> int:
         step_s = (time.perf_counter() - t0) / steps
         out = {"step_s": step_s, "context": prompt_tokens + warmup + steps // 2}
         if context is not None:
+            settle(eng)
             out["bytes"], _ = account(lambda: eagerly(eng, eng.step))
         if detail:
             for _ in range(max(0, HISTOGRAM_STEPS - steps)):
@@ -184,6 +195,7 @@ def main() -> int:
             times = [1e3 * t for t in eng.step_seconds]
             out["step_ms"] = {"p50": round(percentile(times, 0.5), 4), "p90": round(percentile(times, 0.9), 4),
                               "max": round(max(times), 4), "n": len(times)}
+            settle(eng)
             out["bytes"], _ = account(lambda: eagerly(eng, eng.step))
             if not args.skip_kernels:
                 out.update(trace_decode(eng, step_s))
@@ -256,7 +268,8 @@ def main() -> int:
         cfg = EngineConfig(dtype=args.dtype, block_size=BLOCK_SIZE, num_blocks=args.offline_seqs * per_seq + 64,
                            max_model_len=max_model_len, max_num_seqs=args.offline_seqs, max_num_batched_tokens=2048,
                            enable_chunked_prefill=args.chunked, hip_graphs=not args.no_graphs,
-                           tune_gemm=not args.no_tune, tune_gemm_every=args.tune_every and not args.no_tune)
+                           tune_gemm=not args.no_tune, tune_gemm_every=args.tune_every and not args.no_tune,
+                           pipeline_decode=pipelined)
         eng = LLMEngine(cfg, model=model)
         sp = SamplingParams(max_tokens=args.offline_gen, ignore_eos=True)
         serve(eng, prompts(min(n, 2 * args.offline_seqs), args.offline_prompt), sp)
@@ -272,7 +285,8 @@ def main() -> int:
         pages = seqs * (-(-(4096 + gen_tokens) // BLOCK_SIZE)) + 64
         cfg = EngineConfig(dtype=args.dtype, block_size=BLOCK_SIZE, num_blocks=pages, max_model_len=max_model_len,
                            max_num_seqs=seqs, max_num_batched_tokens=budget, enable_chunked_prefill=True,
-                           hip_graphs=not args.no_graphs, tune_gemm=not args.no_tune, tune_gemm_every=args.tune_every and not args.no_tune)
+                           hip_graphs=not args.no_graphs, tune_gemm=not args.no_tune, tune_gemm_every=args.tune_every and not args.no_tune,
+                           pipeline_decode=pipelined)
         eng = LLMEngine(cfg, model=model)
         sp = SamplingParams(max_tokens=gen_tokens, ignore_eos=True)
         serve(eng, [prompts(1, L)[0] for L in lengths[:8]], SamplingParams(max_tokens=8, ignore_eos=True))    # warm-up
@@ -297,7 +311,8 @@ def main() -> int:
         n, gen_tokens, pages = args.requests or 64, 64, 8192
         cfg = EngineConfig(dtype=args.dtype, block_size=BLOCK_SIZE, num_blocks=pages, max_model_len=max_model_len,
                            max_num_seqs=n, max_num_batched_tokens=2048, watermark=0.0,
-                           hip_graphs=not args.no_graphs, tune_gemm=not args.no_tune, tune_gemm_every=args.tune_every and not args.no_tune)
+                           hip_graphs=not args.no_graphs, tune_gemm=not args.no_tune, tune_gemm_every=args.tune_every and not args.no_tune,
+                           pipeline_decode=pipelined)
         eng = LLMEngine(cfg, model=model)
         sp = SamplingParams(max_tokens=gen_tokens, ignore_eos=True)
         serve(eng, prompts(2), SamplingParams(max_tokens=4, ignore_eos=True))                                 # warm-up
@@ -372,7 +387,7 @@ def main() -> int:
         "dtype": "bf16" if dtype == torch.bfloat16 else "fp32", "data": "synthetic token ids, random weights",
         "config": {**sizes(), "global_batch": args.batch, "seq_len": prompt_len, "context": dec["context"],
                    "max_model_len": max_model_len, "block_size": BLOCK_SIZE, "parallelism": "single GPU",
-                   "hip_graphs": not args.no_graphs, "tune_gemm": ("every" if args.tune_every else True) if not args.no_tune else False, "packed_weights": True},
+                   "hip_graphs": not args.no_graphs, "tune_gemm": ("every" if args.tune_every else True) if not args.no_tune else False, "packed_weights": True, "pipeline_decode": pipelined},
         "prefill": {"value": round(prompt_len / pre["s"], 1), "tokens": prompt_len, "ms": round(pre["s"] * 1e3, 3),
                     "frac": round(pre["flops"] / pre["s"] / profiling.PEAK_FLOPS_S[args.dtype], 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": peak_gbs, "unit": "GB/s",

@@ -686,3 +686,101 @@ def test_the_step_program_refuses_what_its_kernels_do_not_run(model_dirs):
     assert torch.equal(program.run(step), want)                            # and nothing of this broke the program
     session.manager.free(cache)
 
+
+
+# ------------------------------------------------------------------------------------------------
+# decode steps queued ahead of their tokens
+# ------------------------------------------------------------------------------------------------
+
+def _both(model_dir, dtype_name, run, **kw):
+    """``run(engine)`` on an engine that reads every step's tokens before it plans the next, and on one that queues
+    decode steps ahead; both results."""
+    results = []
+    for ahead in (False, True):
+        eng = make_engine(model_dir, dtype_name, hip_graphs=True, pipeline_decode=ahead, **kw)
+        results.append((run(eng), eng))
+    return results
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_decode_steps_queued_ahead_give_the_same_tokens(model_dirs, plains, dtype_name):
+    """With ``pipeline_decode`` the next decode step is queued behind the running one, its ids fed on the device:
+    requests that end by length at different steps, pages crossed every 16 tokens, and requests that end at an
+    end-of-sequence token after the step ahead of them was queued (their extra token is dropped): the same tokens
+    as the engine that waits for every step, and they are the plain implementation's."""
+    from tokenmill_amd import SamplingParams
+    dt = {"float32": torch.float32, "bfloat16": torch.bfloat16}[dtype_name]
+    prompts = [random_ids(n, 256, 300 + i) for i, n in enumerate((5, 17, 33, 30, 12))]
+    limits = [3, 40, 64, 17, 50]
+
+    def by_length(eng):
+        return eng.generate(prompts, [SamplingParams(max_tokens=m, ignore_eos=True) for m in limits])
+
+    (plain_out, waiting), (ahead_out, ahead) = _both(model_dirs["A"], dtype_name, by_length)
+    assert ahead_out == plain_out and [len(o) for o in ahead_out] == limits
+    assert ahead.stats["steps_ahead"] > 30 and waiting.stats["steps_ahead"] == 0
+    for p, o in zip(prompts, ahead_out):
+        verify(plains["A"], p, o, dt)
+    # now one of those tokens ends requests: one that no request meets before its 7th token (by then the request with
+    # three tokens is gone and steps are queued ahead) and some request meets well before its limit
+    def first_met(tok):
+        return min((o.index(tok) for o in ahead_out if tok in o), default=10 ** 6)
+    stops = {next(o[j] for o, m in zip(ahead_out, limits) for j in range(6, m - 4) if first_met(o[j]) == j)}
+
+    def by_stop_token(eng):
+        eng.eos_ids = set(stops)
+        return eng.generate(prompts, [SamplingParams(max_tokens=m) for m in limits])
+
+    (plain_out, waiting), (ahead_out, ahead) = _both(model_dirs["A"], dtype_name, by_stop_token)
+    assert ahead_out == plain_out
+    assert any(o[-1] in stops and len(o) < m for o, m in zip(ahead_out, limits))
+    assert ahead.stats["tokens_dropped"] > 0 and waiting.stats["tokens_dropped"] == 0, (ahead.stats, [len(o) for o in ahead_out])
+    for eng in (waiting, ahead):
+        eng.cache.check_invariants()
+        assert eng.cache.num_free_pages == eng.cache.num_pages
+
+
+def test_decode_steps_queued_ahead_with_sampling_arrivals_aborts_and_few_pages(model_dirs, plains):
+    """The same with sampled tokens (the random number of a token is a function of the request's seed and the token's
+    index, which the step ahead knows), with requests that arrive and are aborted while a step is in flight, with
+    prompts cut into portions, and on a pool so small that requests are evicted: nothing is queued ahead where the
+    next step is not simply the same requests one position on, and every request's tokens are as without it."""
+    from tokenmill_amd import SamplingParams
+    prompts = [random_ids(n, 256, 400 + i) for i, n in enumerate((9, 21, 40, 33, 14, 27))]
+    sampled = [SamplingParams(max_tokens=24, temperature=0.8, top_k=40, top_p=0.9, seed=50 + i, ignore_eos=True)
+               for i in range(len(prompts))]
+    (a, _), (b, ahead) = _both(model_dirs["A"], "float32", lambda eng: eng.generate(prompts, sampled))
+    assert a == b and ahead.stats["steps_ahead"] > 10
+    for p, o, sp in zip(prompts, b, sampled):
+        verify(plains["A"], p, o, torch.float32, sp, sp.seed)
+
+    def arrivals_and_an_abort(eng):
+        got: dict[str, list[int]] = {}
+        sp = SamplingParams(max_tokens=30, ignore_eos=True)
+        for i in range(3):
+            eng.add_request(f"r{i}", prompts[i], sp)
+        calls = 0
+        while eng.has_unfinished():
+            for o in eng.step():
+                got.setdefault(o.request_id, []).extend(o.new_token_ids)
+            calls += 1
+            if calls == 6:
+                eng.add_request("late", prompts[3], sp)
+            if calls == 11:
+                eng.abort_request("r1")
+        got.pop("r1")                                  # ended at a call, not at a token: how far it got differs
+        return got
+
+    (a, _), (b, ahead) = _both(model_dirs["A"], "float32", arrivals_and_an_abort, enable_chunked_prefill=True,
+                               max_num_batched_tokens=16)
+    assert a == b and set(b) == {"r0", "r2", "late"} and all(len(t) == 30 for t in b.values())
+    assert ahead.stats["steps_ahead"] > 10
+    ahead.cache.check_invariants()
+    assert ahead.cache.num_free_pages == ahead.cache.num_pages
+
+    greedy = SamplingParams(max_tokens=40, ignore_eos=True)
+    (a, waiting), (b, ahead) = _both(model_dirs["A"], "float32", lambda eng: eng.generate(prompts, greedy),
+                                     kv_cache_mb=None, num_blocks=14)
+    assert a == b and waiting.scheduler.evictions > 0 and ahead.scheduler.evictions > 0
+    ahead.cache.check_invariants()
+    assert ahead.cache.num_free_pages == ahead.cache.num_pages

@@ -13,16 +13,18 @@ import logging
 import random
 import time
 from collections import deque
+from dataclasses import dataclass
 
 from tokenmill_amd.cache.manager import CacheManager
 from tokenmill_amd.cache.pool import CachePools
 from tokenmill_amd.config.engine_config import EngineConfig
 from tokenmill_amd.engine.loading import load_model, resolve_device, resolve_dtype
 from tokenmill_amd.engine.request import Request, RequestOutput
-from tokenmill_amd.engine.runner import ModelRunner
+from tokenmill_amd.engine.request import Phase
+from tokenmill_amd.engine.runner import ModelRunner, StepEntry
 from tokenmill_amd.engine.scheduler import Scheduler, StepPlan
 from tokenmill_amd.engine.sizing import num_cache_pages
-from tokenmill_amd.sampling.sampler import Sampler, SamplingParams
+from tokenmill_amd.sampling.sampler import Drawn, Sampler, SamplingParams
 
 log = logging.getLogger("tokenmill_amd.engine")
 
@@ -34,6 +36,15 @@ DOES_NOT_FIT = "prompt does not fit in the KV cache"
 
 class RequestRejected(ValueError):
     """The request can never be served as given (empty, too long, a token outside the vocabulary, an id in use)."""
+
+
+@dataclass
+class _InFlight:
+    """A step that has been queued on the GPU and whose tokens have not been read yet."""
+    plan: StepPlan
+    winners: list[Request]
+    drawn: Drawn | None              # None: no entry of the step yields a token
+    ahead: bool = False              # queued behind the step before it, before that step's tokens were known
 
 
 class LLMEngine:
@@ -65,8 +76,9 @@ class LLMEngine:
         self.requests: dict[str, Request] = {}           # every request that has not ended
         self._seeds = random.Random(cfg.seed)            # stream seeds of requests that bring none
         self._generate_calls = 0
+        self._in_flight: _InFlight | None = None         # with pipeline_decode: the step queued by the call before
         self.stats = {"steps": 0, "prompt_steps": 0, "decode_steps": 0, "mixed_steps": 0, "tokens_out": 0,
-                      "tokens_in": 0, "busy_s": 0.0, "peak_live": 0}
+                      "tokens_in": 0, "busy_s": 0.0, "peak_live": 0, "steps_ahead": 0, "tokens_dropped": 0}
         self.step_seconds: deque[float] = deque(maxlen=STEP_TIMES_KEPT)
         log.info("engine ready: %d pages of %d tokens per layer group (%.0f MiB), %s on %s", pages, cfg.block_size,
                  self.pools.nbytes / 2**20, self.dtype, self.device)
@@ -123,6 +135,8 @@ class LLMEngine:
     # --- one step -----------------------------------------------------------------------------------
 
     def step(self) -> list[RequestOutput]:
+        """One step's outputs. With ``pipeline_decode`` the step whose outputs these are was queued by the call
+        before, and this call queues the next one behind it before it waits for its tokens."""
         started = time.perf_counter()
         out: list[RequestOutput] = []
         if self.cfg.request_timeout:
@@ -132,41 +146,120 @@ class LLMEngine:
             for req in [r for r in self.requests.values() if r.expires and r.t_arrived < too_old]:
                 self._end(req, "timeout", time.monotonic())
                 out.append(RequestOutput(req, []))
-        plan = self.scheduler.plan()
-        for req in plan.unfit:
-            # an evicted request that has grown past the pool ends with what it has; a fresh one with an error
-            self._end(req, "length", time.monotonic(), None if req.n_generated else DOES_NOT_FIT)
-            out.append(RequestOutput(req, []))
-        if not plan:
-            return out
+        flight, self._in_flight = self._in_flight, None
+        if flight is None:
+            plan = self.scheduler.plan()
+            for req in plan.unfit:
+                # an evicted request that has grown past the pool ends with what it has; a fresh one with an error
+                self._end(req, "length", time.monotonic(), None if req.n_generated else DOES_NOT_FIT)
+                out.append(RequestOutput(req, []))
+            if not plan:
+                return out
+            flight = self._launch(plan)
+        ahead = self._launch_ahead(flight) if self.cfg.pipeline_decode else None
+        try:
+            out.extend(self._finish(flight, started))
+        except BaseException:
+            if ahead is not None:                     # queued behind a step that failed: what it computed is void
+                self._fail(ahead.plan, RuntimeError("the step before this one failed"))
+            raise
+        self._in_flight = ahead
+        return out
+
+    def flush(self) -> list[RequestOutput]:
+        """The outputs of the step that is in flight (with ``pipeline_decode``: queued by the last call), if any, without
+        queueing another behind it: after this the GPU holds no work of the engine's."""
+        flight, self._in_flight = self._in_flight, None
+        return self._finish(flight, time.perf_counter()) if flight is not None else []
+
+    def _fail(self, plan: StepPlan, e: BaseException) -> None:
+        """The step did not run to its end, so what the cache holds for its requests is unknown: they end
+        here with the error and give their pages back (the reference's loop ends every request in
+        flight with the error and goes on serving, reference src/infer/engine/engine.py:342-349).
+        Requests that were not part of the step are untouched."""
+        now = time.monotonic()
+        for req in dict.fromkeys(plan.owners):
+            if req.phase is Phase.LIVE:
+                self._end(req, "error", now, f"{type(e).__name__}: {e}")
+
+    def _launch(self, plan: StepPlan) -> _InFlight:
+        """Queue the plan's step and the sampling of its tokens; nothing is waited for."""
         winners = [plan.owners[i] for i in plan.yields]
         try:
             logits = self.runner.step(plan.entries)
-            tokens = self.sampler.sample(logits, [r.params for r in winners], [r.stream_seed for r in winners],
-                                         [r.n_generated for r in winners]) if winners else []
+            drawn = self.sampler.start(logits, [r.params for r in winners], [r.stream_seed for r in winners],
+                                       [r.n_generated for r in winners]) if winners else None
         except Exception as e:
-            # The step did not run to its end, so what the cache holds for its requests is unknown: they end
-            # here with the error and give their pages back (the reference's loop ends every request in
-            # flight with the error and goes on serving, reference src/infer/engine/engine.py:342-349).
-            # Requests that were not part of the step are untouched.
-            now = time.monotonic()
-            for req in dict.fromkeys(plan.owners):
-                self._end(req, "error", now, f"{type(e).__name__}: {e}")
+            self._fail(plan, e)
+            raise
+        return _InFlight(plan, winners, drawn)
+
+    def _launch_ahead(self, flight: _InFlight) -> _InFlight | None:
+        """While ``flight`` runs: queue the step after it, if that step is known without ``flight``'s tokens but for
+        their values. That is so when ``flight`` is a decode step of requests that all go on unless they meet an
+        end-of-sequence token (none reaches its ``max_tokens`` or the model's length with this token), nobody waits
+        to be admitted, and every request has a page for its next position: then the next step is the same requests,
+        one position on, and the ids go from the sampler's output to the step's input on the device. A request that
+        does end at an end-of-sequence token has then run one token too many; it is dropped when that step's tokens
+        are read. None: the next step is planned the usual way, after ``flight``'s tokens."""
+        plan = flight.plan
+        n = len(plan.entries)
+        if (flight.drawn is None or plan.n_decode != n or len(plan.yields) != n or self.scheduler.queue
+                or self.runner.graphs is None):
+            return None
+        limit = self.cfg.max_model_len
+        for req in plan.owners:
+            if (req.phase is not Phase.LIVE or req.n_generated + 1 >= req.params.max_tokens or req.n_tokens + 1 >= limit):
+                return None
+        for req in plan.owners:
+            if not self.cache.try_append(req.cache, req.n_tokens + 1):
+                return None
+        # flight's token is not in req.tokens yet: it will sit at position req.cached + 1 = req.n_tokens
+        entries = [StepEntry(req.cache, req.cached + 1, [0], [0]) for req in plan.owners]
+        try:
+            logits = self.runner.step_behind(entries, flight.drawn.device)
+            if logits is None:
+                return None
+            owners = list(plan.owners)
+            drawn = self.sampler.start(logits, [r.params for r in owners], [r.stream_seed for r in owners],
+                                       [r.n_generated + 1 for r in owners])
+        except Exception as e:                        # nothing of it counts; the usual way takes over
+            log.warning("no step queued ahead (%s: %s)", type(e).__name__, e)
+            return None
+        self.stats["steps_ahead"] += 1
+        return _InFlight(StepPlan(entries=entries, owners=owners, yields=list(range(n)), n_decode=n), owners, drawn,
+                         ahead=True)
+
+    def _finish(self, flight: _InFlight, started: float) -> list[RequestOutput]:
+        """Wait for the step's tokens and advance its requests. A request that ended since the step was queued (an
+        end-of-sequence token in the step before a step queued ahead, an abort, a timeout) is passed over: its
+        row's token is dropped."""
+        plan, out = flight.plan, []
+        try:
+            tokens = flight.drawn.tokens() if flight.drawn is not None else []
+        except Exception as e:
+            self._fail(plan, e)
             raise
         now = time.monotonic()
         release = self.cache.release_behind_window
         for req, entry in zip(plan.owners, plan.entries):
-            req.cached += len(entry.tokens)
-            release(req.cache, req.cached)
-        for req, token in zip(winners, tokens):
+            if req.phase is Phase.LIVE and req.cache is entry.cache:
+                req.cached += len(entry.tokens)
+                release(req.cache, req.cached)
+        n_out = 0
+        for req, token in zip(flight.winners, tokens):
+            if req.phase is not Phase.LIVE:
+                self.stats["tokens_dropped"] += 1
+                continue
             req.tokens.append(token)
+            n_out += 1
             if req.t_first_token is None:
                 req.t_first_token = now
             why = self._why_stop(req, token)
             if why is not None:
                 self._end(req, why, now)
             out.append(RequestOutput(req, [token]))
-        self._account(plan, len(tokens), time.perf_counter() - started)
+        self._account(plan, n_out, time.perf_counter() - started)
         return out
 
     def _why_stop(self, req: Request, token: int) -> str | None:

@@ -107,11 +107,13 @@ class DecodeGraphs:
         return self.buckets[B]
 
     @torch.inference_mode()
-    def run(self, entries) -> torch.Tensor | None:
+    def run(self, entries, ids_from: torch.Tensor | None = None) -> torch.Tensor | None:
         """Float32 logits [wanted, vocab], entries in the given order (each wants place 0 or nothing); None
         if the graph of this batch size could not be captured (the caller then runs the step kernel by
         kernel, as the reference does when it runs out of memory for graphs: reference
-        src/infer/engine/cuda_graphs.py:88-110)."""
+        src/infer/engine/cuda_graphs.py:88-110). With ``ids_from`` (int32 on the device, one id per entry) the
+        entries' tokens are taken from there, in stream order, instead of from the entries: the step before this
+        one may still be running, and what it samples goes into this one without a trip to the host."""
         runner = self.runner
         bk = self._bucket(len(entries))
         B, W, page = bk.B, bk.W, self.page
@@ -159,6 +161,8 @@ class DecodeGraphs:
                 rows[i] = None
         bk.dev.copy_(bk.pinned, non_blocking=True)
         self._copied.record()
+        if ids_from is not None:
+            bk.view(bk.ids)[:n].copy_(ids_from[:n])
         if bk.graph is None:
             if bk.B in self.failed:
                 return None

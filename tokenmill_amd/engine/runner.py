@@ -307,6 +307,17 @@ class ModelRunner:
         ctx, _ = self.prepare(entries)
         return self.forward(ctx)
 
+    def step_behind(self, entries: list[StepEntry], ids_from: torch.Tensor) -> torch.Tensor | None:
+        """A step of single tokens queued behind the step whose sampled ids ``ids_from`` holds on the device (one per
+        entry, in the entries' order; the entries' own ``tokens`` are placeholders). Only as a graph replay: None if
+        this batch has no graph, and nothing was queued then."""
+        if self.graphs is None or not self.graphs.can_run(entries) or any(e.cache.fresh for e in entries):
+            return None
+        bucket = self.graphs._bucket(len(entries))
+        if bucket.graph is None:                  # a capture runs the step outside the graph first: not behind another
+            return None
+        return self.graphs.run(entries, ids_from=ids_from)
+
     def forward(self, step: StepContext, about_to_be_captured: bool = False) -> torch.Tensor:
         """The step's float32 logits [R, vocab], by the model's step program."""
         return self.program.run(step, at_once=about_to_be_captured)

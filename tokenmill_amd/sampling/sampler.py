@@ -51,27 +51,65 @@ def uniform_from_counter(seed: int, index: int) -> float:
     return (_mix(_mix(z)) >> 40) / float(1 << 24)
 
 
+class Drawn:
+    """The tokens of one step's rows, on their way to the host: ``device`` holds them (int32 [R]) in stream order,
+    ``tokens()`` waits for the copy that was asked for behind them and returns them as a list."""
+
+    def __init__(self, device: torch.Tensor, host: torch.Tensor, copied: torch.cuda.Event):
+        self.device, self._host, self._copied = device, host, copied
+
+    def tokens(self) -> list[int]:
+        self._copied.synchronize()
+        return self._host[:self.device.shape[0]].tolist()
+
+
 class Sampler:
+    HOST_BUFFERS = 4          # pinned buffers for the tokens' way back, used in turn (two steps can be in flight)
+
     def __init__(self, device):
         self.device = device
+        self._host: list[torch.Tensor] = []
+        self._turn = 0
+
+    def _host_buffer(self, rows: int) -> torch.Tensor:
+        """A pinned buffer for ``rows`` tokens; the one whose last use is the longest ago."""
+        i = self._turn % self.HOST_BUFFERS
+        self._turn += 1
+        if len(self._host) <= i:
+            self._host.append(torch.empty(max(rows, 256), dtype=torch.int32, pin_memory=True))
+        elif self._host[i].numel() < rows:
+            self._host[i] = torch.empty(rows, dtype=torch.int32, pin_memory=True)
+        return self._host[i]
 
     @torch.inference_mode()
     def sample(self, logits: torch.Tensor, params: list[SamplingParams], seeds: list[int],
                counters: list[int]) -> list[int]:
         """logits float32 [R, V] on the GPU; one token per row. ``counters[r]`` is the index of the
         token being generated for row r's request."""
-        R = logits.shape[0]
-        if R == 0:
+        if logits.shape[0] == 0:
             return []
-        with profiling.label("sample", lambda: (logits.numel() * 4, 0)):
-            return self._sample(logits, params, seeds, counters)
+        return self.start(logits, params, seeds, counters).tokens()
 
-    def _sample(self, logits, params, seeds, counters) -> list[int]:
+    @torch.inference_mode()
+    def start(self, logits: torch.Tensor, params: list[SamplingParams], seeds: list[int],
+              counters: list[int]) -> Drawn:
+        """As ``sample``, without waiting: the kernels and the copy to the host are queued, and the caller asks
+        the returned ``Drawn`` for the tokens when it needs them (its ``device`` tensor can feed the next step
+        meanwhile)."""
+        with profiling.label("sample", lambda: (logits.numel() * 4, 0)):
+            out = self._sample(logits, params, seeds, counters)
+        host = self._host_buffer(out.shape[0])
+        host[:out.shape[0]].copy_(out, non_blocking=True)
+        copied = torch.cuda.Event()
+        copied.record()
+        return Drawn(out, host, copied)
+
+    def _sample(self, logits, params, seeds, counters) -> torch.Tensor:
         R = logits.shape[0]
         out = torch.empty(R, dtype=torch.int32, device=logits.device)
         if all(p.greedy for p in params):
             ops.argmax_rows(logits, out)
-            return out.tolist()
+            return out
         host = torch.empty((4, R), dtype=torch.float32, pin_memory=True)
         host[0] = torch.tensor([p.temperature for p in params])
         host[1] = torch.tensor([p.top_p for p in params])
@@ -84,4 +122,4 @@ class Sampler:
         ops.sample_rows(logits, dev[0], dev[3].view(torch.int32), dev[1], dev[2], out,
                         uses_top_k=any(not p.greedy and 0 < p.top_k < vocab for p in params),
                         uses_top_p=any(not p.greedy and p.top_p < 1.0 for p in params))
-        return out.tolist()
+        return out
