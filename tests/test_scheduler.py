@@ -200,6 +200,34 @@ def test_retire_gives_pages_back_wherever_the_request_stands():
     sim.cache.check_invariants()
 
 
+def test_nobody_can_join_says_when_the_next_plan_would_admit_nobody():
+    """What the engine asks before it queues a decode step ahead of the running one's tokens: with nobody waiting,
+    with every slot taken, and with a head of the queue that has to wait for pages, the next plan is the live requests
+    again; a free slot and pages for the head, the policy that counts decode steps while someone waits, and mixed steps
+    need a plan of their own."""
+    sim = Sim(pages=8, page=4, max_num_seqs=2)
+    assert sim.sched.nobody_can_join()
+    a, b = sim.request(6), sim.request(6)
+    assert not sim.sched.nobody_can_join()               # two slots, pages for the head
+    sim.step()
+    assert sim.sched.nobody_can_join()                   # nobody waits
+    c = sim.request(4)
+    assert sim.sched.nobody_can_join()                   # both slots taken
+    sim.sched.retire(b, "stop")
+    assert not sim.sched.nobody_can_join()               # a slot and 6 free pages for a prompt of one page
+    sim.sched.retire(c, "abort")
+    d = sim.request(26)                                  # 7 pages: one more than are free while a holds 2
+    assert sim.sched.nobody_can_join()
+    sim.sched.retire(a, "stop")
+    assert not sim.sched.nobody_can_join()
+    sim.sched.retire(d, "abort")
+    for options in (dict(policy="decode_first"), dict(enable_chunked_prefill=True)):
+        other = Sim(pages=8, page=4, max_num_seqs=1, **options)
+        other.request(4), other.request(4)
+        other.step()
+        assert not other.sched.nobody_can_join()         # the slot is taken, and still the plan has to be made
+
+
 def test_decode_first_makes_the_queue_wait():
     sim = Sim(pages=64, policy="decode_first", max_waiting_steps=3)
     a = sim.request(4)

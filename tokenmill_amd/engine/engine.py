@@ -197,15 +197,15 @@ class LLMEngine:
     def _launch_ahead(self, flight: _InFlight) -> _InFlight | None:
         """While ``flight`` runs: queue the step after it, if that step is known without ``flight``'s tokens but for
         their values. That is so when ``flight`` is a decode step of requests that all go on unless they meet an
-        end-of-sequence token (none reaches its ``max_tokens`` or the model's length with this token), nobody waits
-        to be admitted, and every request has a page for its next position: then the next step is the same requests,
+        end-of-sequence token (none reaches its ``max_tokens`` or the model's length with this token), nobody who waits
+        could be admitted now, and every request has a page for its next position: then the next step is the same requests,
         one position on, and the ids go from the sampler's output to the step's input on the device. A request that
         does end at an end-of-sequence token has then run one token too many; it is dropped when that step's tokens
         are read. None: the next step is planned the usual way, after ``flight``'s tokens."""
         plan = flight.plan
         n = len(plan.entries)
-        if (flight.drawn is None or plan.n_decode != n or len(plan.yields) != n or self.scheduler.queue
-                or self.runner.graphs is None):
+        if (flight.drawn is None or plan.n_decode != n or len(plan.yields) != n or self.runner.graphs is None
+                or len(self.scheduler.live) != n or not self.scheduler.nobody_can_join()):
             return None
         limit = self.cfg.max_model_len
         for req in plan.owners:

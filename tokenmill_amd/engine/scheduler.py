@@ -97,6 +97,18 @@ class Scheduler:
     def busy(self) -> bool:
         return bool(self.queue) or bool(self.live)
 
+    def nobody_can_join(self) -> bool:
+        """Would the next plan, made now, admit nobody? True when nobody waits; and, for the policy that admits
+        whenever it can, when every slot of a live request is taken or the head of the queue has to wait for pages. (With
+        the policy that lets decode steps run while someone waits, a plan counts those steps: then it has to be made.)"""
+        if not self.queue:
+            return True
+        if not self.prompts_first or self.mixed:
+            return False
+        if len(self.live) >= self.max_live:
+            return True
+        return self.cache.allocation_status(self.queue[0].n_tokens) is AllocStatus.LATER
+
     def retire(self, req: Request, why: str) -> None:
         """The request ends here, wherever it stands; what it holds goes back. Idempotent."""
         if req.phase is Phase.LIVE:
