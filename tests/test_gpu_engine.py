@@ -347,10 +347,10 @@ def test_command_line(model_dirs, plains):
 def test_command_line_random_weights(model_dirs):
     """--random CONFIG: weights drawn on the device from --weights-seed; the same seed gives the same tokens,
     another seed another model. A shipped shape's name stands for its config.json."""
-    def run(seed, source=None):
+    def run(seed, source=None, more=()):
         r = subprocess.run([sys.executable, "-m", "tokenmill_amd.generate", "--random", source or str(model_dirs["B"]),
                             "--weights-seed", str(seed), "--prompt-lens", "9,4", "--max-tokens", "8", "--ignore-eos",
-                            "--num-blocks", "16", "--max-model-len", "64", "--block-size", "8"],
+                            "--num-blocks", "16", "--max-model-len", "64", "--block-size", "8", *more],
                            capture_output=True, text=True, cwd=ROOT, timeout=300)
         assert r.returncode == 0, r.stderr[-2000:]
         return [json.loads(ln)["output_ids"] for ln in r.stdout.splitlines() if ln.startswith("{")]
@@ -358,6 +358,7 @@ def test_command_line_random_weights(model_dirs):
     assert [len(o) for o in first] == [8, 8]
     assert first == again
     assert first != other
+    assert run(3, more=("--hip-graphs", "--pipeline-decode")) == first     # replayed, each step queued ahead of the last one's tokens
     named = run(3, "tiny-a")
     by_path = run(3, str(ROOT / "tokenmill_amd" / "config" / "shapes" / "tiny-a.json"))
     assert [len(o) for o in named] == [8, 8] and named == by_path and named != first
