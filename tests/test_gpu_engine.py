@@ -781,8 +781,10 @@ def test_decode_steps_queued_ahead_with_sampling_arrivals_aborts_and_few_pages(m
 
     # more requests than slots: steps are queued ahead while the rest wait for a slot
     several = [SamplingParams(max_tokens=m, ignore_eos=True) for m in (20, 9, 31, 14, 25, 18)]
-    (a, _), (b, ahead) = _both(model_dirs["A"], "float32", lambda eng: eng.generate(prompts, several), max_num_seqs=3)
-    assert a == b and ahead.stats["steps_ahead"] > 20 and ahead.stats["peak_live"] == 3
+    for more in ({}, dict(enable_chunked_prefill=True, max_num_batched_tokens=24)):
+        (a, _), (b, ahead) = _both(model_dirs["A"], "float32", lambda eng: eng.generate(prompts, several),
+                                   max_num_seqs=3, **more)
+        assert a == b and ahead.stats["steps_ahead"] > 20 and ahead.stats["peak_live"] == 3
 
     greedy = SamplingParams(max_tokens=40, ignore_eos=True)
     (a, waiting), (b, ahead) = _both(model_dirs["A"], "float32", lambda eng: eng.generate(prompts, greedy),

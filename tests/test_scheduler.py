@@ -203,8 +203,8 @@ def test_retire_gives_pages_back_wherever_the_request_stands():
 def test_nobody_can_join_says_when_the_next_plan_would_admit_nobody():
     """What the engine asks before it queues a decode step ahead of the running one's tokens: with nobody waiting,
     with every slot taken, and with a head of the queue that has to wait for pages, the next plan is the live requests
-    again; a free slot and pages for the head, the policy that counts decode steps while someone waits, and mixed steps
-    need a plan of their own."""
+    again; a free slot and pages for the head, and the policy that counts decode steps while someone waits, need a
+    plan of their own."""
     sim = Sim(pages=8, page=4, max_num_seqs=2)
     assert sim.sched.nobody_can_join()
     a, b = sim.request(6), sim.request(6)
@@ -221,11 +221,14 @@ def test_nobody_can_join_says_when_the_next_plan_would_admit_nobody():
     sim.sched.retire(a, "stop")
     assert not sim.sched.nobody_can_join()
     sim.sched.retire(d, "abort")
-    for options in (dict(policy="decode_first"), dict(enable_chunked_prefill=True)):
-        other = Sim(pages=8, page=4, max_num_seqs=1, **options)
-        other.request(4), other.request(4)
-        other.step()
-        assert not other.sched.nobody_can_join()         # the slot is taken, and still the plan has to be made
+    other = Sim(pages=8, page=4, max_num_seqs=1, policy="decode_first")
+    other.request(4), other.request(4)
+    other.step()
+    assert not other.sched.nobody_can_join()             # the slot is taken, and still the plan has to be made: it counts
+    mixed = Sim(pages=8, page=4, max_num_seqs=1, enable_chunked_prefill=True)
+    mixed.request(4), mixed.request(4)
+    mixed.step()
+    assert mixed.sched.nobody_can_join()                 # mixed steps admit whenever they can, and now they cannot
 
 
 def test_decode_first_makes_the_queue_wait():

@@ -98,12 +98,13 @@ class Scheduler:
         return bool(self.queue) or bool(self.live)
 
     def nobody_can_join(self) -> bool:
-        """Would the next plan, made now, admit nobody? True when nobody waits; and, for the policy that admits
-        whenever it can, when every slot of a live request is taken or the head of the queue has to wait for pages. (With
-        the policy that lets decode steps run while someone waits, a plan counts those steps: then it has to be made.)"""
+        """Would the next plan, made now, admit nobody? True when nobody waits; and, where a plan admits whenever it
+        can (mixed steps, or whole prompts first), when every slot of a live request is taken or the head of the queue
+        has to wait for pages. (With the policy that lets decode steps run while someone waits, a plan counts those
+        steps: then it has to be made.)"""
         if not self.queue:
             return True
-        if not self.prompts_first or self.mixed:
+        if not self.prompts_first and not self.mixed:
             return False
         if len(self.live) >= self.max_live:
             return True
