@@ -364,9 +364,10 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path, dtype_na
     prompts = [random_ids(n, 200, 350 + i) for i, n in enumerate([12, 3, 30, 7, 21, 16, 9, 25, 5, 18])]
     params = [SamplingParams(max_tokens=6 + 3 * (i % 4), ignore_eos=True) for i in range(len(prompts))]
     outs = {}
-    for mode in ("eager", "graphs", "refused"):
+    for mode in ("eager", "graphs", "ahead", "refused"):
         eng = LLMEngine(EngineConfig(model=str(d), dtype=dtype_name, block_size=8, num_blocks=64, max_model_len=64,
-                                     max_num_seqs=4, max_num_batched_tokens=64, watermark=0.0, hip_graphs=mode != "eager"))
+                                     max_num_seqs=4, max_num_batched_tokens=64, watermark=0.0, hip_graphs=mode != "eager",
+                                     pipeline_decode=mode == "ahead"))
         # the mixer with state runs through its own code, between the library's operations: two hops a step, not the model
         assert [type(p).__name__ for p in eng.runner.program.foreign_parts] == ["DecayedSumMixer"] * 2
         assert len(eng.runner.program.parts) == 2 + 2 + 4      # embedding, head, two attentions, four feed-forwards
@@ -377,12 +378,14 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path, dtype_na
             eng.runner.graphs = DecodeGraphs(eng.runner, eng.cfg)
             assert not eng.runner.graphs.stateful_ok
         outs[mode] = eng.generate(prompts, params)
-        if mode == "graphs":
+        if mode in ("graphs", "ahead"):
             assert eng.runner.graphs.replays > 10
+        # decode steps queued ahead of the running step's tokens advance every live request's state once a step too
+        assert (eng.stats["steps_ahead"] > 5) == (mode == "ahead")
         if mode == "refused":
             assert eng.runner.graphs.replays == 0
         assert eng.cache.num_free_pages == eng.cache.num_pages
-    assert outs["graphs"] == outs["eager"] == outs["refused"]
+    assert outs["graphs"] == outs["eager"] == outs["refused"] == outs["ahead"]
 
 
 # ----------------------------------------------------------------------------------------------- windows, a layer twice, a shared cache
