@@ -19,8 +19,7 @@ from tokenmill_amd.cache.manager import CacheManager
 from tokenmill_amd.cache.pool import CachePools
 from tokenmill_amd.config.engine_config import EngineConfig
 from tokenmill_amd.engine.loading import load_model, resolve_device, resolve_dtype
-from tokenmill_amd.engine.request import Request, RequestOutput
-from tokenmill_amd.engine.request import Phase
+from tokenmill_amd.engine.request import Phase, Request, RequestOutput
 from tokenmill_amd.engine.runner import ModelRunner, StepEntry
 from tokenmill_amd.engine.scheduler import Scheduler, StepPlan
 from tokenmill_amd.engine.sizing import num_cache_pages

@@ -11,7 +11,7 @@ from dataclasses import dataclass
 
 import torch
 
-from tokenmill_amd.parts.base import KVCacheSpec, Norm, Part, StateSpec, StepContext
+from tokenmill_amd.parts.base import KVCacheSpec, Norm, Part, StateSpec
 from tokenmill_amd.weights.loader import TensorSpec
 
 
