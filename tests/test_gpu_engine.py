@@ -792,3 +792,44 @@ def test_decode_steps_queued_ahead_with_sampling_arrivals_aborts_and_few_pages(m
     assert a == b and waiting.scheduler.evictions > 0 and ahead.scheduler.evictions > 0
     ahead.cache.check_invariants()
     assert ahead.cache.num_free_pages == ahead.cache.num_pages
+
+
+def test_no_graph_is_destroyed_while_another_is_recorded(model_dirs):
+    """An engine that was dropped frees nothing at once (it holds reference cycles); if Python's collector found it
+    while a later engine records a graph, its graphs would be destroyed inside the recording, which HIP refuses from a
+    destructor: the process would end. A recording therefore collects what is garbage before it starts and lets the
+    collector rest until it ends."""
+    import contextlib
+    import gc
+    import weakref
+    from tokenmill_amd import SamplingParams
+    from tokenmill_amd.engine import graphs as G
+    sp = SamplingParams(max_tokens=6, ignore_eos=True)
+    prompts = [random_ids(n, 256, 700 + i) for i, n in enumerate((5, 9))]
+    gc.collect()
+    gc.disable()
+    try:
+        first = make_engine(model_dirs["A"], "float32", hip_graphs=True)
+        want = first.generate(prompts, sp)
+        dropped = weakref.ref(next(iter(first.runner.graphs.buckets.values())).graph)
+        del first                                   # no collection runs: what the engine holds in cycles stays
+        gc.enable()
+        second = make_engine(model_dirs["A"], "float32", hip_graphs=True)
+        seen = []
+        recording = G._recording
+
+        @contextlib.contextmanager
+        def watched(graph):
+            with recording(graph):
+                seen.append((dropped() is not None, gc.isenabled()))
+                yield
+
+        G._recording = watched
+        try:
+            assert second.generate(prompts, sp) == want
+        finally:
+            G._recording = recording
+        assert seen and all(s == (False, False) for s in seen)    # the dropped graph is gone, the collector rests
+        assert gc.isenabled()
+    finally:
+        gc.enable()

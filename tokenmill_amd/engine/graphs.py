@@ -17,6 +17,8 @@ steps of a serving run replay a handful of graphs: ``StepGraphs``.
 """
 from __future__ import annotations
 
+import contextlib
+import gc
 import logging
 
 import numpy as np
@@ -27,6 +29,24 @@ from tokenmill_amd.hip import ops
 from tokenmill_amd.parts.base import GroupStep, StepContext
 
 log = logging.getLogger(__name__)
+
+
+@contextlib.contextmanager
+def _recording(graph: torch.cuda.CUDAGraph):
+    """``torch.cuda.graph(graph)`` during which nothing is destroyed. While a stream records, HIP refuses to
+    destroy a graph; Python's collector runs whenever enough objects have been made, and if it then finds an engine
+    that was dropped earlier (engines hold reference cycles, so dropping one frees nothing at once), that engine's
+    graphs are destroyed in the middle of the recording: an error inside a destructor, which ends the process.
+    So what is garbage is collected before the recording starts, and the collector rests until it ends."""
+    gc.collect()
+    resting = gc.isenabled()
+    gc.disable()
+    try:
+        with torch.cuda.graph(graph):
+            yield
+    finally:
+        if resting:
+            gc.enable()
 
 
 class _Bucket:
@@ -198,7 +218,7 @@ class DecodeGraphs:
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
+        with _recording(graph):
             bk.logits = runner.forward(step)
         slots.copy_(real_slots)
         bk.graph = graph
@@ -312,7 +332,7 @@ class StepGraphs:
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
+        with _recording(graph):
             slot.logits = runner.forward(step)
         slot.graph = graph
         return slot
