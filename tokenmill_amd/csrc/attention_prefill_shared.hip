@@ -89,8 +89,9 @@ struct StageCopy {
                 const uint64_t at = lane_value(places.k, 4 * rel + (kk >> 4));
                 k[i] = *(const u32x4_t*)(k_pool + at + ((size_t)(kk & 15) * KVH * D + pc * 8) * sizeof(bf16_t));
             }
-            {   // values: half `half` of the 16 keys of tile j in row d
-                const int j = idx / (2 * D), d = (idx % (2 * D)) / 2, half = idx & 1;
+            {   // values: half `half` of the 16 keys of tile j in row d; consecutive lanes take consecutive rows, whose
+                // 16-byte pieces then go to 16 different places of LDS's banks (two halves of a row side by side collide)
+                const int j = idx / (2 * D), half = (idx % (2 * D)) / D, d = idx % D;
                 const uint64_t at = lane_value(places.v, 4 * rel + j);
                 v[i] = *(const u32x4_t*)(v_pool + at + (((size_t)d << page_shift) + half * 8) * sizeof(bf16_t));
             }
@@ -107,7 +108,7 @@ struct StageCopy {
             if (!EXACT && idx >= PIECES) continue;
             const int kk = idx / (D / 8), pc = idx % (D / 8);
             *(u32x4_t*)(stage + stage_row(kk) * SharedShape<D>::K_STRIDE + pc * 16) = k[i];
-            const int j = idx / (2 * D), d = (idx % (2 * D)) / 2, half = idx & 1;
+            const int j = idx / (2 * D), half = (idx % (2 * D)) / D, d = idx % D;
             u32x4_t val = v[i];
             if (keys < PS_KEYS) {                                    // block-uniform: a tile's last stage only
                 const int first = 16 * j + 8 * half;
