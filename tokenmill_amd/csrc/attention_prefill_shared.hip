@@ -38,9 +38,12 @@ __device__ __forceinline__ int stage_row(int kk) {
 
 template <int D>
 struct SharedShape {
-    // rows padded by 16 bytes: the 16 rows that the lanes of an operand load touch then start in 16 different
-    // groups of four banks
-    static constexpr int K_STRIDE = D * 2 + 16, V_STRIDE = PS_KEYS * 2 + 16;
+    // Rows padded by 32 bytes. An operand load has lane (r, g) read 16 bytes at row r, piece g; measured with the
+    // bank-conflict counter, such loads are free of conflicts when the row stride is 32 bytes more than a multiple of
+    // 64 (288, 160, 224, 96 bytes here) and take twice as long with a stride 16 bytes more than a multiple of 32 (272,
+    // 144), the usual padding. The stores (whole key rows; value rows two lanes a row) are free of conflicts with these
+    // strides too.
+    static constexpr int K_STRIDE = D * 2 + 32, V_STRIDE = PS_KEYS * 2 + 32;
     static constexpr int K_BYTES = PS_KEYS * K_STRIDE, V_BYTES = D * V_STRIDE, STAGE = K_BYTES + V_BYTES;
     static constexpr int PIECES = PS_KEYS * D / 8;               // 16-byte pieces of a stage's keys; as many of its values
 };
@@ -89,9 +92,9 @@ struct StageCopy {
                 const uint64_t at = lane_value(places.k, 4 * rel + (kk >> 4));
                 k[i] = *(const u32x4_t*)(k_pool + at + ((size_t)(kk & 15) * KVH * D + pc * 8) * sizeof(bf16_t));
             }
-            {   // values: half `half` of the 16 keys of tile j in row d; consecutive lanes take consecutive rows, whose
-                // 16-byte pieces then go to 16 different places of LDS's banks (two halves of a row side by side collide)
-                const int j = idx / (2 * D), half = (idx % (2 * D)) / D, d = idx % D;
+            {   // values: half `half` of the 16 keys of tile j in row d (two lanes a row: with rows 160 bytes apart the 16
+                // pieces of 8 rows go to 16 different places of LDS's banks)
+                const int j = idx / (2 * D), d = (idx % (2 * D)) / 2, half = idx & 1;
                 const uint64_t at = lane_value(places.v, 4 * rel + j);
                 v[i] = *(const u32x4_t*)(v_pool + at + (((size_t)d << page_shift) + half * 8) * sizeof(bf16_t));
             }
@@ -108,7 +111,7 @@ struct StageCopy {
             if (!EXACT && idx >= PIECES) continue;
             const int kk = idx / (D / 8), pc = idx % (D / 8);
             *(u32x4_t*)(stage + stage_row(kk) * SharedShape<D>::K_STRIDE + pc * 16) = k[i];
-            const int j = idx / (2 * D), half = (idx % (2 * D)) / D, d = idx % D;
+            const int j = idx / (2 * D), d = (idx % (2 * D)) / 2, half = idx & 1;
             u32x4_t val = v[i];
             if (keys < PS_KEYS) {                                    // block-uniform: a tile's last stage only
                 const int first = 16 * j + 8 * half;

@@ -25,7 +25,7 @@ __device__ __forceinline__ float fd_round(float a) { return bf16_to_f32(f32_to_b
 #define FD_EPI_SILU 1
 #define FD_KCH 8            // k-steps of one register group of matrix loads, per wavefront (one group in all)
 #define FD_KCH_PIPE 6       // the same where two groups take turns
-#define FD_XPAD 8           // padding of an LDS row of x, in elements
+#define FD_XPAD 16          // padding of an LDS row of x, in elements: with K a multiple of 32 the rows are 32 bytes more than a multiple of 64 apart, which the operand loads read free of bank conflicts (with 8 they take twice as long)
 #define FD_RC 8             // 4-element vectors of a residual row a thread keeps in registers
 
 // rows of x a block keeps in LDS for M tokens

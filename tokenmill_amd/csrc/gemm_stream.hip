@@ -35,7 +35,7 @@
 #define ST_WD 8             // k-steps of the matrix a wavefront has in registers or on their way (a multiple of ST_KCH)
 // the matrix is read once and never again: loads that do not displace the activations in the caches
 #define ST_WLOAD(p) __builtin_nontemporal_load((const u32x4_t*)(p))
-#define ST_XPAD 8           // padding of an LDS row of activations, in elements
+#define ST_XPAD 16          // padding of an LDS row of activations, in elements: rows 288 bytes apart, which the operand loads (lane (r, g): 16 bytes of row r at piece g) read free of bank conflicts; with 8 (272 bytes) they take twice as long
 
 struct StreamArgs {
     FusedArgs f;            // activations X [M, K], the packed matrix, and what the q|k|v and SiLU epilogues need
