@@ -136,14 +136,11 @@ extern "C" int tm_gemm_f32_mfma(const float* A, int lda, const float* W, const f
                                 int N, int K, hipStream_t stream) {
     if (M <= 0 || N <= 0) return TM_OK;
     if (!tm_gemm_f32_mfma_fits(A, lda, W, bias, C, ldc, M, N, K)) return TM_ERR_ARG;
-    // large tiles where they still give every CU a block, else smaller ones
-    const long long big = (long long)((M + 127) / 128) * ((N + 127) / 128);
+    // 64 x 128 tiles where they still give every CU a block, else 64 x 64. (128 x 128 tiles were the faster ones while
+    // one set of accumulators sufficed; with the running total beside the block's sum they leave two wavefronts a
+    // SIMD instead of three and are the slower ones: 21.2 ms against 20.8 ms for the 2,048-token prefill.)
     const long long mid = (long long)((M + 63) / 64) * ((N + 127) / 128);
-    if (big >= 256) {
-        dim3 grid((N + 127) / 128, (M + 127) / 128);
-        if (grid.y > 65535u) return TM_ERR_ARG;
-        gemm_nt_mfma_f32_kernel<128, 128><<<grid, 256, 0, stream>>>(A, lda, W, bias, C, ldc, M, N, K);
-    } else if (mid >= 256) {
+    if (mid >= 256) {
         dim3 grid((N + 127) / 128, (M + 63) / 64);
         if (grid.y > 65535u) return TM_ERR_ARG;
         gemm_nt_mfma_f32_kernel<64, 128><<<grid, 256, 0, stream>>>(A, lda, W, bias, C, ldc, M, N, K);
