@@ -70,6 +70,8 @@ class LLMEngine:
             from tokenmill_amd.engine.graphs import DecodeGraphs, StepGraphs
             self.runner.graphs = DecodeGraphs(self.runner, cfg)
             self.runner.step_graphs = StepGraphs(self.runner)
+        if cfg.pipeline_decode and not cfg.hip_graphs:
+            log.warning("pipeline_decode queues graph replays ahead: without hip_graphs no step is queued ahead")
         self.scheduler = Scheduler(cfg, self.cache)
         self.sampler = Sampler(self.device)
         self.requests: dict[str, Request] = {}           # every request that has not ended
