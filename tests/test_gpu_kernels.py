@@ -49,7 +49,7 @@ def test_embed_gather(ops, dt):
 
 
 @pytest.mark.parametrize("dt", DTS)
-@pytest.mark.parametrize("hidden", [64, 120, 896, 5000])
+@pytest.mark.parametrize("hidden", [64, 120, 896, 2048, 3584, 5000, 16384, 16388])
 def test_add_rmsnorm(ops, dt, hidden):
     torch.manual_seed(1)
     T, eps = 7, 1e-5
@@ -1046,7 +1046,8 @@ def test_stream_qkv_rope(ops, M, K, H, KVH, D, page, rows):
     assert torch.equal(q_one[0], q_all[M - 1])
 
 
-@pytest.mark.parametrize("M,K,I", [(64, 896, 4864), (17, 64, 128), (48, 3584, 1000), (33, 120, 200), (9, 1048, 100)])
+@pytest.mark.parametrize("M,K,I", [(64, 896, 4864), (17, 64, 128), (48, 3584, 1000), (33, 120, 200), (9, 1048, 100),
+                                   (64, 264, 16400), (20, 3584, 18944)])
 def test_stream_gate_up_silu(ops, M, K, I):
     torch.manual_seed(24)
     dt = torch.bfloat16
@@ -1093,8 +1094,10 @@ def test_stream_linear_stores_or_adds_into_the_residual(ops, M, N, K, rows):
     assert torch.equal(other, out)
 
 
-@pytest.mark.parametrize("M,N,K,rows", [(64, 896, 4864, 4), (33, 3584, 18944, 16), (20, 200, 120, 8), (48, 1001, 9000, 16)])
-def test_stream_linear_with_k_split_over_blocks_and_the_norm_that_adds_the_parts(ops, M, N, K, rows):
+@pytest.mark.parametrize("M,N,K,rows,groups", [(64, 896, 4864, 4, 8), (33, 3584, 18944, 16, 8), (20, 200, 120, 8, 1),
+                                               (48, 1001, 9000, 16, 8), (64, 5120, 27648, 16, 8), (17, 3584, 3584, 8, 8),
+                                               (40, 512, 1024, 16, 2)])
+def test_stream_linear_with_k_split_over_blocks_and_the_norm_that_adds_the_parts(ops, M, N, K, rows, groups):
     """A plain product with few rows of output and a long K splits K over groups of blocks, which leave 32-bit partial
     sums; the norm that follows adds them up in their order, rounds the sum as the product's own epilogue would have,
     and goes on as if it had been handed that tensor: the same bits as the two steps one after the other."""
@@ -1106,7 +1109,7 @@ def test_stream_linear_with_k_split_over_blocks_and_the_norm_that_adds_the_parts
     Wp = ops.pack_weight(w.to(dt).to(DEV), rows)
     parts = ops.stream_linear_split(da, Wp, db)
     n_parts = parts.shape[0]
-    assert (n_parts >= 2 if K >= 4000 else n_parts == 1) and tuple(parts.shape[1:]) == (M, N)
+    assert n_parts == groups and tuple(parts.shape[1:]) == (M, N)
     delta = ops.sum_parts(parts, torch.empty(M, N, dtype=dt, device=DEV))
     torch.testing.assert_close(delta.float().cpu(), q(want, dt), **tol(dt))
     assert torch.equal(delta.float().cpu(), q(parts.sum(0).cpu(), dt)) or n_parts > 2   # (two parts: one order only)

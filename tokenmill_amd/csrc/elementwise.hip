@@ -86,8 +86,8 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const Pending<T> p
     }
 }
 
-// The same for widths that are a multiple of 4 and at most 4096: every thread keeps its (up to four)
-// 4-element groups of the row in registers, so the row is read once.
+// The same for widths that are a multiple of 4 and at most 16,384: every thread (256, 512 or 1,024 of them) keeps
+// its (up to four) 4-element groups of the row in registers, so the row is read once.
 typedef float ew_f32x4 __attribute__((ext_vector_type(4)));
 
 template <typename T> struct Vec4;
@@ -111,12 +111,12 @@ template <> struct Vec4<bf16_t> {
 
 #define ADD_NORM_MAX_PARTS 8       // most partial sums the vector kernel adds (more: the plain kernel)
 
-template <typename T, typename WT>
-__global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict__ resid, const Pending<T> pending,
+template <typename T, typename WT, int THREADS>
+__global__ __launch_bounds__(THREADS) void add_rmsnorm_vec_kernel(float* __restrict__ resid, const Pending<T> pending,
                                                               const int* __restrict__ rows,
                                                               const WT* __restrict__ weight, T* __restrict__ out,
                                                               int hidden, float eps) {
-    __shared__ float red[4];
+    __shared__ float red[THREADS / 64];
     const int r = blockIdx.x;
     const size_t src = rows ? (size_t)rows[r] : (size_t)r;
     float* x = resid + src * hidden;
@@ -128,7 +128,7 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
     float ss = 0.f;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const int gidx = threadIdx.x + i * 256;
+        const int gidx = threadIdx.x + i * THREADS;
         v[i] = ew_f32x4{0.f, 0.f, 0.f, 0.f};
         if (gidx < groups) {
             v[i] = Vec4<float>::load(x + 4 * gidx);
@@ -152,11 +152,11 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
             ss += v[i][0] * v[i][0] + v[i][1] * v[i][1] + v[i][2] * v[i][2] + v[i][3] * v[i][3];
         }
     }
-    ss = block_sum<256>(ss, red);
+    ss = block_sum<THREADS>(ss, red);
     const float rs = rsqrtf(ss / (float)hidden + eps);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const int gidx = threadIdx.x + i * 256;
+        const int gidx = threadIdx.x + i * THREADS;
         if (gidx < groups) {
             const ew_f32x4 w = Vec4<WT>::load(weight + 4 * gidx);
             ew_f32x4 y;
@@ -171,12 +171,20 @@ template <typename T, typename WT>
 static void launch_add_rmsnorm(float* resid, const void* delta, const float* parts, int n_parts, size_t stride,
                                const int* rows, const void* weight, void* out, int R, int hidden, float eps,
                                hipStream_t stream) {
-    const bool vec = hidden % 4 == 0 && hidden <= 4096 && ((uintptr_t)resid % 16) == 0 && ((uintptr_t)weight % 16) == 0 &&
+    const bool vec = hidden % 4 == 0 && hidden <= 16384 && ((uintptr_t)resid % 16) == 0 && ((uintptr_t)weight % 16) == 0 &&
                      ((uintptr_t)out % 16) == 0 && (!delta || ((uintptr_t)delta % 16) == 0) &&
                      (!parts || (((uintptr_t)parts % 16) == 0 && stride % 4 == 0 && n_parts <= ADD_NORM_MAX_PARTS));
     const Pending<T> pending{(const T*)delta, parts, n_parts, stride};
-    if (vec)
-        add_rmsnorm_vec_kernel<T, WT><<<R, 256, 0, stream>>>(resid, pending, rows, (const WT*)weight, (T*)out, hidden, eps);
+    // a thread for every 4-element group where 1,024 reach (measured on an MI355X, 64 rows with 4 partial sums: width
+    // 3,584 6.5 us with 256 threads, 4.9 with 512, 4.5 with 1,024; width 5,120 5.7 with 512, 5.1 with 1,024; width 896
+    // 3.4 us with any); from the width alone: the sum of squares has one order per model
+    const int threads = hidden <= 1024 ? 256 : hidden <= 2048 ? 512 : 1024;
+    if (vec && threads == 256)
+        add_rmsnorm_vec_kernel<T, WT, 256><<<R, 256, 0, stream>>>(resid, pending, rows, (const WT*)weight, (T*)out, hidden, eps);
+    else if (vec && threads == 512)
+        add_rmsnorm_vec_kernel<T, WT, 512><<<R, 512, 0, stream>>>(resid, pending, rows, (const WT*)weight, (T*)out, hidden, eps);
+    else if (vec)
+        add_rmsnorm_vec_kernel<T, WT, 1024><<<R, 1024, 0, stream>>>(resid, pending, rows, (const WT*)weight, (T*)out, hidden, eps);
     else
         add_rmsnorm_kernel<T, WT><<<R, 256, 0, stream>>>(resid, pending, rows, (const WT*)weight, (T*)out, hidden, eps);
 }

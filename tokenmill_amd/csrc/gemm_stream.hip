@@ -382,17 +382,45 @@ __global__ __launch_bounds__(64 * KS * US) void gemm_stream_kernel(const StreamA
 // the matrix's shape alone (never from the number of tokens: that keeps a token's sums in one order). Many units
 // (gate|up): the units share, K is split little; few units over a long K (the down projection): K is split over
 // the whole block, so that the chip still has a few thousand wavefronts streaming.
-static void stream_config(int n_units, int ksteps, int tiles, int* ks, int* us) {
-    // From the matrix alone (KS fixes the order of a token's sums). Measured on an MI355X at the 0.5B and 7B layer
-    // sizes, 32 / 48 / 64 tokens: gate|up 7B (1,184 units) 1 x 4: 60 / 67 / 68 us (2 x 2: 57 / 68 / 76, 2 x 4: 63 / 65 / 79,
-    // 4 x 2: 56 / 74 / 81, 8 x 1: 72 / - / 111), gate|up 32B (1,728 units) 1 x 4: 96 / 103 / 109 us = 5.9 / 5.5 / 5.2 TB/s
-    // (2 x 2: 110 / 117 / 130); gate|up 0.5B (304 units) 4 x 2: 9 / - / 12 us; q|k|v 7B (144 units) 8 x 1: 17 / - / 25 us
-    // (4 x 2: 20 / - / 27).
-    if (n_units >= 1024) { *ks = 1; *us = 4; }
+static void stream_config(int n_units, int* ks, int* us) {
+    // From the matrix alone (KS fixes the order of a token's sums). Measured on an MI355X at the 0.5B, 7B and 32B layer
+    // sizes, 17 / 32 / 48 / 64 tokens: gate|up 7B (1,184 units) 2 x 8: 63 / 61 / 66 / 63-67 us (1 x 4: 59 / 60 / 68 / 73,
+    // 1 x 8: - / 69 / - / 71, 2 x 4: 62 / 63 / 66 / 79, 2 x 2: - / 56 / - / 76, 4 x 4: - / 70 / - / 100, 1 x 16: - / 96 / - / 97),
+    // gate|up 32B (1,728 units) 2 x 8: 99 / 97 / 102 / 103 us (1 x 4: 96 / 97 / 104 / 109-112, 2 x 2: - / 110 / - / 130);
+    // gate|up 0.5B (304 units) 4 x 2: 9 / - / 12 us; q|k|v 7B (144 units) 8 x 1: 17 / - / 25 us (4 x 2: 20 / - / 27).
+    // With many units, sixteen wavefronts on eight units share one window of the activations: at 64 tokens every
+    // block's copy of the activations is half as many bytes as the matrix itself (1 x 4), a quarter with 2 x 8.
+    if (n_units >= 1024) { *ks = 2; *us = 8; }
     else if (n_units >= 256) { *ks = 4; *us = 2; }
     else { *ks = 8; *us = 1; }
-    (void)ksteps;
-    (void)tiles;
+}
+
+// The same for a plain product whose K is split over `parts` groups of blocks, which leave 32-bit partial sums
+// (1: not split). From the matrix's shape alone.
+static void stream_plain_shape(int N, int K, int* parts, int* ks, int* us) {
+    const int n_units = (N + 31) / 32, ksteps = (K + 31) / 32;
+    // Wide outputs over a K that gives every wavefront four k-steps: eight groups, two wavefronts a unit, and as many
+    // units a block as leave about 150 blocks. Measured on an MI355X, 17 / 32 / 48 / 64 tokens: 7B down (112 units,
+    // K 18,944) 8 groups of 2 x 4: 29 / 29 / 31 / 34 us (4 groups of 4 x 2: 31 / 30 / 35 / 39; 8 of 2 x 8: 36 / 36 / 39 / 42;
+    // unsplit 56 / 81 us at 32 / 64; the library's product with its algorithm chosen by timing 52 / 69); 7B o: 9.5 / 9.6 /
+    // 11.0 / 12.3 us (4 of 4 x 2: 9.7 / 9.8 / 11.8 / 13.0); 32B down (160 units, K 27,648) 8 groups of 2 x 8: 58 / 55 / 63 /
+    // 61 us (4 of 4 x 2: 64 / 65 / 84 / 92; 8 of 2 x 4: 61 / 61 / 74 / 78); 32B o: 15 / 15 / 17 / 18 us (4 of 4 x 2: 17 / 17 /
+    // 24 / 27).
+    if (n_units >= 96 && ksteps >= 64) {
+        *parts = 8;
+        *ks = 2;
+        *us = n_units >= 144 ? 8 : 4;
+        return;
+    }
+    // Narrow outputs: the fewest groups (a power of two, at most 8) that give the matrix about 400 blocks' worth of
+    // units, as long as a wavefront (of the four that split a block's share of K) keeps four k-steps to itself:
+    // 0.5B down 8 groups: 8 / 11 us at 32 / 64 tokens against 10 / 10 us. 1: not worth splitting (the library's
+    // product is the faster one then).
+    int p = 1;
+    while (p < 8 && n_units * p < 384) p *= 2;
+    while (p > 1 && ksteps / (p * 4) < 4) p /= 2;
+    *parts = p;
+    stream_config(n_units * p, ks, us);
 }
 
 template <int EPI, int NT, int KS, int US>
@@ -411,23 +439,25 @@ static int launch_stream_config(const StreamArgs& a, int n_units, int kparts, hi
 }
 
 template <int EPI, int NT>
-static int launch_stream_tiles(const StreamArgs& a, int n_units, int kparts, hipStream_t stream) {
-    int ks = 0, us = 0;
-    stream_config(n_units * kparts, (a.f.K + 31) / 32 / kparts, NT, &ks, &us);
-    switch (ks * 16 + us) {                     // the shapes stream_config names
+static int launch_stream_tiles(const StreamArgs& a, int n_units, int kparts, int ks, int us, hipStream_t stream) {
+    switch (ks * 16 + us) {                     // the shapes stream_config and stream_plain_shape name
         case 4 * 16 + 2: return launch_stream_config<EPI, NT, 4, 2>(a, n_units, kparts, stream);
         case 8 * 16 + 1: return launch_stream_config<EPI, NT, 8, 1>(a, n_units, kparts, stream);
-        default: return launch_stream_config<EPI, NT, 1, 4>(a, n_units, kparts, stream);
+        case 2 * 16 + 4: return launch_stream_config<EPI, NT, 2, 4>(a, n_units, kparts, stream);
+        case 2 * 16 + 8: return launch_stream_config<EPI, NT, 2, 8>(a, n_units, kparts, stream);
+        default: return TM_ERR_ARG;
     }
 }
 
+// kparts == 1: the block's shape from the number of units; else the caller's (stream_plain_shape).
 template <int EPI>
-static int launch_stream(const StreamArgs& a, int n_units, hipStream_t stream, int kparts = 1) {
+static int launch_stream(const StreamArgs& a, int n_units, hipStream_t stream, int kparts = 1, int ks = 0, int us = 0) {
+    if (ks == 0) stream_config(n_units, &ks, &us);
     switch ((a.f.M + 15) / 16) {
         case 1:
-        case 2: return launch_stream_tiles<EPI, 2>(a, n_units, kparts, stream);
-        case 3: return launch_stream_tiles<EPI, 3>(a, n_units, kparts, stream);
-        default: return launch_stream_tiles<EPI, 4>(a, n_units, kparts, stream);
+        case 2: return launch_stream_tiles<EPI, 2>(a, n_units, kparts, ks, us, stream);
+        case 3: return launch_stream_tiles<EPI, 3>(a, n_units, kparts, ks, us, stream);
+        default: return launch_stream_tiles<EPI, 4>(a, n_units, kparts, ks, us, stream);
     }
 }
 
@@ -500,15 +530,8 @@ extern "C" int tm_stream_linear(const void* X, int ldx, int M, int K, const void
 // Groups of blocks a plain product's K is split over: enough that a matrix with few rows still has a few thousand
 // wavefronts streaming it, each with a few rounds of k-steps to itself. From the matrix's shape alone.
 extern "C" int tm_stream_linear_parts(int N, int K) {
-    // The fewest groups (a power of two, at most 8) that give the matrix about 400 blocks, as long as a wavefront (of
-    // the four that split a block's share of K) keeps four k-steps to itself. Measured on an MI355X, 32 and 64 rows:
-    // 7B down (112 units, K 18,944) 4 groups: 30 / 39 us against 56 / 81 us unsplit and 52 / 69 us for the library's
-    // product with its algorithm chosen by timing; 7B o 4 groups: 10 / 13 us against 13 / 13 us; 0.5B down 8 groups:
-    // 8 / 11 us against 10 / 10 us. 1: not worth splitting (the library's product is the faster one then).
-    const int n_units = (N + 31) / 32, ksteps = (K + 31) / 32;
-    int parts = 1;
-    while (parts < 8 && n_units * parts < 384) parts *= 2;
-    while (parts > 1 && ksteps / (parts * 4) < 4) parts /= 2;
+    int parts = 1, ks = 0, us = 0;
+    stream_plain_shape(N, K, &parts, &ks, &us);
     return parts;
 }
 
@@ -523,5 +546,7 @@ extern "C" int tm_stream_linear_split(const void* X, int ldx, int M, int K, cons
     a.rows = rows;
     a.n_strips = (N + rows - 1) / rows;
     a.N = N; a.parts = parts;
-    return launch_stream<ST_EPI_PLAIN>(a, (N + 31) / 32, stream, tm_stream_linear_parts(N, K));
+    int kparts = 1, ks = 0, us = 0;
+    stream_plain_shape(N, K, &kparts, &ks, &us);
+    return launch_stream<ST_EPI_PLAIN>(a, (N + 31) / 32, stream, kparts, ks, us);
 }
