@@ -112,7 +112,12 @@ def test_every_cut_at_the_layer_sizes_of_the_published_shapes(layer_models, monk
         assert_all_given_back(session)
     took = session.runner.program.counters()
     if dtype_name == "bfloat16":
-        assert took["qkv_from_norm"] > 0 and took["gate_up_from_norm"] > 0 and took["qkv_plain"] > 0
+        assert took["qkv_plain"] > 0
+        if name == "32B":       # at this width the products that stream the matrix through windows of K take every step of up to 64 rows
+            assert took["qkv_from_norm"] == 0 and took["gate_up_from_norm"] == 0
+            assert took["qkv_stream"] > 0 and took["gate_up_stream"] > 0
+        else:
+            assert took["qkv_from_norm"] > 0 and took["gate_up_from_norm"] > 0
         assert took["qkv_panel"] > 0 or name != "0.5B"        # widths of 3,584 and 5,120 do not fit a block's LDS
     else:
         assert took["qkv_plain"] > 0 and took["qkv_from_norm"] == 0

@@ -8,6 +8,18 @@
 // up to this many rows the kernels that stream the matrix once win: the products over packed matrices with
 // the layer's epilogue (bias, rotary + cache write, SiLU*up, residual add), and the ones that start at the norm
 constexpr int TM_SKINNY_ROWS = 16;
+// ... while the model is narrow. They keep all of K of every row in LDS (or re-read the rows per block); from a
+// width of 2,048 the products that stream the matrix through windows of K (gemm_stream.hip, with the partial sums
+// of the output and down projections added by the next norm) take over at fewer rows. Measured on an MI355X, a
+// decode step with this family against the stream family: width 896 (0.5B shape) 16 rows 1.16 against 1.23 ms;
+// width 3,584 (7B) 4 rows 3.45 against 3.71, 8 rows 3.72 against 3.81, 10 rows 4.04 against 3.84, 16 rows 4.42
+// against 4.02; width 5,120 (32B, 16 layers) 1 row 3.64 against 3.53, 4 rows 3.80 against 3.54, 8 rows 4.10 against
+// 3.65, 16 rows 4.92 against 3.90. The two families do not mix within a layer: the kernels that start at the norm
+// need the residual stream complete, the stream family leaves partial sums for the norm.
+inline int tm_skinny_rows(int hidden) { return hidden < 2048 ? TM_SKINNY_ROWS : hidden < 4096 ? 8 : 0; }
+// ... and the two of them that start at the norm (q|k|v, gate|up) at most to 8 rows: with 9 to 16 rows in LDS a CU
+// holds one block (0.5B shape, 16 rows: 1.195 ms a step against 1.156 with the panel kernels behind a norm of its own)
+inline int tm_from_norm_rows(int hidden) { const int s = tm_skinny_rows(hidden); return s < 8 ? s : 8; }
 // up to this many rows gate|up keeps the normed input in LDS (where it fits) and carries its epilogue; q|k|v, whose
 // matrix is small enough that the copy of the input is most of the kernel's work, does so for every row count the
 // panel kernels take (measured at the 0.5B shape, 64 rows: 10.9 us against 14.9 us streamed)

@@ -6,7 +6,7 @@
 // copy the decode kernels for up to 16 tokens read, whatever its strips' height (16, 8 or 4 rows): a wavefront
 // always multiplies two tiles of 16 matrix rows (a "unit": the two halves of 16 rotary pairs, 16 gate rows and
 // the 16 up rows that meet them, or 32 consecutive rows), each tile made of 1, 2 or 4 packed strips, with all
-// row tiles of the activations (2 to 4 tiles of 16 tokens), so a 16-byte piece of the matrix is used for up to
+// row tiles of the activations (1 to 4 tiles of 16 tokens), so a 16-byte piece of the matrix is used for up to
 // 64 tokens.
 //
 // A block has KS x US wavefronts: US units side by side, each unit's K split over KS wavefronts. The block walks K
@@ -94,7 +94,7 @@ __host__ __device__ constexpr int stream_lds_bytes(int NT, int KS, int US) {
     return window > sums ? window : sums;
 }
 
-// NT: 16-token tiles of the activations (2..4). KS: wavefronts that split a unit's K. US: units of a block.
+// NT: 16-token tiles of the activations (1..4). KS: wavefronts that split a unit's K. US: units of a block.
 template <int EPI, int NT, int KS, int US>
 __global__ __launch_bounds__(64 * KS * US) void gemm_stream_kernel(const StreamArgs a, const int n_units) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -454,7 +454,7 @@ template <int EPI>
 static int launch_stream(const StreamArgs& a, int n_units, hipStream_t stream, int kparts = 1, int ks = 0, int us = 0) {
     if (ks == 0) stream_config(n_units, &ks, &us);
     switch ((a.f.M + 15) / 16) {
-        case 1:
+        case 1: return launch_stream_tiles<EPI, 1>(a, n_units, kparts, ks, us, stream);
         case 2: return launch_stream_tiles<EPI, 2>(a, n_units, kparts, ks, us, stream);
         case 3: return launch_stream_tiles<EPI, 3>(a, n_units, kparts, ks, us, stream);
         default: return launch_stream_tiles<EPI, 4>(a, n_units, kparts, ks, us, stream);

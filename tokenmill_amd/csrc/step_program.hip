@@ -64,12 +64,13 @@ bool fused_lds_fits(int M, int K) {
     return (size_t)rows * (K + 8) * 2 + (size_t)4 * waves * 2 * 64 * 5 + 1024 <= 160 * 1024;
 }
 
-bool fused_decode_ok(const float* resid, const TmLinear& L, int M) {
-    return resid && L.packed && M > 0 && M <= TM_SKINNY_ROWS && L.K % 8 == 0 && fused_lds_fits(M, L.K) && aligned(resid, 16);
+// `most`: the most rows the family is preferred for at this model's width (tm_skinny_rows, tm_from_norm_rows)
+bool fused_decode_ok(const float* resid, const TmLinear& L, int M, int most) {
+    return resid && L.packed && M > 0 && M <= most && L.K % 8 == 0 && fused_lds_fits(M, L.K) && aligned(resid, 16);
 }
 
-bool packed_ok(const TmLinear& L, const void* x, int ldx, int M, int dtype) {
-    return L.packed && M > 0 && M <= TM_SKINNY_ROWS && dtype == TM_BF16 && L.dtype == TM_BF16 && L.K % 8 == 0 && ldx % 8 == 0 &&
+bool packed_ok(const TmLinear& L, const void* x, int ldx, int M, int dtype, int most) {
+    return L.packed && M > 0 && M <= most && dtype == TM_BF16 && L.dtype == TM_BF16 && L.K % 8 == 0 && ldx % 8 == 0 &&
            aligned(x, 16);
 }
 
@@ -77,14 +78,15 @@ bool skinny_ok(const TmLinear& L, const void* x, int ldx, int dtype) {
     return dtype == TM_BF16 && L.dtype == TM_BF16 && L.K % 8 == 0 && ldx % 8 == 0 && aligned(x, 16) && aligned(L.w, 16);
 }
 
-bool panel_ok(const TmLinear& L, const void* x, int ldx, int M, int dtype, int most_rows = TM_PANEL_ROWS) {
-    return L.packed && M > TM_SKINNY_ROWS && M <= most_rows && dtype == TM_BF16 && ldx % 8 == 0 && aligned(x, 16) &&
+// `beyond`: the rows up to which the kernels for at most 16 rows are preferred
+bool panel_ok(const TmLinear& L, const void* x, int ldx, int M, int dtype, int beyond, int most_rows = TM_PANEL_ROWS) {
+    return L.packed && M > beyond && M <= most_rows && dtype == TM_BF16 && ldx % 8 == 0 && aligned(x, 16) &&
            tm_gemm_panel_fits(M, L.K);
 }
 
 // the products that stream a packed matrix once for up to 64 tokens (gemm_stream.hip)
-bool stream_ok(const TmLinear& L, const void* x, int ldx, int M, int dtype) {
-    return L.packed && M > TM_SKINNY_ROWS && M <= TM_STREAM_ROWS && dtype == TM_BF16 && L.dtype == TM_BF16 && ldx % 8 == 0 &&
+bool stream_ok(const TmLinear& L, const void* x, int ldx, int M, int dtype, int beyond) {
+    return L.packed && M > beyond && M <= TM_STREAM_ROWS && dtype == TM_BF16 && L.dtype == TM_BF16 && ldx % 8 == 0 &&
            aligned(x, 16) && tm_gemm_stream_fits(M, L.K);
 }
 
@@ -96,6 +98,7 @@ struct Products {
     TmTune tune;
     float* wide_in = nullptr;           // room for a product's input and output in 32-bit (see TmProgram::max_wide_in)
     float* wide_out = nullptr;
+    int skinny_rows = TM_SKINNY_ROWS;   // rows up to which the packed products for at most 16 rows are preferred (tm_skinny_rows)
 
     int library(const TmLinear& L, const void* x, int ldx, int M, void* out, int ldc, int out_dtype) const {
         return tm_gemm_library(x, ldx, L.w, L.K, L.bias, L.bias_dtype, out, ldc, out_dtype == TM_F32, M, L.N, L.K, lib_ws,
@@ -115,7 +118,7 @@ struct Products {
             if ((rc = linear(L, TM_F32, wide_in, L.K, M, wide_out, L.N, TM_F32))) return rc;
             return tm_convert(wide_out, TM_F32, out, TM_BF16, (long long)M * L.N, stream);
         }
-        if (L.packed_parts == 1 && packed_ok(L, x, ldx, M, dtype) && !L.library_first)
+        if (L.packed_parts == 1 && packed_ok(L, x, ldx, M, dtype, skinny_rows) && !L.library_first)
             return tm_gemm_skinny_packed(x, ldx, L.packed, L.packed_rows, L.bias, L.bias_dtype, out, ldc, M, L.N, L.K,
                                          out_dtype, 0, nullptr, 0, stream);
         if (dtype != TM_BF16) {
@@ -153,12 +156,12 @@ struct Products {
     // Is there a kernel that adds round(x W^T + b) into a 32-bit accumulator in its epilogue?
     bool accumulates(const TmLinear& L, int dtype, const void* x, int ldx, int M) const {
         if (L.dtype != dtype || M <= 0) return false;
-        return (L.packed_parts == 1 && packed_ok(L, x, ldx, M, dtype)) ||
+        return (L.packed_parts == 1 && packed_ok(L, x, ldx, M, dtype, skinny_rows)) ||
                (M <= TM_SKINNY_ROWS && skinny_ok(L, x, ldx, dtype));
     }
 
     int accumulate(const TmLinear& L, int dtype, const void* x, int ldx, int M, float* accum, int ldacc) const {
-        if (L.packed_parts == 1 && packed_ok(L, x, ldx, M, dtype))
+        if (L.packed_parts == 1 && packed_ok(L, x, ldx, M, dtype, skinny_rows))
             return tm_gemm_skinny_packed(x, ldx, L.packed, L.packed_rows, L.bias, L.bias_dtype, nullptr, L.N, M, L.N, L.K, TM_BF16,
                                          0, accum, ldacc, stream);
         return tm_gemm_skinny(x, ldx, L.w, L.bias, L.bias_dtype, nullptr, L.N, M, L.N, L.K, TM_BF16, 0, accum, ldacc, stream);
@@ -171,6 +174,7 @@ struct Run {
     hipStream_t stream;
     Products products;
     int dtype;
+    int from_norm_rows;                 // rows up to which q|k|v and gate|up start at the norm (tm_from_norm_rows)
     bool labels;
     // what crosses between operations
     float* resid;
@@ -204,7 +208,7 @@ struct Run {
     int project(const TmLinear& L, const void* x_, int ldx, int M) {
         // 17 to 64 rows over a matrix with few rows of output: K split over groups of blocks, whose partial sums the
         // next norm adds up (or, where the caller wants the result itself, a small kernel)
-        const int groups = (sums && L.N == p->hidden && L.packed_parts == 1 && stream_ok(L, x_, ldx, M, dtype))
+        const int groups = (sums && L.N == p->hidden && L.packed_parts == 1 && stream_ok(L, x_, ldx, M, dtype, products.skinny_rows))
                                ? tm_stream_linear_parts(L.N, L.K) : 1;
         if (groups >= 2 && groups <= TM_MAX_SUMS) {
             const int rc = tm_stream_linear_split(x_, ldx, M, L.K, L.packed, L.packed_rows, L.N, L.bias, L.bias_dtype, sums, stream);
@@ -283,7 +287,7 @@ struct Run {
             const bool own_norm = x_in == nullptr;
             // 1. the kernel that starts at the norm (at most 16 tokens)
             if (own_norm && dtype == TM_BF16 && a.qkv.dtype == TM_BF16 && a.D % 32 == 0 && delta == nullptr && !pending_sums && a.norm.w &&
-                tables_fusable && fused_decode_ok(resid, a.qkv, T) && is_pow2(a.page) && bias_ok) {
+                tables_fusable && fused_decode_ok(resid, a.qkv, T, from_norm_rows) && is_pow2(a.page) && bias_ok) {
                 rc = tm_fused_norm_qkv_rope(resid, a.norm.w, a.norm.w_dtype, a.norm.eps, T, hidden, a.qkv.packed, a.qkv.bias,
                                             a.qkv.bias_dtype, qkv, a.H, a.KVH, a.D, a.cos_t, a.sin_t, s->positions, slots, kp, vp,
                                             a.page, stream);
@@ -298,14 +302,14 @@ struct Run {
                     xn = x;
                 }
                 // 2. the normed input kept in LDS (17 to 48 tokens)
-                if (tables_fusable && a.D % 32 == 0 && a.qkv.dtype == TM_BF16 && panel_ok(a.qkv, xn, hidden, T, dtype, TM_PANEL_QKV_ROWS) &&
+                if (tables_fusable && a.D % 32 == 0 && a.qkv.dtype == TM_BF16 && panel_ok(a.qkv, xn, hidden, T, dtype, from_norm_rows, TM_PANEL_QKV_ROWS) &&
                     is_pow2(a.page) && bias_ok) {
                     rc = tm_panel_qkv_rope(xn, hidden, T, hidden, a.qkv.packed, a.qkv.bias, a.qkv.bias_dtype, qkv, a.H, a.KVH, a.D,
                                            a.cos_t, a.sin_t, s->positions, slots, kp, vp, a.page, stream);
                     q = qkv;
                     q_stride = HD;
                     ++p->taken[TM_QKV_PANEL];
-                } else if (tables_fusable && a.D % 32 == 0 && a.qkv.packed_parts == 1 && stream_ok(a.qkv, xn, hidden, T, dtype) &&
+                } else if (tables_fusable && a.D % 32 == 0 && a.qkv.packed_parts == 1 && stream_ok(a.qkv, xn, hidden, T, dtype, from_norm_rows) &&
                            is_pow2(a.page)) {
                     // 3. the packed matrix streamed once for up to 64 tokens
                     rc = tm_stream_qkv_rope(xn, hidden, T, hidden, a.qkv.packed, a.qkv.packed_rows, a.qkv.bias, a.qkv.bias_dtype,
@@ -390,7 +394,7 @@ struct Run {
             const bool plain = f.gate_up.dtype == dtype && f.gate_up.bias == nullptr;
             const bool two_parts = f.gate_up.packed_parts == 2 && f.gate_up.packed_rows == 16;
             if (own_norm && dtype == TM_BF16 && plain && f.I % 4 == 0 && delta == nullptr && !pending_sums && f.norm.w && two_parts &&
-                fused_decode_ok(resid, f.gate_up, T)) {
+                fused_decode_ok(resid, f.gate_up, T, from_norm_rows)) {
                 rc = tm_fused_norm_gate_up_silu(resid, f.norm.w, f.norm.w_dtype, f.norm.eps, T, hidden, f.gate_up.packed, act, f.I, stream);
                 ++p->taken[TM_GATE_UP_FROM_NORM];
             } else {
@@ -400,19 +404,19 @@ struct Run {
                     if ((rc = normed(f.norm))) return rc;
                     xn = x;
                 }
-                if (plain && two_parts && packed_ok(f.gate_up, xn, hidden, T, dtype)) {
+                if (plain && two_parts && packed_ok(f.gate_up, xn, hidden, T, dtype, from_norm_rows)) {
                     rc = tm_gemm_skinny_packed(xn, hidden, f.gate_up.packed, 16, nullptr, TM_NONE, act, f.I, T, f.I, hidden, TM_BF16, 1,
                                                nullptr, 0, stream);
                     ++p->taken[TM_GATE_UP_PLAIN];
-                } else if (plain && T <= TM_SKINNY_ROWS && skinny_ok(f.gate_up, xn, hidden, dtype)) {
-                    rc = tm_gemm_skinny(xn, hidden, f.gate_up.w, nullptr, TM_NONE, act, f.I, T, f.I, hidden, TM_BF16, 1, nullptr, 0, stream);
-                    ++p->taken[TM_GATE_UP_PLAIN];
-                } else if (plain && two_parts && f.I % 4 == 0 && panel_ok(f.gate_up, xn, hidden, T, dtype)) {
+                } else if (plain && two_parts && f.I % 4 == 0 && panel_ok(f.gate_up, xn, hidden, T, dtype, from_norm_rows)) {
                     rc = tm_panel_gate_up_silu(xn, hidden, T, hidden, f.gate_up.packed, act, f.I, stream);
                     ++p->taken[TM_GATE_UP_PANEL];
-                } else if (plain && two_parts && f.I % 4 == 0 && stream_ok(f.gate_up, xn, hidden, T, dtype)) {
+                } else if (plain && two_parts && f.I % 4 == 0 && stream_ok(f.gate_up, xn, hidden, T, dtype, from_norm_rows)) {
                     rc = tm_stream_gate_up_silu(xn, hidden, T, hidden, f.gate_up.packed, act, f.I, stream);
                     ++p->taken[TM_GATE_UP_STREAM];
+                } else if (plain && T <= TM_SKINNY_ROWS && skinny_ok(f.gate_up, xn, hidden, dtype)) {   // (a matrix without a packed copy)
+                    rc = tm_gemm_skinny(xn, hidden, f.gate_up.w, nullptr, TM_NONE, act, f.I, T, f.I, hidden, TM_BF16, 1, nullptr, 0, stream);
+                    ++p->taken[TM_GATE_UP_PLAIN];
                 } else {
                     if ((rc = linear(f.gate_up, xn, hidden, T, gu, 2 * f.I, dtype))) return rc;
                     rc = tm_silu_mul(gu, act, dtype, T, f.I, stream);
@@ -582,6 +586,8 @@ int tm_program_run(const TmProgram* p, int first, int count, const TmStep* s, Tm
     r.products.stream = stream; r.products.lib_ws = library_workspace; r.products.lib_ws_bytes = library_workspace_bytes;
     r.products.tune = p->tune;
     if (flags & TM_RUN_TUNE_AT_ONCE) r.products.tune.after = 1;
+    r.products.skinny_rows = tm_skinny_rows(p->hidden);
+    r.from_norm_rows = tm_from_norm_rows(p->hidden);
     r.labels = (flags & TM_RUN_LABELS) != 0;
     r.resid = io->resid; r.delta = io->delta; r.x_in = io->x; r.qkv_in = io->qkv; r.accumulate = io->accumulate != 0;
     r.x = take((size_t)T * p->hidden * es);
