@@ -379,37 +379,38 @@ __global__ __launch_bounds__(64 * KS * US) void gemm_stream_kernel(const StreamA
 }
 
 // How a block is made for a matrix: KS wavefronts split a unit's K, US units share the activations in LDS. From
-// the matrix's shape alone (never from the number of tokens: that keeps a token's sums in one order). Many units
-// (gate|up): the units share, K is split little; few units over a long K (the down projection): K is split over
-// the whole block, so that the chip still has a few thousand wavefronts streaming.
+// the matrix's shape alone (never from the number of tokens: that keeps a token's sums in one order).
+//
+// A CU holds one block of these kernels (at 128 registers a lane a CU has room for 16 wavefronts), so a launch
+// should be one round of at most 256 blocks, as close to 256 as the units allow: US = the fewest units a block
+// that leave at most 256 blocks, and two wavefronts a unit from three units a block on (four with two units,
+// eight with one). Measured on an MI355X, 8 / 32 / 64 tokens (us): gate|up 7B (1,184 units) 2 x 5 = 237 blocks:
+// 53 / 50 / 55 (2 x 8 = 148 blocks: 58 / 61 / 68; 2 x 6: 54 / 53 / 57; 3 x 5: 48 / 50 / 78; 1 x 4 = 296 blocks: - / 60 / 73;
+// 4 x 4: - / 70 / 100); gate|up 32B (1,728 units) 2 x 8 = 216 blocks: 95 / 98 / 101 (2 x 7 = 247: 94 / 97 / 106, a few registers spilled; 2 x 6 = 288
+// blocks, a second round: 133 / 134 / 142; 1 x 4: - / 97 / 110); gate|up 0.5B (304 units) 4 x 2: - / 9 / 13 (8 x 1: - / 14 / 21);
+// q|k|v 7B (144 units) 8 x 1: - / 17 / 25 (4 x 2: - / 20 / 27).
 static void stream_config(int n_units, int* ks, int* us) {
-    // From the matrix alone (KS fixes the order of a token's sums). Measured on an MI355X at the 0.5B, 7B and 32B layer
-    // sizes, 17 / 32 / 48 / 64 tokens: gate|up 7B (1,184 units) 2 x 8: 63 / 61 / 66 / 63-67 us (1 x 4: 59 / 60 / 68 / 73,
-    // 1 x 8: - / 69 / - / 71, 2 x 4: 62 / 63 / 66 / 79, 2 x 2: - / 56 / - / 76, 4 x 4: - / 70 / - / 100, 1 x 16: - / 96 / - / 97),
-    // gate|up 32B (1,728 units) 2 x 8: 99 / 97 / 102 / 103 us (1 x 4: 96 / 97 / 104 / 109-112, 2 x 2: - / 110 / - / 130);
-    // gate|up 0.5B (304 units) 4 x 2: 9 / - / 12 us; q|k|v 7B (144 units) 8 x 1: 17 / - / 25 us (4 x 2: 20 / - / 27).
-    // With many units, sixteen wavefronts on eight units share one window of the activations: at 64 tokens every
-    // block's copy of the activations is half as many bytes as the matrix itself (1 x 4), a quarter with 2 x 8.
-    if (n_units >= 1024) { *ks = 2; *us = 8; }
-    else if (n_units >= 256) { *ks = 4; *us = 2; }
-    else { *ks = 8; *us = 1; }
+    int u = (n_units + 255) / 256;
+    if (u > 6) u = 8;                           // (seven units, 14 wavefronts, need a few registers more than the 128 there are)
+    *us = u;
+    *ks = u == 1 ? 8 : u == 2 ? 4 : 2;
 }
 
 // The same for a plain product whose K is split over `parts` groups of blocks, which leave 32-bit partial sums
 // (1: not split). From the matrix's shape alone.
 static void stream_plain_shape(int N, int K, int* parts, int* ks, int* us) {
     const int n_units = (N + 31) / 32, ksteps = (K + 31) / 32;
-    // Wide outputs over a K that gives every wavefront four k-steps: eight groups, two wavefronts a unit, and as many
-    // units a block as leave about 150 blocks. Measured on an MI355X, 17 / 32 / 48 / 64 tokens: 7B down (112 units,
-    // K 18,944) 8 groups of 2 x 4: 29 / 29 / 31 / 34 us (4 groups of 4 x 2: 31 / 30 / 35 / 39; 8 of 2 x 8: 36 / 36 / 39 / 42;
-    // unsplit 56 / 81 us at 32 / 64; the library's product with its algorithm chosen by timing 52 / 69); 7B o: 9.5 / 9.6 /
-    // 11.0 / 12.3 us (4 of 4 x 2: 9.7 / 9.8 / 11.8 / 13.0); 32B down (160 units, K 27,648) 8 groups of 2 x 8: 58 / 55 / 63 /
-    // 61 us (4 of 4 x 2: 64 / 65 / 84 / 92; 8 of 2 x 4: 61 / 61 / 74 / 78); 32B o: 15 / 15 / 17 / 18 us (4 of 4 x 2: 17 / 17 /
-    // 24 / 27).
+    // Wide outputs over a K that gives every wavefront four k-steps: eight groups of blocks, two wavefronts a unit, and
+    // the fewest units a block that leave at most 256 blocks. Measured on an MI355X, 8 / 32 / 64 tokens (us): 7B down
+    // (112 units, K 18,944) 8 groups of 2 x 4 = 224 blocks: 27 / 29 / 34 (3 x 4: 26 / 29 / 33; 4 x 4: 26 / 29 / 41; 4 groups
+    // of 4 x 2: - / 30 / 39; 8 of 2 x 8 = 112 blocks: - / 36 / 42; unsplit - / 56 / 81; the library's product with its
+    // algorithm chosen by timing - / 52 / 69); 7B o: 8 / 10 / 13 (4 groups of 4 x 2: - / 10 / 13); 32B down (160 units,
+    // K 27,648) 8 groups of 2 x 5 = 256 blocks: 52 / 51 / 57 (2 x 8 = 160 blocks: 56 / 58 / 65; 3 x 5: 51 / 52 / 143; 4 groups
+    // of 4 x 2: - / 65 / 92); 32B o: 12.5 / 14 / 17 (2 x 8: 14 / 16 / 19; 4 groups of 4 x 2: - / 17 / 27).
     if (n_units >= 96 && ksteps >= 64) {
         *parts = 8;
         *ks = 2;
-        *us = n_units >= 144 ? 8 : 4;
+        *us = (n_units + 31) / 32 < 7 ? (n_units + 31) / 32 : 8;
         return;
     }
     // Narrow outputs: the fewest groups (a power of two, at most 8) that give the matrix about 400 blocks' worth of
@@ -443,7 +444,10 @@ static int launch_stream_tiles(const StreamArgs& a, int n_units, int kparts, int
     switch (ks * 16 + us) {                     // the shapes stream_config and stream_plain_shape name
         case 4 * 16 + 2: return launch_stream_config<EPI, NT, 4, 2>(a, n_units, kparts, stream);
         case 8 * 16 + 1: return launch_stream_config<EPI, NT, 8, 1>(a, n_units, kparts, stream);
+        case 2 * 16 + 3: return launch_stream_config<EPI, NT, 2, 3>(a, n_units, kparts, stream);
         case 2 * 16 + 4: return launch_stream_config<EPI, NT, 2, 4>(a, n_units, kparts, stream);
+        case 2 * 16 + 5: return launch_stream_config<EPI, NT, 2, 5>(a, n_units, kparts, stream);
+        case 2 * 16 + 6: return launch_stream_config<EPI, NT, 2, 6>(a, n_units, kparts, stream);
         case 2 * 16 + 8: return launch_stream_config<EPI, NT, 2, 8>(a, n_units, kparts, stream);
         default: return TM_ERR_ARG;
     }
