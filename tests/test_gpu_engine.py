@@ -159,10 +159,10 @@ def test_same_tokens_under_every_cutting_and_a_starved_pool(model_dirs, plains, 
         assert outs == base
 
 
-def test_steps_of_17_to_48_tokens_take_the_panel_products(model_dirs, plains):
-    """24 requests decoding together, and prompt steps of 20 to 40 tokens: the q|k|v and gate|up products
-    that keep the normed input in LDS run (counted by the step program), and every token is the plain
-    implementation's."""
+def test_steps_of_17_to_48_tokens_take_the_panel_and_stream_products(model_dirs, plains):
+    """24 requests decoding together, and prompt steps of 20 to 40 tokens: the q|k|v product that keeps the normed
+    input in LDS and the gate|up product that streams its matrix run (counted by the step program), and every token
+    is the plain implementation's."""
     from tokenmill_amd import SamplingParams
     prompts = [random_ids(1 + (7 * i) % 19, 384, 300 + i) for i in range(24)]
     layers = 3
@@ -173,7 +173,7 @@ def test_steps_of_17_to_48_tokens_take_the_panel_products(model_dirs, plains):
         assert len(o) == 10
         verify(plains["B"], p, o, torch.bfloat16)
     took = eng.runner.program.counters()
-    assert took["qkv_panel"] >= 9 * layers and took["gate_up_panel"] == took["qkv_panel"]      # the decode steps of 24 tokens at least
+    assert took["qkv_panel"] >= 9 * layers and took["gate_up_stream"] == took["qkv_panel"]     # the decode steps of 24 tokens at least
     assert eng.cache.num_free_pages == eng.cache.num_pages
 
 

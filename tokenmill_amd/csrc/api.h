@@ -72,7 +72,6 @@ int tm_gemm_panel_fits(int M, int K);
 int tm_panel_qkv_rope(const void* X, int ldx, int M, int K, const void* W, const void* bias, int bias_dtype, void* q_out,
                       int H, int KVH, int D, const float* cos_t, const float* sin_t, const int* positions,
                       const int* slots, void* k_pool, void* v_pool, int page, hipStream_t stream);
-int tm_panel_gate_up_silu(const void* X, int ldx, int M, int K, const void* W, void* act_out, int I, hipStream_t stream);
 
 // The same products for up to 64 tokens at any width (K a multiple of 8), the matrix streamed once from its packed
 // copy in strips of `rows` rows (16, 8 or 4), and the plain product with bias whose result is stored or, rounded to

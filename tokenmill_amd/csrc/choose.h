@@ -20,10 +20,11 @@ inline int tm_skinny_rows(int hidden) { return hidden < 2048 ? TM_SKINNY_ROWS : 
 // ... and the two of them that start at the norm (q|k|v, gate|up) at most to 8 rows: with 9 to 16 rows in LDS a CU
 // holds one block (0.5B shape, 16 rows: 1.195 ms a step against 1.156 with the panel kernels behind a norm of its own)
 inline int tm_from_norm_rows(int hidden) { const int s = tm_skinny_rows(hidden); return s < 8 ? s : 8; }
-// up to this many rows gate|up keeps the normed input in LDS (where it fits) and carries its epilogue; q|k|v, whose
-// matrix is small enough that the copy of the input is most of the kernel's work, does so for every row count the
-// panel kernels take (measured at the 0.5B shape, 64 rows: 10.9 us against 14.9 us streamed)
-constexpr int TM_PANEL_ROWS = 48;
+// q|k|v keeps the normed input in LDS behind a norm of its own up to this many rows where it fits (a width of at
+// most 1,024): its matrix is small enough that the copy of the input is most of any kernel's work (measured at the
+// 0.5B shape, 64 rows: 10.9 us against 14.9 us streamed). gate|up had such a kernel too; the stream product, with
+// the tiles of tokens dealt to two groups of blocks beyond 32 rows, is as fast or faster at every row count (0.5B
+// shape, a decode step of 12 / 24 / 32 / 48 requests: 1.07 / 1.29 / 1.34 / 1.54 ms against 1.08 / 1.32 / 1.38 / 1.54 ms).
 constexpr int TM_PANEL_QKV_ROWS = 64;
 // up to this many rows the products stream the packed matrix once for several row tiles, with their epilogues
 constexpr int TM_STREAM_ROWS = 64;

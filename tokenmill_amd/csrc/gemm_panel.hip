@@ -1,5 +1,5 @@
-// The q|k|v and gate|up products of a decode step with 17 to 64 tokens, each with its layer's own
-// epilogue (bias + rotary + cache write; SiLU·up), behind a norm that ran as a kernel of its own.
+// The q|k|v product of a decode step with 9 to 64 tokens of a narrow model (a width of at most 1,024), with
+// its layer's own epilogue (bias + rotary + cache write), behind a norm that ran as a kernel of its own.
 //
 // With this many rows a block cannot afford to compute the norm itself (every block would read all
 // rows of the residual stream), and it cannot read its activations from the cache k-step by k-step
@@ -11,7 +11,7 @@
 // through LDS in wavefront order, and wavefront t does the epilogue of row tile t.
 //
 // The matrix is read in strip order (tm_pack_layout in api.h) like the decode kernels for fewer rows,
-// the strips pair up the same way (the two halves of a rotary pair; gate and up), and everything is
+// the strips pair up the same way (the two halves of a rotary pair), and everything is
 // rounded where the unfused path stores a bfloat16 tensor, so both paths agree up to the order of
 // 32-bit sums (reference src/infer/model/layers.py:142-147,60-64,163-164; src/infer/kv/paged_cache.py:40-43).
 // Which k goes to which wavefront depends on K alone: a token's result does not depend on how many
@@ -23,11 +23,13 @@
 #define PN_WAVES 4
 #define PN_KCH 8            // k-steps a wavefront holds: K <= 4 * 8 * 32 = 1024
 
-// NT: 16-row tiles of x (2..4). ROWS: rows of a matrix strip (16 or 8).
-template <int EPI, int ROWS, int NT>
+// NT: 16-row tiles of x a block takes (1..4). ROWS: rows of a matrix strip (16 or 8).
+template <int ROWS, int NT>
 __global__ __launch_bounds__(64 * PN_WAVES, 1) void gemm_panel_kernel(const FusedArgs a, const int n_units) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    const int K = a.K, M = a.M;
+    // the tokens of this block: all of them, or (gridDim.y > 1) the NT tiles from tok0 on
+    const int tok0 = blockIdx.y * (NT * 16);
+    const int K = a.K, M = a.M - tok0 < NT * 16 ? a.M - tok0 : NT * 16;
     const int xstride = K + FD_XPAD;
     bf16_t* xs = (bf16_t*)smem_raw;                                  // [NT * 16][K + FD_XPAD]
     float* red = (float*)(smem_raw + (size_t)NT * 16 * xstride * sizeof(bf16_t));   // [waves][2][NT][64][5]
@@ -40,7 +42,7 @@ __global__ __launch_bounds__(64 * PN_WAVES, 1) void gemm_panel_kernel(const Fuse
     const int ks0 = wave * per;
     const int ks1 = ks0 + per < ksteps ? ks0 + per : ksteps;
     int u = blockIdx.x;
-    FusedUnit cu = fused_unit_of<EPI, ROWS>(a, u, r);
+    FusedUnit cu = fused_unit_of<FD_EPI_QKV, ROWS>(a, u, r);
 
     // This wavefront's epilogue is that of row tile `wave`: token 16 wave + r. Its position comes by
     // scalar loads (addresses the same in every lane), which are counted apart from the vector loads.
@@ -49,14 +51,12 @@ __global__ __launch_bounds__(64 * PN_WAVES, 1) void gemm_panel_kernel(const Fuse
     const bool epi_wave = tile < NT;
     const bool epi_lane = epi_wave && tok < M && 4 * g < ROWS;
     int tok_pos = 0;
-    if constexpr (EPI == FD_EPI_QKV) {
-        if (epi_wave) {
+    if (epi_wave) {
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const int ti = 16 * tile + i;
-                const int pos_i = a.positions[ti < M ? ti : 0];
-                tok_pos = r == i ? pos_i : tok_pos;
-            }
+        for (int i = 0; i < 16; ++i) {
+            const int ti = 16 * tile + i;
+            const int pos_i = a.positions[tok0 + (ti < M ? ti : 0)];
+            tok_pos = r == i ? pos_i : tok_pos;
         }
     }
 
@@ -88,22 +88,20 @@ __global__ __launch_bounds__(64 * PN_WAVES, 1) void gemm_panel_kernel(const Fuse
     const int bias_kind = !a.bias ? 0 : (a.bias_f32 ? 2 : 1);
     auto epilogue_inputs = [&](const FusedUnit& t) {
         EpilogueInputs e;
-        if constexpr (EPI == FD_EPI_QKV) {
-            const int ge = 4 * g < ROWS ? 4 * g : 0;
-            const int ia = t.nA + ge, ib = t.nB + ge;
-            if (bias_kind == 2) {
-                e.bias_f[0] = *(const f32x4_t*)((const float*)a.bias + ia);
-                e.bias_f[1] = *(const f32x4_t*)((const float*)a.bias + ib);
-            } else if (bias_kind == 1) {
-                e.bias_h[0] = *(const uint2*)((const bf16_t*)a.bias + ia);
-                e.bias_h[1] = *(const uint2*)((const bf16_t*)a.bias + ib);
-            }
-            const int jt = t.head < a.H + a.KVH ? t.jt : 0;          // value heads have no rotary row
-            const size_t at = (size_t)tok_pos * (a.D / 2) + ROWS * jt + ge;
-            e.cos = *(const f32x4_t*)(a.cos_t + at);
-            e.sin = *(const f32x4_t*)(a.sin_t + at);
-            e.slot = (a.slots ? a.slots : a.positions)[tok < M ? tok : 0];
+        const int ge = 4 * g < ROWS ? 4 * g : 0;
+        const int ia = t.nA + ge, ib = t.nB + ge;
+        if (bias_kind == 2) {
+            e.bias_f[0] = *(const f32x4_t*)((const float*)a.bias + ia);
+            e.bias_f[1] = *(const f32x4_t*)((const float*)a.bias + ib);
+        } else if (bias_kind == 1) {
+            e.bias_h[0] = *(const uint2*)((const bf16_t*)a.bias + ia);
+            e.bias_h[1] = *(const uint2*)((const bf16_t*)a.bias + ib);
         }
+        const int jt = t.head < a.H + a.KVH ? t.jt : 0;          // value heads have no rotary row
+        const size_t at = (size_t)tok_pos * (a.D / 2) + ROWS * jt + ge;
+        e.cos = *(const f32x4_t*)(a.cos_t + at);
+        e.sin = *(const f32x4_t*)(a.sin_t + at);
+        e.slot = (a.slots ? a.slots : a.positions)[tok0 + (tok < M ? tok : 0)];
         return e;
     };
     EpilogueInputs e_next = epilogue_inputs(cu);
@@ -122,7 +120,7 @@ __global__ __launch_bounds__(64 * PN_WAVES, 1) void gemm_panel_kernel(const Fuse
             const int pc = p < pieces ? p : 0;
             int row = pc / per_row + row_shift;
             row = row < M ? row : row - M;
-            v[i] = *(const u32x4_t*)(a.X + (size_t)row * a.ldx + (pc % per_row) * 8);
+            v[i] = *(const u32x4_t*)(a.X + (size_t)(tok0 + row) * a.ldx + (pc % per_row) * 8);
         }
 #pragma unroll
         for (int i = 0; i < XL; ++i) {
@@ -173,7 +171,7 @@ __global__ __launch_bounds__(64 * PN_WAVES, 1) void gemm_panel_kernel(const Fuse
         const bool more = un < n_units;
         const FusedUnit done = cu;
         if (more) {
-            cu = fused_unit_of<EPI, ROWS>(a, un, r);
+            cu = fused_unit_of<FD_EPI_QKV, ROWS>(a, un, r);
             wA = strip_pointer(cu.sA);
             wB = strip_pointer(cu.sB);
             load_group();
@@ -194,68 +192,50 @@ __global__ __launch_bounds__(64 * PN_WAVES, 1) void gemm_panel_kernel(const Fuse
                 sB[i] = vb;
             }
             // lane: token tok, rows nA + 4g + i and nB + 4g + i
-            if (EPI == FD_EPI_SILU) {
-                const int col = done.nA + 4 * g;
-                if (col < a.I) {
-                    float v[4];
+            f32x4_t bA = {0.f, 0.f, 0.f, 0.f}, bB = {0.f, 0.f, 0.f, 0.f};
+            if (bias_kind == 2) {
+                bA = e.bias_f[0];
+                bB = e.bias_f[1];
+            } else if (bias_kind == 1) {
+                bA = f32x4_t{__uint_as_float(e.bias_h[0].x << 16), __uint_as_float(e.bias_h[0].x & 0xffff0000u),
+                             __uint_as_float(e.bias_h[0].y << 16), __uint_as_float(e.bias_h[0].y & 0xffff0000u)};
+                bB = f32x4_t{__uint_as_float(e.bias_h[1].x << 16), __uint_as_float(e.bias_h[1].x & 0xffff0000u),
+                             __uint_as_float(e.bias_h[1].y << 16), __uint_as_float(e.bias_h[1].y & 0xffff0000u)};
+            }
+            float xA[4], xB[4];
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const float gt = fd_round(sA[i]), up = fd_round(sB[i]);
-                        v[i] = gt / (1.f + expf(-gt)) * up;
-                    }
-                    bf16_t* dst = a.act_out + (size_t)tok * a.I + col;
-                    if (col + 4 <= a.I) {
-                        *(uint2*)dst = uint2{fd_pack(v[0], v[1]), fd_pack(v[2], v[3])};
-                    } else {
-                        for (int i = 0; i < 4 && col + i < a.I; ++i) dst[i] = f32_to_bf16(v[i]);
-                    }
-                }
-            } else {
-                f32x4_t bA = {0.f, 0.f, 0.f, 0.f}, bB = {0.f, 0.f, 0.f, 0.f};
-                if (bias_kind == 2) {
-                    bA = e.bias_f[0];
-                    bB = e.bias_f[1];
-                } else if (bias_kind == 1) {
-                    bA = f32x4_t{__uint_as_float(e.bias_h[0].x << 16), __uint_as_float(e.bias_h[0].x & 0xffff0000u),
-                                 __uint_as_float(e.bias_h[0].y << 16), __uint_as_float(e.bias_h[0].y & 0xffff0000u)};
-                    bB = f32x4_t{__uint_as_float(e.bias_h[1].x << 16), __uint_as_float(e.bias_h[1].x & 0xffff0000u),
-                                 __uint_as_float(e.bias_h[1].y << 16), __uint_as_float(e.bias_h[1].y & 0xffff0000u)};
-                }
-                float xA[4], xB[4];
+            for (int i = 0; i < 4; ++i) {
+                xA[i] = fd_round(sA[i] + bA[i]);
+                xB[i] = fd_round(sB[i] + bB[i]);
+            }
+            const int slot = a.slots ? e.slot : -1;
+            if (done.head < a.H + a.KVH) {
+                const int half = a.D / 2;
+                const int j0 = ROWS * done.jt + 4 * g;                       // pair index of element 0
+                float y1[4], y2[4];
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    xA[i] = fd_round(sA[i] + bA[i]);
-                    xB[i] = fd_round(sB[i] + bB[i]);
+                    y1[i] = xA[i] * e.cos[i] - xB[i] * e.sin[i];
+                    y2[i] = xB[i] * e.cos[i] + xA[i] * e.sin[i];
                 }
-                const int slot = a.slots ? e.slot : -1;
-                if (done.head < a.H + a.KVH) {
-                    const int half = a.D / 2;
-                    const int j0 = ROWS * done.jt + 4 * g;                       // pair index of element 0
-                    float y1[4], y2[4];
+                bf16_t* dst = nullptr;
+                if (done.head < a.H)
+                    dst = a.q_out + (size_t)(tok0 + tok) * a.H * a.D + (size_t)done.head * a.D + j0;
+                else if (slot >= 0)
+                    dst = a.k_pool + ((size_t)slot * a.KVH + (done.head - a.H)) * a.D + j0;
+                if (dst) {
+                    *(uint2*)dst = uint2{fd_pack(y1[0], y1[1]), fd_pack(y1[2], y1[3])};
+                    *(uint2*)(dst + half) = uint2{fd_pack(y2[0], y2[1]), fd_pack(y2[2], y2[3])};
+                }
+            } else if (slot >= 0) {
+                const int vh = done.head - a.H - a.KVH;
+                const int pg = slot >> a.page_shift, in_page = slot & ((1 << a.page_shift) - 1);
+                const int d0 = 2 * ROWS * done.jt + 4 * g;
+                bf16_t* dst = a.v_pool + ((((size_t)pg * a.KVH + vh) * a.D + d0) << a.page_shift) + in_page;
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        y1[i] = xA[i] * e.cos[i] - xB[i] * e.sin[i];
-                        y2[i] = xB[i] * e.cos[i] + xA[i] * e.sin[i];
-                    }
-                    bf16_t* dst = nullptr;
-                    if (done.head < a.H)
-                        dst = a.q_out + (size_t)tok * a.H * a.D + (size_t)done.head * a.D + j0;
-                    else if (slot >= 0)
-                        dst = a.k_pool + ((size_t)slot * a.KVH + (done.head - a.H)) * a.D + j0;
-                    if (dst) {
-                        *(uint2*)dst = uint2{fd_pack(y1[0], y1[1]), fd_pack(y1[2], y1[3])};
-                        *(uint2*)(dst + half) = uint2{fd_pack(y2[0], y2[1]), fd_pack(y2[2], y2[3])};
-                    }
-                } else if (slot >= 0) {
-                    const int vh = done.head - a.H - a.KVH;
-                    const int pg = slot >> a.page_shift, in_page = slot & ((1 << a.page_shift) - 1);
-                    const int d0 = 2 * ROWS * done.jt + 4 * g;
-                    bf16_t* dst = a.v_pool + ((((size_t)pg * a.KVH + vh) * a.D + d0) << a.page_shift) + in_page;
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        dst[(size_t)i << a.page_shift] = f32_to_bf16(xA[i]);
-                        dst[(size_t)(i + ROWS) << a.page_shift] = f32_to_bf16(xB[i]);
-                    }
+                for (int i = 0; i < 4; ++i) {
+                    dst[(size_t)i << a.page_shift] = f32_to_bf16(xA[i]);
+                    dst[(size_t)(i + ROWS) << a.page_shift] = f32_to_bf16(xB[i]);
                 }
             }
         }
@@ -276,30 +256,36 @@ extern "C" int tm_gemm_panel_fits(int M, int K) {
     return panel_lds_bytes((M + 15) / 16, K) + 1024 <= 160 * 1024 ? 1 : 0;
 }
 
-template <int EPI, int ROWS, int NT>
-static int launch_panel_tiles(const FusedArgs& a, int n_units, int blocks, hipStream_t stream) {
+template <int ROWS, int NT>
+static int launch_panel_tiles(const FusedArgs& a, int n_units, int blocks, int row_parts, hipStream_t stream) {
     const int lds = panel_lds_bytes(NT, a.K);
     static int raised = 0;          // largest dynamic LDS size this kernel has been allowed so far
     if (lds > 48 * 1024 && lds > raised) {
-        if (hipFuncSetAttribute((const void*)gemm_panel_kernel<EPI, ROWS, NT>, hipFuncAttributeMaxDynamicSharedMemorySize,
+        if (hipFuncSetAttribute((const void*)gemm_panel_kernel<ROWS, NT>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                 lds) != hipSuccess)
             return TM_ERR_LAUNCH;
         raised = lds;
     }
-    gemm_panel_kernel<EPI, ROWS, NT><<<blocks, 64 * PN_WAVES, lds, stream>>>(a, n_units);
+    gemm_panel_kernel<ROWS, NT><<<dim3(blocks, row_parts), 64 * PN_WAVES, lds, stream>>>(a, n_units);
     TM_CHECK_LAUNCH();
     return TM_OK;
 }
 
-template <int EPI, int ROWS>
+template <int ROWS>
 static int launch_panel(const FusedArgs& a, int n_units, hipStream_t stream) {
-    // one block a CU (x fills most of its LDS): beyond that a block takes several units after one copy of x
+    // one block a CU (x fills most of its LDS): beyond that a block takes several units after one copy of x. With
+    // fewer units than half the chip's CUs the tiles of tokens are dealt to groups of blocks (the matrix is small:
+    // read again from the cache), as many groups as still give at most a block a CU.
     const int blocks = n_units < 256 ? n_units : 256;
-    switch ((a.M + 15) / 16) {
-        case 1: return launch_panel_tiles<EPI, ROWS, 1>(a, n_units, blocks, stream);
-        case 2: return launch_panel_tiles<EPI, ROWS, 2>(a, n_units, blocks, stream);
-        case 3: return launch_panel_tiles<EPI, ROWS, 3>(a, n_units, blocks, stream);
-        default: return launch_panel_tiles<EPI, ROWS, 4>(a, n_units, blocks, stream);
+    const int all_tiles = (a.M + 15) / 16, room = 256 / blocks;
+    int row_parts = room < all_tiles ? room : all_tiles;
+    const int tiles = (all_tiles + row_parts - 1) / row_parts;
+    row_parts = (all_tiles + tiles - 1) / tiles;
+    switch (tiles) {
+        case 1: return launch_panel_tiles<ROWS, 1>(a, n_units, blocks, row_parts, stream);
+        case 2: return launch_panel_tiles<ROWS, 2>(a, n_units, blocks, row_parts, stream);
+        case 3: return launch_panel_tiles<ROWS, 3>(a, n_units, blocks, row_parts, stream);
+        default: return launch_panel_tiles<ROWS, 4>(a, n_units, blocks, row_parts, stream);
     }
 }
 
@@ -328,19 +314,6 @@ extern "C" int tm_panel_qkv_rope(const void* X, int ldx, int M, int K, const voi
     a.page_shift = 0;
     while ((1 << a.page_shift) < page) ++a.page_shift;
     const int units16 = (H + 2 * KVH) * (D / 32);
-    if (tm_fused_qkv_strip_rows(H, KVH, D, K) == 16) return launch_panel<FD_EPI_QKV, 16>(a, units16, stream);
-    return launch_panel<FD_EPI_QKV, 8>(a, 2 * units16, stream);
-}
-
-// act[M, I] <- silu(X Wg^T) * (X Wu^T) for up to 64 tokens; W as for tm_fused_norm_gate_up_silu.
-extern "C" int tm_panel_gate_up_silu(const void* X, int ldx, int M, int K, const void* W, void* act_out, int I,
-                                     hipStream_t stream) {
-    if (M == 0) return TM_OK;
-    if (!panel_common_ok(M, K, X, ldx, W) || I <= 0 || !act_out || ((uintptr_t)act_out % 8) || (I % 4)) return TM_ERR_ARG;
-    FusedArgs a{};
-    a.X = (const bf16_t*)X; a.ldx = ldx; a.M = M; a.K = K;
-    a.W = (const bf16_t*)W; a.act_out = (bf16_t*)act_out; a.I = I;
-    const int units = (I + 15) / 16;
-    a.up_strip0 = units;
-    return launch_panel<FD_EPI_SILU, 16>(a, units, stream);
+    if (tm_fused_qkv_strip_rows(H, KVH, D, K) == 16) return launch_panel<16>(a, units16, stream);
+    return launch_panel<8>(a, 2 * units16, stream);
 }

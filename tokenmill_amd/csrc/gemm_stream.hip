@@ -103,7 +103,9 @@ __global__ __launch_bounds__(64 * KS * US) void gemm_stream_kernel(const StreamA
     constexpr int ROWS_X = NT * 16;
     bf16_t* xs = (bf16_t*)smem_raw;                                  // [KS][ROWS_X][XROW]
     const FusedArgs& f = a.f;
-    const int K = f.K, M = f.M;
+    // the tokens of this block: all of them, or (gridDim.z > 1) the NT tiles from tok0 on
+    const int tok0 = blockIdx.z * (NT * 16);
+    const int K = f.K, M = f.M - tok0 < NT * 16 ? f.M - tok0 : NT * 16;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / TM_WAVE), lane = threadIdx.x % TM_WAVE;
     const int kw = wave % KS, uw = wave / KS;                        // which range of K, which unit of the block
     const int r = lane % 16, g = lane / 16;
@@ -145,7 +147,7 @@ __global__ __launch_bounds__(64 * KS * US) void gemm_stream_kernel(const StreamA
             const int row = in / PIECES_ROW, piece = in % PIECES_ROW;
             int k = (k_begin + (win < KS ? win : KS - 1) * per + round * ST_KCH) * 32 + piece * 8;
             k = k + 8 <= k_end ? k : 0;                               // beyond the row: a piece that exists (zeroed when stored)
-            xv[i] = *(const u32x4_t*)(f.X + (size_t)(row < M ? row : M - 1) * f.ldx + k);
+            xv[i] = *(const u32x4_t*)(f.X + (size_t)(tok0 + (row < M ? row : M - 1)) * f.ldx + k);
         }
     };
     auto store_x = [&](int round) {
@@ -178,7 +180,7 @@ __global__ __launch_bounds__(64 * KS * US) void gemm_stream_kernel(const StreamA
     float pre_bA[4] = {0.f, 0.f, 0.f, 0.f}, pre_bB[4] = {0.f, 0.f, 0.f, 0.f};
     f32x4_t pre_cs = {0.f, 0.f, 0.f, 0.f}, pre_sn = {0.f, 0.f, 0.f, 0.f};
     if constexpr (PRE) {
-        const int tok = 16 * kw + r < M ? 16 * kw + r : M - 1;       // (tile kw may not exist: a token that does)
+        const int tok = tok0 + (16 * kw + r < M ? 16 * kw + r : M - 1);    // (tile kw may not exist: a token that does)
         pre_pos = f.positions[tok];
         pre_slot = f.slots ? f.slots[tok] : -1;
         if (f.bias) {
@@ -250,8 +252,8 @@ __global__ __launch_bounds__(64 * KS * US) void gemm_stream_kernel(const StreamA
         }
         __syncthreads();
         if (kw != t % KS || !have_unit) continue;
-        const int tok = 16 * t + r;
-        if (tok >= M) continue;
+        if (16 * t + r >= M) continue;
+        const int tok = tok0 + 16 * t + r;
         float sA[4], sB[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -346,7 +348,7 @@ __global__ __launch_bounds__(64 * KS * US) void gemm_stream_kernel(const StreamA
                 }
                 const bool whole = nf + 4 <= a.N;
                 if (a.parts) {          // this block's share of K: 32-bit, unrounded, for whoever adds the parts up
-                    float* dst = a.parts + ((size_t)blockIdx.y * M + tok) * a.N + nf;
+                    float* dst = a.parts + ((size_t)blockIdx.y * f.M + tok) * a.N + nf;
                     if (whole && (a.N % 4) == 0) {
                         *(f32x4_t*)dst = f32x4_t{v[0], v[1], v[2], v[3]};
                     } else {
@@ -425,7 +427,7 @@ static void stream_plain_shape(int N, int K, int* parts, int* ks, int* us) {
 }
 
 template <int EPI, int NT, int KS, int US>
-static int launch_stream_config(const StreamArgs& a, int n_units, int kparts, hipStream_t stream) {
+static int launch_stream_config(const StreamArgs& a, int n_units, int kparts, int row_parts, hipStream_t stream) {
     constexpr int lds = stream_lds_bytes(NT, KS, US);
     static bool raised = false;
     if (lds > 48 * 1024 && !raised) {
@@ -434,21 +436,21 @@ static int launch_stream_config(const StreamArgs& a, int n_units, int kparts, hi
             return TM_ERR_LAUNCH;
         raised = true;
     }
-    gemm_stream_kernel<EPI, NT, KS, US><<<dim3((n_units + US - 1) / US, kparts), 64 * KS * US, lds, stream>>>(a, n_units);
+    gemm_stream_kernel<EPI, NT, KS, US><<<dim3((n_units + US - 1) / US, kparts, row_parts), 64 * KS * US, lds, stream>>>(a, n_units);
     TM_CHECK_LAUNCH();
     return TM_OK;
 }
 
 template <int EPI, int NT>
-static int launch_stream_tiles(const StreamArgs& a, int n_units, int kparts, int ks, int us, hipStream_t stream) {
+static int launch_stream_tiles(const StreamArgs& a, int n_units, int kparts, int row_parts, int ks, int us, hipStream_t stream) {
     switch (ks * 16 + us) {                     // the shapes stream_config and stream_plain_shape name
-        case 4 * 16 + 2: return launch_stream_config<EPI, NT, 4, 2>(a, n_units, kparts, stream);
-        case 8 * 16 + 1: return launch_stream_config<EPI, NT, 8, 1>(a, n_units, kparts, stream);
-        case 2 * 16 + 3: return launch_stream_config<EPI, NT, 2, 3>(a, n_units, kparts, stream);
-        case 2 * 16 + 4: return launch_stream_config<EPI, NT, 2, 4>(a, n_units, kparts, stream);
-        case 2 * 16 + 5: return launch_stream_config<EPI, NT, 2, 5>(a, n_units, kparts, stream);
-        case 2 * 16 + 6: return launch_stream_config<EPI, NT, 2, 6>(a, n_units, kparts, stream);
-        case 2 * 16 + 8: return launch_stream_config<EPI, NT, 2, 8>(a, n_units, kparts, stream);
+        case 4 * 16 + 2: return launch_stream_config<EPI, NT, 4, 2>(a, n_units, kparts, row_parts, stream);
+        case 8 * 16 + 1: return launch_stream_config<EPI, NT, 8, 1>(a, n_units, kparts, row_parts, stream);
+        case 2 * 16 + 3: return launch_stream_config<EPI, NT, 2, 3>(a, n_units, kparts, row_parts, stream);
+        case 2 * 16 + 4: return launch_stream_config<EPI, NT, 2, 4>(a, n_units, kparts, row_parts, stream);
+        case 2 * 16 + 5: return launch_stream_config<EPI, NT, 2, 5>(a, n_units, kparts, row_parts, stream);
+        case 2 * 16 + 6: return launch_stream_config<EPI, NT, 2, 6>(a, n_units, kparts, row_parts, stream);
+        case 2 * 16 + 8: return launch_stream_config<EPI, NT, 2, 8>(a, n_units, kparts, row_parts, stream);
         default: return TM_ERR_ARG;
     }
 }
@@ -457,11 +459,21 @@ static int launch_stream_tiles(const StreamArgs& a, int n_units, int kparts, int
 template <int EPI>
 static int launch_stream(const StreamArgs& a, int n_units, hipStream_t stream, int kparts = 1, int ks = 0, int us = 0) {
     if (ks == 0) stream_config(n_units, &ks, &us);
-    switch ((a.f.M + 15) / 16) {
-        case 1: return launch_stream_tiles<EPI, 1>(a, n_units, kparts, ks, us, stream);
-        case 2: return launch_stream_tiles<EPI, 2>(a, n_units, kparts, ks, us, stream);
-        case 3: return launch_stream_tiles<EPI, 3>(a, n_units, kparts, ks, us, stream);
-        default: return launch_stream_tiles<EPI, 4>(a, n_units, kparts, ks, us, stream);
+    int tiles = (a.f.M + 15) / 16, row_parts = 1;
+    // gate|up over a matrix small enough that reading it twice from the cache costs little, in blocks of 8 wavefronts
+    // of which a CU holds two when they carry two tiles of tokens (124 registers instead of 164): the further tiles
+    // go to blocks of their own (0.5B shape, a decode step of 48 / 64 requests 1.65 / 1.88 to 1.54 / 1.73 ms together
+    // with the same for q|k|v in gemm_panel.hip; at the 7B shape's q|k|v, whose matrix is 33 MB, it lost: 25 us
+    // against 20 us at 64 rows)
+    if (EPI == ST_EPI_SILU && ks * us <= 8 && n_units <= 512 && tiles > 2) {
+        row_parts = 2;
+        tiles = 2;
+    }
+    switch (tiles) {
+        case 1: return launch_stream_tiles<EPI, 1>(a, n_units, kparts, row_parts, ks, us, stream);
+        case 2: return launch_stream_tiles<EPI, 2>(a, n_units, kparts, row_parts, ks, us, stream);
+        case 3: return launch_stream_tiles<EPI, 3>(a, n_units, kparts, row_parts, ks, us, stream);
+        default: return launch_stream_tiles<EPI, 4>(a, n_units, kparts, row_parts, ks, us, stream);
     }
 }
 

@@ -101,7 +101,6 @@ enum {
     TM_QKV_STREAM,              // ... by the kernel that streams the packed matrix for up to 64 tokens
     TM_QKV_PLAIN,               // ... by a product, then rotation and cache write
     TM_GATE_UP_FROM_NORM,
-    TM_GATE_UP_PANEL,
     TM_GATE_UP_STREAM,
     TM_GATE_UP_PLAIN,           // a product with the SiLU*up epilogue, or a product and then SiLU*up
     TM_PREFILL_SPLIT_KEYS,      // bfloat16 attention of prompt portions: wavefronts split a tile's key blocks
@@ -146,7 +145,7 @@ int tm_linear_run(const TmLinear* L, int x_dtype, const void* x, int ldx, int M,
                   float* accum, int ldacc, void* library_workspace, size_t library_workspace_bytes, const TmTune* tune,
                   hipStream_t stream);
 
-// A number of choose.h by name ("skinny_rows", "panel_rows", "stream_rows", "skinny_max_rows", "gemv_f32_rows",
+// A number of choose.h by name ("skinny_rows", "panel_qkv_rows", "stream_rows", "skinny_max_rows", "gemv_f32_rows",
 // "decode_chunk", "decode_split_pairs"); -1 for a name it does not know.
 int tm_rule(const char* name);
 // Chunks a decode step's contexts are split into, or 0 if this step does not split them.

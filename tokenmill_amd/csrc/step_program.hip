@@ -79,7 +79,7 @@ bool skinny_ok(const TmLinear& L, const void* x, int ldx, int dtype) {
 }
 
 // `beyond`: the rows up to which the kernels for at most 16 rows are preferred
-bool panel_ok(const TmLinear& L, const void* x, int ldx, int M, int dtype, int beyond, int most_rows = TM_PANEL_ROWS) {
+bool panel_ok(const TmLinear& L, const void* x, int ldx, int M, int dtype, int beyond, int most_rows) {
     return L.packed && M > beyond && M <= most_rows && dtype == TM_BF16 && ldx % 8 == 0 && aligned(x, 16) &&
            tm_gemm_panel_fits(M, L.K);
 }
@@ -408,9 +408,6 @@ struct Run {
                     rc = tm_gemm_skinny_packed(xn, hidden, f.gate_up.packed, 16, nullptr, TM_NONE, act, f.I, T, f.I, hidden, TM_BF16, 1,
                                                nullptr, 0, stream);
                     ++p->taken[TM_GATE_UP_PLAIN];
-                } else if (plain && two_parts && f.I % 4 == 0 && panel_ok(f.gate_up, xn, hidden, T, dtype, from_norm_rows)) {
-                    rc = tm_panel_gate_up_silu(xn, hidden, T, hidden, f.gate_up.packed, act, f.I, stream);
-                    ++p->taken[TM_GATE_UP_PANEL];
                 } else if (plain && two_parts && f.I % 4 == 0 && stream_ok(f.gate_up, xn, hidden, T, dtype, from_norm_rows)) {
                     rc = tm_stream_gate_up_silu(xn, hidden, T, hidden, f.gate_up.packed, act, f.I, stream);
                     ++p->taken[TM_GATE_UP_STREAM];
@@ -646,7 +643,7 @@ int tm_linear_run(const TmLinear* L, int x_dtype, const void* x, int ldx, int M,
 int tm_rule(const char* name) {
     if (!name) return -1;
     if (!strcmp(name, "skinny_rows")) return TM_SKINNY_ROWS;
-    if (!strcmp(name, "panel_rows")) return TM_PANEL_ROWS;
+    if (!strcmp(name, "panel_qkv_rows")) return TM_PANEL_QKV_ROWS;
     if (!strcmp(name, "stream_rows")) return TM_STREAM_ROWS;
     if (!strcmp(name, "skinny_max_rows")) return TM_SKINNY_MAX_ROWS;
     if (!strcmp(name, "gemv_f32_rows")) return TM_GEMV_F32_ROWS;

@@ -62,7 +62,7 @@ RUN_LABELS, RUN_TUNE_AT_ONCE = 1, 2
 
 # how q|k|v, the feed-forward's activation and the attention of prompt portions were computed, in the order of the
 # header's counters
-COUNTERS = ("qkv_from_norm", "qkv_panel", "qkv_stream", "qkv_plain", "gate_up_from_norm", "gate_up_panel",
+COUNTERS = ("qkv_from_norm", "qkv_panel", "qkv_stream", "qkv_plain", "gate_up_from_norm",
             "gate_up_stream", "gate_up_plain", "prefill_split_keys", "prefill_shared_keys")
 
 

@@ -224,7 +224,7 @@ def _tune_arg(tune: tuple[int, int, bool] | None):
 
 def rule(name: str) -> int:
     """A number of the library's kernel-choosing rules (``csrc/choose.h``), for sizing a buffer or checking an
-    argument: "skinny_rows", "panel_rows", "stream_rows", "skinny_max_rows", "gemv_f32_rows", "decode_chunk",
+    argument: "skinny_rows", "panel_qkv_rows", "stream_rows", "skinny_max_rows", "gemv_f32_rows", "decode_chunk",
     "decode_split_pairs". The rules themselves are applied inside the library only."""
     value = _rules.get(name)
     if value is None:
@@ -811,22 +811,6 @@ def panel_qkv_rope(x: torch.Tensor, w: PackedWeight, bias: torch.Tensor | None, 
                                        _p(v_pool if slots is not None else None), c_int(page), _stream()),
            "panel_qkv_rope")
     return q_out
-
-
-def panel_gate_up_silu(x: torch.Tensor, w: PackedWeight, out: torch.Tensor) -> torch.Tensor:
-    """out[M, I] <- silu(x Wg^T) * (x Wu^T) for up to 64 tokens; x bfloat16 [M, K] is the normed input, w as
-    for ``fused_norm_gate_up_silu``."""
-    _gpu(x, out)
-    M, K = x.shape
-    I = out.shape[1]
-    ldx = _panel_input(x, "panel gate-up")
-    _packed_operand(w, 16, "panel gate-up")
-    _need((w.n, w.k) == (2 * I, K) and w.parts == (I, I) and I % 4 == 0,
-          "panel gate-up: w must be the packed [2I, K] matrix in two parts of I rows; I % 4 == 0")
-    _need(out.dtype == torch.bfloat16 and out.is_contiguous() and out.shape[0] == M, "panel gate-up: out bfloat16 [M, I]")
-    _check(library().tm_panel_gate_up_silu(_p(x), c_int(ldx), c_int(M), c_int(K), _p(w.data), _p(out), c_int(I),
-                                           _stream()), "panel_gate_up_silu")
-    return out
 
 
 def stream_fits(M: int, K: int) -> bool:
