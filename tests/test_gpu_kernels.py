@@ -1029,7 +1029,8 @@ def test_stream_qkv_rope(ops, M, K, H, KVH, D, page, rows):
 
 
 @pytest.mark.parametrize("M,K,I", [(64, 896, 4864), (17, 64, 128), (48, 3584, 1000), (33, 120, 200), (9, 1048, 100),
-                                   (64, 264, 16400), (20, 3584, 18944)])
+                                   (64, 264, 16400), (20, 3584, 18944), (40, 72, 10000), (64, 72, 22000), (33, 72, 30000),
+                                   (8, 136, 4864)])
 def test_stream_gate_up_silu(ops, M, K, I):
     torch.manual_seed(24)
     dt = torch.bfloat16
@@ -1078,7 +1079,8 @@ def test_stream_linear_stores_or_adds_into_the_residual(ops, M, N, K, rows):
 
 @pytest.mark.parametrize("M,N,K,rows,groups", [(64, 896, 4864, 4, 8), (33, 3584, 18944, 16, 8), (20, 200, 120, 8, 1),
                                                (48, 1001, 9000, 16, 8), (64, 5120, 27648, 16, 8), (17, 3584, 3584, 8, 8),
-                                               (40, 512, 1024, 16, 2)])
+                                               (40, 512, 1024, 16, 2), (20, 3072, 2048, 16, 8), (5, 6144, 2048, 8, 8),
+                                               (33, 8192, 2048, 16, 8)])
 def test_stream_linear_with_k_split_over_blocks_and_the_norm_that_adds_the_parts(ops, M, N, K, rows, groups):
     """A plain product with few rows of output and a long K splits K over groups of blocks, which leave 32-bit partial
     sums; the norm that follows adds them up in their order, rounds the sum as the product's own epilogue would have,
