@@ -13,6 +13,7 @@ import shutil
 import subprocess
 import sys
 import tempfile
+import time
 from concurrent.futures import ThreadPoolExecutor
 from pathlib import Path
 
@@ -90,14 +91,18 @@ def build(verbose: bool = True) -> Path:
         obj = obj_dir / (src.stem + ".o")
         if verbose:
             print(f"[tokenmill_amd] hipcc {src.name} ({ARCH})", flush=True)
+        t0 = time.monotonic()
         r = subprocess.run([cc, *HIPCC_FLAGS, "-I", str(CSRC), "-c", str(src), "-o", str(obj)],
                            capture_output=True, text=True, env=env)
         if r.returncode != 0:
             raise RuntimeError(f"hipcc failed on {src.name}:\n{r.stdout}\n{r.stderr}")
+        if verbose:
+            print(f"[tokenmill_amd] {src.name} compiled in {time.monotonic() - t0:.0f} s", flush=True)
         return obj
 
+    # the largest sources first: they take the longest, and the build is over when the last of them is
     with ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 4)) as pool:
-        objs = list(pool.map(compile_one, sources()))
+        objs = list(pool.map(compile_one, sorted(sources(), key=lambda p: -p.stat().st_size)))
     lib = out_dir / LIB_NAME
     tmp = out_dir / (LIB_NAME + f".tmp{os.getpid()}")
     r = subprocess.run([cc, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", str(tmp), *map(str, objs), *LINK_LIBS],
