@@ -979,7 +979,8 @@ def test_panel_qkv_rope(ops, M, K, H, KVH, D, page):
 
 
 @pytest.mark.parametrize("M,K,H,KVH,D,page,rows", [(64, 896, 14, 2, 64, 16, 8), (17, 192, 6, 1, 32, 16, 16), (40, 3584, 4, 4, 128, 32, 16),
-                                                    (33, 120, 3, 1, 96, 64, 4), (5, 1096, 14, 2, 64, 16, 8), (64, 5120, 5, 1, 128, 16, 16)])
+                                                    (33, 120, 3, 1, 96, 64, 4), (5, 1096, 14, 2, 64, 16, 8), (64, 5120, 5, 1, 128, 16, 16),
+                                                    (40, 72, 130, 2, 128, 16, 16), (64, 64, 260, 4, 128, 16, 8), (9, 72, 80, 5, 64, 16, 16)])
 def test_stream_qkv_rope(ops, M, K, H, KVH, D, page, rows):
     """q|k|v + bias + rotary + cache write for up to 64 tokens at any width (K no multiple of 32 or of the k-steps a
     wavefront asks for at once; beyond what a block's LDS holds), the matrix streamed from its packed copy whatever

@@ -43,6 +43,18 @@ template <> struct Elem<bf16_t> {
     static __device__ __forceinline__ float round(float v) { return bf16_to_f32(f32_to_bf16(v)); }
 };
 
+// The rotation of a pair (x1, x2) by the angle whose cosine and sine are c and s (reference
+// src/infer/model/layers.py:60-64). Every product and each sum is rounded to 32-bit on its own, as a tensor
+// library's x1 * cos - x2 * sin is: left to itself the compiler fuses a product into the sum, and which one it
+// picks differs from one kernel (or one instantiation of a kernel) to the next, so that the same token would get
+// other last bits from the kernel for 8 rows than from the kernel for 40.
+__device__ __forceinline__ void rotate_pair(float x1, float x2, float c, float s, float& y1, float& y2) {
+#pragma clang fp contract(off)
+    const float a = x1 * c, b = x2 * s, d = x2 * c, e = x1 * s;
+    y1 = a - b;
+    y2 = d + e;
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int off = TM_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, TM_WAVE);

@@ -274,8 +274,8 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int H, int KVH, int D,
             const int hh = idx / half, j = idx - hh * half;
             T* x = row + (size_t)hh * D;
             const float x1 = Elem<T>::load(x + j), x2 = Elem<T>::load(x + j + half);
-            const float y1 = x1 * c[j] - x2 * s[j];
-            const float y2 = x2 * c[j] + x1 * s[j];
+            float y1, y2;
+            rotate_pair(x1, x2, c[j], s[j], y1, y2);
             Elem<T>::store(x + j, y1);
             Elem<T>::store(x + j + half, y2);
             if (store && hh >= H) {

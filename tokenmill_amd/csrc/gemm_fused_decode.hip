@@ -329,8 +329,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void fused_norm_gem
                     float y1[4], y2[4];
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
-                        y1[i] = xA[i] * e.cos[i] - xB[i] * e.sin[i];
-                        y2[i] = xB[i] * e.cos[i] + xA[i] * e.sin[i];
+                        rotate_pair(xA[i], xB[i], e.cos[i], e.sin[i], y1[i], y2[i]);
                     }
                     bf16_t* dst = nullptr;
                     if (done.head < a.H)

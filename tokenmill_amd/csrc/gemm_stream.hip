@@ -309,8 +309,7 @@ __global__ __launch_bounds__(64 * KS * US) void gemm_stream_kernel(const StreamA
                 float y1[4], y2[4];
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    y1[i] = xA[i] * cs[i] - xB[i] * sn[i];
-                    y2[i] = xB[i] * cs[i] + xA[i] * sn[i];
+                    rotate_pair(xA[i], xB[i], cs[i], sn[i], y1[i], y2[i]);
                 }
                 bf16_t* dst = nullptr;
                 if (cu.head < f.H)
