@@ -8,15 +8,17 @@
 // up to this many rows the kernels that stream the matrix once win: the products over packed matrices with
 // the layer's epilogue (bias, rotary + cache write, SiLU*up, residual add), and the ones that start at the norm
 constexpr int TM_SKINNY_ROWS = 16;
-// ... while the model is narrow. They keep all of K of every row in LDS (or re-read the rows per block); from a
-// width of 2,048 the products that stream the matrix through windows of K (gemm_stream.hip, with the partial sums
-// of the output and down projections added by the next norm) take over at fewer rows. Measured on an MI355X, a
-// decode step with this family against the stream family: width 896 (0.5B shape) 16 rows 1.16 against 1.23 ms;
-// width 3,584 (7B) 1 row 3.38 against 3.53, 4 rows 3.45 against 3.53, 8 rows 3.72 against 3.63, 16 rows 4.42
-// against 3.84; width 5,120 (32B, 16 layers) 1 row 3.64 against 3.49, 4 rows 3.80 against 3.44, 8 rows 4.10 against
-// 3.56, 16 rows 4.92 against 3.81. The two families do not mix within a layer: the kernels that start at the norm
-// need the residual stream complete, the stream family leaves partial sums for the norm.
-inline int tm_skinny_rows(int hidden) { return hidden < 2048 ? TM_SKINNY_ROWS : hidden < 4096 ? 4 : 0; }
+// ... while the model is narrow. They keep all of K of every row in LDS (or re-read the rows per block); beyond a
+// width of 1,024 the products that stream the matrix through windows of K (gemm_stream.hip, with the partial sums
+// of the output and down projections added by the next norm) take over at fewer rows, the wider the earlier.
+// Measured on an MI355X, a decode step (ms) with this family against the stream family: width 896 (0.5B shape)
+// 16 rows 1.16 against 1.23; width 1,536 (12 layers of 8,960) 8 rows 0.82 against 0.86, 16 rows 0.95 against 0.92;
+// width 2,048 (12 layers of 11,008) 4 rows 0.85 against 0.99, 8 rows 0.90 against 1.00, 16 rows 1.10 against 1.06;
+// width 3,584 (7B) 1 row 3.38 against 3.53, 4 rows 3.45 against 3.53, 8 rows 3.72 against 3.63, 16 rows 4.42 against
+// 3.84; width 5,120 (32B, 16 layers) 1 row 3.64 against 3.49, 4 rows 3.80 against 3.44, 8 rows 4.10 against 3.56,
+// 16 rows 4.92 against 3.81. The two families do not mix within a layer: the kernels that start at the norm need the
+// residual stream complete, the stream family leaves partial sums for the norm.
+inline int tm_skinny_rows(int hidden) { return hidden <= 1024 ? TM_SKINNY_ROWS : hidden < 3072 ? 8 : hidden < 4096 ? 4 : 0; }
 // ... and the two of them that start at the norm (q|k|v, gate|up) at most to 8 rows: with 9 to 16 rows in LDS a CU
 // holds one block (0.5B shape, 16 rows: 1.195 ms a step against 1.156 with the panel kernels behind a norm of its own)
 inline int tm_from_norm_rows(int hidden) { const int s = tm_skinny_rows(hidden); return s < 8 ? s : 8; }
